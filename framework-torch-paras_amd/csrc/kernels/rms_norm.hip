@@ -1,0 +1,286 @@
+// Fused RMSNorm forward/backward for gfx950.
+//
+// Arithmetic follows the reference's host engine (csrc/ops/fused_ops.cpp:67-85,
+// 105-156): everything is evaluated in fp64 and rounded once to the tensor
+// dtype (double -> float -> T).  fp64 FMA runs at the same per-lane rate as
+// unpacked fp32 on CDNA4 and these kernels are HBM-bound, so the wide math is
+// free; it makes the result agree with the host engine bit for bit except
+// where the summation order changes the last bit of the fp64 sum.
+//
+// Forward: one 256-thread workgroup per row at a time, grid-stride over rows.
+// Each thread owns NV 16-byte vectors of the row (kept in registers between
+// the sum-of-squares pass and the scaling pass, so x is read from HBM once),
+// the four wave sums meet in LDS.
+#include <hip/hip_runtime.h>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+
+namespace paras {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+// Sum over the workgroup; result valid in every thread.  `slots` is LDS of
+// kWavesPerBlock doubles.  Safe to call repeatedly with the same slots.
+__device__ __forceinline__ double block_sum(double v, double* slots) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();  // previous readers of slots are done
+    if ((threadIdx.x & (kWave - 1)) == 0) slots[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+#pragma unroll
+    for (int i = 0; i < kWavesPerBlock; ++i) t += slots[i];
+    return t;
+}
+
+// Register-resident row: H == vectors per row * kVec, vectors per row <= kBlock*NV.
+template <typename T, int NV>
+__global__ __launch_bounds__(kBlock) void rms_norm_fwd_vec(
+    const typename Elem<T>::store_t* __restrict__ x, const typename Elem<T>::store_t* __restrict__ w,
+    typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, int H,
+    double eps) {
+    using E = Elem<T>;
+    using S = typename E::store_t;
+    constexpr int V = E::kVec;
+    __shared__ double slots[kWavesPerBlock];
+
+    const int nvec = H / V;  // 16-byte vectors per row
+    u32x4 wv[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * kBlock;
+        if (c < nvec) wv[i] = load16(w + static_cast<long>(c) * V);
+    }
+
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        const S* xr = x + r * H;
+        S* outr = out + r * H;
+        u32x4 xv[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * kBlock;
+            if (c < nvec) xv[i] = load16_nt(xr + static_cast<long>(c) * V);
+        }
+        double ss = 0.0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * kBlock;
+            if (c < nvec) {
+                const S* e = reinterpret_cast<const S*>(&xv[i]);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const double v = E::to_f64(e[j]);
+                    ss = fma(v, v, ss);
+                }
+            }
+        }
+        ss = block_sum(ss, slots);
+        const double rs = 1.0 / sqrt(ss / static_cast<double>(H) + eps);
+        if (threadIdx.x == 0) rstd[r] = static_cast<float>(rs);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * kBlock;
+            if (c < nvec) {
+                const S* e  = reinterpret_cast<const S*>(&xv[i]);
+                const S* we = reinterpret_cast<const S*>(&wv[i]);
+                u32x4 o;
+                S* oe = reinterpret_cast<S*>(&o);
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    oe[j] = E::from_f64(E::to_f64(e[j]) * rs * E::to_f64(we[j]));
+                store16_nt(outr + static_cast<long>(c) * V, o);
+            }
+        }
+    }
+}
+
+// Any H, any alignment: scalar accesses, row re-read for the second pass.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rms_norm_fwd_any(
+    const typename Elem<T>::store_t* __restrict__ x, const typename Elem<T>::store_t* __restrict__ w,
+    typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, long H,
+    double eps) {
+    using E = Elem<T>;
+    __shared__ double slots[kWavesPerBlock];
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        const auto* xr = x + r * H;
+        auto* outr = out + r * H;
+        double ss = 0.0;
+        for (long j = threadIdx.x; j < H; j += kBlock) {
+            const double v = E::to_f64(xr[j]);
+            ss = fma(v, v, ss);
+        }
+        ss = block_sum(ss, slots);
+        const double rs = 1.0 / sqrt(ss / static_cast<double>(H) + eps);
+        if (threadIdx.x == 0) rstd[r] = static_cast<float>(rs);
+        for (long j = threadIdx.x; j < H; j += kBlock)
+            outr[j] = E::from_f64(E::to_f64(xr[j]) * rs * E::to_f64(w[j]));
+    }
+}
+
+// ---- backward ---------------------------------------------------------------
+// dx: one workgroup per row (dot over the row, then the elementwise formula).
+// dw: column sums over all rows.  Pass 1 writes, per row-slab, a partial fp64
+// column sum into the workspace; pass 2 adds the slabs in slab order, so the
+// result does not depend on scheduling.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rms_norm_bwd_dx(
+    const typename Elem<T>::store_t* __restrict__ go, const typename Elem<T>::store_t* __restrict__ x,
+    const typename Elem<T>::store_t* __restrict__ w, const float* __restrict__ rstd,
+    typename Elem<T>::store_t* __restrict__ gx, long rows, long H) {
+    using E = Elem<T>;
+    __shared__ double slots[kWavesPerBlock];
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        const auto* gr = go + r * H;
+        const auto* xr = x + r * H;
+        auto* gxr = gx + r * H;
+        const double rr = static_cast<double>(rstd[r]);
+        double dot = 0.0;
+        for (long j = threadIdx.x; j < H; j += kBlock)
+            dot += E::to_f64(gr[j]) * E::to_f64(w[j]) * E::to_f64(xr[j]);
+        dot = block_sum(dot, slots);
+        const double coef = rr * rr * rr / static_cast<double>(H);
+        for (long j = threadIdx.x; j < H; j += kBlock) {
+            const double gj = E::to_f64(gr[j]), wj = E::to_f64(w[j]), xj = E::to_f64(xr[j]);
+            gxr[j] = E::from_f64(gj * wj * rr - coef * xj * dot);
+        }
+    }
+}
+
+constexpr int kDwSlabRows = 256;  // rows per partial column sum
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_partial(
+    const typename Elem<T>::store_t* __restrict__ go, const typename Elem<T>::store_t* __restrict__ x,
+    const float* __restrict__ rstd, double* __restrict__ partial, long rows, long H) {
+    using E = Elem<T>;
+    const long j = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    const long slab = blockIdx.y;
+    if (j >= H) return;
+    const long r0 = slab * kDwSlabRows;
+    const long r1 = r0 + kDwSlabRows < rows ? r0 + kDwSlabRows : rows;
+    double acc = 0.0;
+    for (long r = r0; r < r1; ++r)
+        acc += E::to_f64(go[r * H + j]) * E::to_f64(x[r * H + j]) * static_cast<double>(rstd[r]);
+    partial[slab * H + j] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final(
+    const double* __restrict__ partial, typename Elem<T>::store_t* __restrict__ gw, long slabs,
+    long H) {
+    using E = Elem<T>;
+    const long j = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (j >= H) return;
+    double acc = 0.0;
+    for (long s = 0; s < slabs; ++s) acc += partial[s * H + j];
+    gw[j] = E::from_f64(acc);
+}
+
+int grid_for_rows(long rows) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto* st = DeviceContext::instance().device(dev);
+    const long cus = st ? st->compute_units : 256;
+    const long cap = cus * 8;  // eight 256-thread workgroups fill a CU
+    return static_cast<int>(rows < cap ? rows : cap);
+}
+
+template <typename T>
+int launch_fwd(const void* x, const void* w, void* out, float* rstd, long rows, long H,
+               double eps, hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    constexpr int V = Elem<T>::kVec;
+    const auto* xs = static_cast<const S*>(x);
+    const auto* ws = static_cast<const S*>(w);
+    auto* os = static_cast<S*>(out);
+    const int grid = grid_for_rows(rows);
+    const bool aligned = (H % V == 0) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
+                                           reinterpret_cast<uintptr_t>(out)) % 16 == 0);
+    const long nvec = H / V;
+    if (aligned && nvec <= kBlock * 1 && H <= INT32_MAX)
+        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 1>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps);
+    else if (aligned && nvec <= kBlock * 2)
+        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps);
+    else if (aligned && nvec <= kBlock * 4)
+        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 4>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps);
+    else
+        hipLaunchKernelGGL((rms_norm_fwd_any<T>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, H, eps);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+template <typename T>
+int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, void* gx,
+               void* gw, void* workspace, long rows, long H, hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    hipLaunchKernelGGL((rms_norm_bwd_dx<T>), dim3(grid_for_rows(rows)), dim3(kBlock), 0, s,
+                       static_cast<const S*>(go), static_cast<const S*>(x), static_cast<const S*>(w),
+                       rstd, static_cast<S*>(gx), rows, H);
+    PARAS_HIP_TRY(hipGetLastError());
+    const long slabs = (rows + kDwSlabRows - 1) / kDwSlabRows;
+    const unsigned gx_blocks = static_cast<unsigned>((H + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL((rms_norm_bwd_dw_partial<T>), dim3(gx_blocks, static_cast<unsigned>(slabs)),
+                       dim3(kBlock), 0, s, static_cast<const S*>(go), static_cast<const S*>(x), rstd,
+                       static_cast<double*>(workspace), rows, H);
+    PARAS_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL((rms_norm_bwd_dw_final<T>), dim3(gx_blocks), dim3(kBlock), 0, s,
+                       static_cast<const double*>(workspace), static_cast<S*>(gw), slabs, H);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // namespace
+}  // namespace paras
+
+extern "C" {
+
+int paras_rms_norm_fwd(const void* x, const void* w, void* out, float* rstd, int64_t rows,
+                       int64_t H, double eps, int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(rows >= 0 && H >= 0, "paras_rms_norm_fwd: negative shape");
+    if (rows == 0 || H == 0) return PARAS_OK;
+    PARAS_REQUIRE(x && w && out && rstd, "paras_rms_norm_fwd: null pointer");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    switch (dtype) {
+        case PARAS_F32:  return launch_fwd<float>(x, w, out, rstd, rows, H, eps, s);
+        case PARAS_F64:  return launch_fwd<double>(x, w, out, rstd, rows, H, eps, s);
+        case PARAS_BF16: return launch_fwd<bf16_t>(x, w, out, rstd, rows, H, eps, s);
+        case PARAS_F16:  return launch_fwd<f16_t>(x, w, out, rstd, rows, H, eps, s);
+        default: return fail(PARAS_ERR_INVALID, "paras_rms_norm_fwd: unknown dtype %d", dtype);
+    }
+}
+
+size_t paras_rms_norm_bwd_workspace(int64_t rows, int64_t H) {
+    if (rows <= 0 || H <= 0) return 0;
+    const int64_t slabs = (rows + paras::kDwSlabRows - 1) / paras::kDwSlabRows;
+    return static_cast<size_t>(slabs) * static_cast<size_t>(H) * sizeof(double);
+}
+
+int paras_rms_norm_bwd(const void* grad_out, const void* x, const void* w, const float* rstd,
+                       void* grad_x, void* grad_w, void* workspace, int64_t rows, int64_t H,
+                       int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(rows >= 0 && H >= 0, "paras_rms_norm_bwd: negative shape");
+    if (rows == 0 || H == 0) return PARAS_OK;
+    PARAS_REQUIRE(grad_out && x && w && rstd && grad_x && grad_w && workspace,
+                  "paras_rms_norm_bwd: null pointer");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    switch (dtype) {
+        case PARAS_F32:  return launch_bwd<float>(grad_out, x, w, rstd, grad_x, grad_w, workspace, rows, H, s);
+        case PARAS_F64:  return launch_bwd<double>(grad_out, x, w, rstd, grad_x, grad_w, workspace, rows, H, s);
+        case PARAS_BF16: return launch_bwd<bf16_t>(grad_out, x, w, rstd, grad_x, grad_w, workspace, rows, H, s);
+        case PARAS_F16:  return launch_bwd<f16_t>(grad_out, x, w, rstd, grad_x, grad_w, workspace, rows, H, s);
+        default: return fail(PARAS_ERR_INVALID, "paras_rms_norm_bwd: unknown dtype %d", dtype);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,375 @@
+// Flash-attention forward for gfx950 (bf16 / fp16 MFMA, fp32 accumulate).
+//
+// out = softmax(q k^T * scale [+ causal mask]) v, computed tile by tile with an
+// online softmax; the [Lq, Lk] score matrix never exists in memory (the
+// reference materialises it: csrc/ops/attention_ops.cpp:101,128).
+//
+// Work decomposition
+//   workgroup = 4 wavefronts = 128 queries of one (batch, head); each wave owns
+//   32 queries.  K/V are streamed in tiles of 64 keys through LDS (double
+//   buffered, one barrier per tile), shared by the 4 waves.
+//
+// The products are formed transposed so that a lane always owns ONE query:
+//   S^T = K Q^T    A = K tile from LDS (lane: key l%32, 8 consecutive d),
+//                  B = Q^T from registers (lane: query l%32, same 8 d)
+//                  -> accumulator lane (query l%32, half h=l/32) holds, for a
+//                  32-key block, keys (r/4)*8 + 4h + r%4, r = 0..15
+//   row max / row sum: in-lane over the accumulator registers plus one
+//                  v_permlane32_swap between the two half-waves
+//   O^T = V^T P^T  B = P^T straight from the S^T accumulators (converted to
+//                  16 bit, no shuffle: the accumulator's key order is simply
+//                  used as the contraction order),
+//                  A = V^T read from the row-major V tile with
+//                  ds_read_b64_tr_b16, which transposes 4 keys x 16 d per
+//                  16-lane group in the LDS crossbar
+//   rescaling O by exp(m_old - m_new) is a per-lane scalar multiply.
+//
+// v_mfma_f32_32x32x16_{bf16,f16}: 32 MFMAs per wave per 64-key tile at D=128.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+#include "kernels/sdpa_internal.h"
+
+namespace paras {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves   = 4;
+constexpr int kBM      = 128;  // queries per workgroup
+constexpr int kBN      = 64;   // keys per tile
+
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
+
+struct FlashParams {
+    const std::uint16_t* q;
+    const std::uint16_t* k;
+    const std::uint16_t* v;
+    std::uint16_t*       out;
+    float*               lse;
+    long qs_b, qs_h, qs_l;  // element strides
+    long ks_b, ks_h, ks_l;
+    long vs_b, vs_h, vs_l;
+    int  B, Hq, Hkv, Lq, Lk;
+    int  n_qblocks;
+    float scale_log2;  // scale * log2(e)
+    float scale;
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ std::uint32_t pack2(float lo, float hi) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, bf16x2));
+    }
+};
+template <> struct Mma<f16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ std::uint32_t pack2(float lo, float hi) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, f16x2));
+    }
+};
+
+// Exchange between the two half-waves that share a query: v_permlane32_swap
+// swaps lanes 32..63 of its first register with lanes 0..31 of its second.
+// Fed the same value twice it leaves the lower half's value in every lane of
+// the first register and the upper half's value in every lane of the second.
+// Written as inline asm because the compiler's builtin for it returns the
+// first result twice (seen with ROCm 7.2's hipcc); the s_nop pairs cover the
+// VALU-write -> permlane-read and permlane-write -> VALU-read wait states the
+// hazard recognizer cannot see inside an asm block.
+__device__ __forceinline__ void half_swap(float x, float& lo, float& hi) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    lo = a;
+    hi = b;
+}
+__device__ __forceinline__ float half_swap_max(float x) {
+    float lo, hi;
+    half_swap(x, lo, hi);
+    return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_swap_sum(float x) {
+    float lo, hi;
+    half_swap(x, lo, hi);
+    return lo + hi;
+}
+
+template <typename T, int D, bool kCausal>
+__global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParams p) {
+    constexpr int KS     = D + 8;    // K row stride in LDS (elements): 16-byte reads of 16 keys hit 64 distinct banks
+    constexpr int VS     = D + 32;   // V row stride: 4 consecutive keys x 64 bytes tile all 64 banks
+    constexpr int KSTEPS = D / 16;   // MFMA k-steps over the head dim
+    constexpr int DBLK   = D / 32;   // 32-wide blocks of the output head dim
+    constexpr int CHUNKS = D / 8;    // 16-byte chunks per row
+    constexpr int LOADS  = kBN * CHUNKS / kThreads;  // chunks per thread per tile
+
+    __shared__ __attribute__((aligned(16))) std::uint16_t k_lds[2][kBN * KS];
+    __shared__ __attribute__((aligned(16))) std::uint16_t v_lds[2][kBN * VS];
+
+    // ---- which (batch, head, query block): heavy causal blocks first, and all
+    // query blocks of one head on one XCD so its K/V stay in that XCD's L2.
+    const int nq = p.n_qblocks;
+    const int BH = p.B * p.Hq;
+    int bh, qi;
+    {
+        const int idx = blockIdx.x;
+        if (BH % 8 == 0) {
+            const int xcd = idx & 7, j = idx >> 3;
+            bh = (j / nq) * 8 + xcd;
+            qi = j % nq;
+        } else {
+            bh = idx / nq;
+            qi = idx % nq;
+        }
+    }
+    const int qblock = nq - 1 - qi;
+    const int b = bh / p.Hq, hq = bh % p.Hq;
+    const int hkv = hq / (p.Hq / p.Hkv);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lq = lane & 31, lh = lane >> 5;
+    const int q0 = qblock * kBM + wave * 32;  // first query of this wave
+    const int my_q = q0 + lq;
+
+    // ---- Q^T operand: this lane's query row, 8 d-values per k-step.
+    i16x8 qreg[KSTEPS];
+    {
+        const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
+        const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks)
+            qreg[ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
+    }
+
+    const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
+    const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
+
+    // Number of key tiles this workgroup needs.
+    int n_tiles = (p.Lk + kBN - 1) / kBN;
+    if (kCausal) {
+        const int last_q = min(qblock * kBM + kBM, p.Lq) - 1;  // keys 0..last_q
+        const int need = min(last_q + 1, p.Lk);
+        n_tiles = (need + kBN - 1) / kBN;
+    }
+
+    // ---- tile staging: each thread moves LOADS 16-byte chunks of K and of V.
+    u32x4 kst[LOADS], vst[LOADS];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = tid + i * kThreads;
+            const int row = c / CHUNKS, col = (c % CHUNKS) * 8;
+            const int key = t * kBN + row;
+            if (key < p.Lk) {
+                kst[i] = load16(kbase + static_cast<long>(key) * p.ks_l + col);
+                vst[i] = load16(vbase + static_cast<long>(key) * p.vs_l + col);
+            } else {
+                kst[i] = u32x4{0, 0, 0, 0};
+                vst[i] = u32x4{0, 0, 0, 0};
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int c = tid + i * kThreads;
+            const int row = c / CHUNKS, col = (c % CHUNKS) * 8;
+            *reinterpret_cast<u32x4*>(&k_lds[buf][row * KS + col]) = kst[i];
+            *reinterpret_cast<u32x4*>(&v_lds[buf][row * VS + col]) = vst[i];
+        }
+    };
+
+    float16_t oacc[DBLK];
+#pragma unroll
+    for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float m_run = -INFINITY;  // running max of raw scores (before scaling)
+    float l_run = 0.f;        // this half-wave's share of the running sum
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    // Per-lane LDS offsets.
+    const int k_off = lq * KS + lh * 8;                                        // + kb*32*KS + ks*16
+    const int grp = lane >> 4, m16 = lane & 15;
+    const int v_off = (4 * lh + (m16 >> 2)) * VS + 16 * (grp & 1) + 4 * (m16 & 3);  // + (kb*32+16s(+8))*VS + db*32
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < n_tiles) load_tile(t + 1);
+
+        // ---- S^T = K Q^T for the two 32-key blocks of the tile
+        float16_t sacc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                const i16x8 a = *reinterpret_cast<const i16x8*>(&k_lds[buf][k_off + kb * 32 * KS + ks * 16]);
+                sacc[kb] = Mma<T>::run(a, qreg[ks], sacc[kb]);
+            }
+        }
+
+        // ---- masking (only tiles that touch the diagonal or the end of K)
+        const int key0 = t * kBN;
+        const bool need_mask = (kCausal && key0 + kBN - 1 > q0) || (key0 + kBN > p.Lk);
+        if (need_mask) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = key0 + kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                    const bool dead = (kCausal && key > my_q) || key >= p.Lk;
+                    if (dead) sacc[kb][r] = -INFINITY;
+                }
+        }
+
+        // ---- online softmax
+        float mloc = sacc[0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
+        mloc = half_swap_max(mloc);
+        const float m_new = fmaxf(m_run, mloc);
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2);
+        const float mc = m_new * p.scale_log2;
+        m_run = m_new;
+        float lsum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = __builtin_amdgcn_exp2f(fmaf(sacc[kb][r], p.scale_log2, -mc));
+                sacc[kb][r] = e;
+                lsum += e;
+            }
+        l_run = l_run * alpha + lsum;
+#pragma unroll
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+
+        // ---- P^T as MFMA B operands (two k-steps of 16 keys per 32-key block)
+        i16x8 pb[2][2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                u32x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    w[e] = Mma<T>::pack2(sacc[kb][8 * s + 2 * e], sacc[kb][8 * s + 2 * e + 1]);
+                pb[kb][s] = __builtin_bit_cast(i16x8, w);
+            }
+
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const std::uint16_t* vp = &v_lds[buf][v_off + (kb * 32 + 16 * s) * VS + db * 32];
+                    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+                    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * VS));
+                    const i16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    oacc[db] = Mma<T>::run(a, pb[kb][s], oacc[db]);
+                }
+
+        // ---- publish the next tile
+        if (t + 1 < n_tiles) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: normalise and store O[q][d]; lane holds 4 consecutive d per (db, r/4)
+    const float l_tot = half_swap_sum(l_run);
+    const float inv_l = 1.0f / l_tot;
+    if (my_q < p.Lq) {
+        std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = db * 32 + g * 8 + 4 * lh;
+                u32x2 w;
+                w[0] = Mma<T>::pack2(oacc[db][4 * g + 0] * inv_l, oacc[db][4 * g + 1] * inv_l);
+                w[1] = Mma<T>::pack2(oacc[db][4 * g + 2] * inv_l, oacc[db][4 * g + 3] * inv_l);
+                *reinterpret_cast<u32x2*>(op + d) = w;
+            }
+        if (p.lse != nullptr && lh == 0)
+            p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run * p.scale + logf(l_tot);
+    }
+}
+
+template <typename T, int D>
+int launch_t(const FlashParams& p, bool causal, hipStream_t s) {
+    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
+    if (causal)
+        hipLaunchKernelGGL((flash_fwd_kernel<T, D, true>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL((flash_fwd_kernel<T, D, false>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, p);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+bool mult8(const int64_t* strides) { return strides[0] % 8 == 0 && strides[1] % 8 == 0 && strides[2] % 8 == 0; }
+
+}  // namespace
+
+bool flash_supported(const paras_sdpa_args& a) {
+    if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
+    if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
+    if (a.mask_kind != 0 || a.attn != nullptr) return false;
+    if (a.Lq < 1 || a.Lk < 1) return false;
+    if (!(a.scale > 0.0) || !std::isfinite(a.scale)) return false;  // the running max is taken on raw scores
+    if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.out)) return false;
+    if (!mult8(a.q_strides) || !mult8(a.k_strides) || !mult8(a.v_strides)) return false;
+    const int64_t nq = (a.Lq + kBM - 1) / kBM;
+    if (a.B * a.Hq * nq > 0x7fffffffLL || a.Lq > 0x3fffffff || a.Lk > 0x3fffffff) return false;
+    return true;
+}
+
+int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
+    FlashParams p;
+    p.q = static_cast<const std::uint16_t*>(a.q);
+    p.k = static_cast<const std::uint16_t*>(a.k);
+    p.v = static_cast<const std::uint16_t*>(a.v);
+    p.out = static_cast<std::uint16_t*>(a.out);
+    p.lse = a.lse;
+    p.qs_b = a.q_strides[0]; p.qs_h = a.q_strides[1]; p.qs_l = a.q_strides[2];
+    p.ks_b = a.k_strides[0]; p.ks_h = a.k_strides[1]; p.ks_l = a.k_strides[2];
+    p.vs_b = a.v_strides[0]; p.vs_h = a.v_strides[1]; p.vs_l = a.v_strides[2];
+    p.B = static_cast<int>(a.B); p.Hq = static_cast<int>(a.Hq); p.Hkv = static_cast<int>(a.Hkv);
+    p.Lq = static_cast<int>(a.Lq); p.Lk = static_cast<int>(a.Lk);
+    p.n_qblocks = static_cast<int>((a.Lq + kBM - 1) / kBM);
+    p.scale = static_cast<float>(a.scale);
+    p.scale_log2 = static_cast<float>(a.scale * 1.4426950408889634);
+    const bool causal = a.is_causal != 0;
+    if (a.dtype == PARAS_BF16)
+        return a.D == 128 ? launch_t<bf16_t, 128>(p, causal, s) : launch_t<bf16_t, 64>(p, causal, s);
+    return a.D == 128 ? launch_t<f16_t, 128>(p, causal, s) : launch_t<f16_t, 64>(p, causal, s);
+}
+
+}  // namespace paras

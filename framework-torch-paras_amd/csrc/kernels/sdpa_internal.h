@@ -1,0 +1,26 @@
+// Launchers of the three attention kernels; the C ABI entry point in sdpa.hip
+// validates the request, picks one of them and calls it.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "paras_hip.h"
+
+namespace paras {
+
+// MFMA flash forward: bf16/f16, D == Dv in {64, 128}, no explicit mask
+// (causal or none), no attention weights returned.
+bool flash_supported(const paras_sdpa_args& a);
+int  launch_flash(const paras_sdpa_args& a, hipStream_t s);
+
+// Split-KV decode: short query (Lq * Hq/Hkv <= 16), long K/V, bf16/f16,
+// D == Dv == 128, no explicit mask, not causal.
+bool   decode_supported(const paras_sdpa_args& a);
+size_t decode_workspace(const paras_sdpa_args& a);
+int    launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s);
+
+// Everything else (fp32/fp64, any head size, bool/additive masks, weights).
+size_t generic_workspace(const paras_sdpa_args& a);
+int    launch_generic(const paras_sdpa_args& a, void* workspace, hipStream_t s);
+
+}  // namespace paras

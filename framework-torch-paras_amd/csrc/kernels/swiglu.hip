@@ -1,0 +1,275 @@
+// Fused SwiGLU forward/backward and rotate_half for gfx950.
+//
+// The reference's host engine evaluates out = (g / (1 + exp(-g))) * u in fp64
+// and rounds once to the tensor dtype through float
+// (csrc/ops/fused_ops.cpp:185-190).  An fp64 exp per element would make this
+// stream compute-bound, so for the 16-bit dtypes the forward kernel works in
+// two tiers:
+//   fast  fp32 evaluation with a proven relative error bound kFastRelErr; the
+//         result is accepted when both ends of the error interval round to
+//         the same 16-bit value, which means the fp64 result rounds there too;
+//   exact the fp64 formula, taken by the few lanes whose interval straddles a
+//         rounding boundary (about 1 element in 1000) or whose gate lies
+//         outside the range the bound was derived for.
+// The output therefore equals the fp64-then-round definition everywhere, not
+// only within a tolerance.  fp32/fp64 tensors use the fp64 formula directly.
+//
+// Layout: flat contiguous streams, 16 bytes per lane per access, kUnroll
+// independent accesses in flight per lane, grid-stride.
+#include <hip/hip_runtime.h>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+
+namespace paras {
+namespace {
+
+constexpr int kBlock  = 256;
+constexpr int kUnroll = 2;  // 16-byte vectors per stream per lane per iteration
+
+// Bound on |fast - exact| / |exact| for gate in [kFastGateMin, kFastGateMax]:
+// the exponent argument g*log2(e) carries at most |g*log2e| * 2^-23 absolute
+// error (product rounding + constant), i.e. <= 8.1e-7 relative on exp for
+// g >= -8 (for g > 0 the term exp(-g) <= 1 is damped by 1/(1+e)); v_exp_f32,
+// the add, v_rcp_f32 and the two multiplies add < 5e-7.  2^-19 = 1.9e-6
+// covers the sum with margin.
+constexpr float kFastRelErr  = 1.9073486328125e-06f;  // 2^-19
+constexpr float kFastGateMin = -8.0f;
+constexpr float kFastGateMax = 60.0f;
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::store_t swiglu_exact(float g, float u) {
+    const double gd = static_cast<double>(g);
+    const double s  = gd / (1.0 + exp(-gd));
+    return Elem<T>::from_f64(s * static_cast<double>(u));
+}
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::store_t swiglu_one(typename Elem<T>::store_t gs,
+                                                                  typename Elem<T>::store_t us) {
+    using E = Elem<T>;
+    if constexpr (sizeof(typename E::store_t) == 2) {
+        const float g = E::to_f32(gs);
+        const float u = E::to_f32(us);
+        const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
+        const float y = g * __builtin_amdgcn_rcpf(1.0f + e) * u;
+        const auto lo = E::from_f32(y * (1.0f - kFastRelErr));
+        const auto hi = E::from_f32(y * (1.0f + kFastRelErr));
+        // NaN gates fail the range test and take the exact tier.  A result in
+        // fp32's denormal range has no relative bound, so it is only accepted
+        // when it is an exact zero (zero gate or zero up).
+        const bool sized = (fabsf(y) >= 1e-30f) || (g == 0.0f) || (u == 0.0f);
+        const bool ok = (lo == hi) && (g >= kFastGateMin) && (g <= kFastGateMax) && sized;
+        if (__builtin_expect(ok, 1)) return lo;
+        return swiglu_exact<T>(g, u);
+    } else {
+        const double g = E::to_f64(gs);
+        const double s = g / (1.0 + exp(-g));
+        return E::from_f64(s * E::to_f64(us));
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_fwd_vec(
+    const typename Elem<T>::store_t* __restrict__ gate, const typename Elem<T>::store_t* __restrict__ up,
+    typename Elem<T>::store_t* __restrict__ out, long nvec) {
+    using E = Elem<T>;
+    using S = typename E::store_t;
+    constexpr int V = E::kVec;
+    const long stride = static_cast<long>(gridDim.x) * kBlock * kUnroll;
+    for (long base = static_cast<long>(blockIdx.x) * kBlock * kUnroll + threadIdx.x; base < nvec;
+         base += stride) {
+        u32x4 gv[kUnroll], uv[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const long i = base + static_cast<long>(k) * kBlock;
+            if (i < nvec) {
+                gv[k] = load16_nt(gate + i * V);
+                uv[k] = load16_nt(up + i * V);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+            const long i = base + static_cast<long>(k) * kBlock;
+            if (i < nvec) {
+                const S* ge = reinterpret_cast<const S*>(&gv[k]);
+                const S* ue = reinterpret_cast<const S*>(&uv[k]);
+                u32x4 o;
+                S* oe = reinterpret_cast<S*>(&o);
+#pragma unroll
+                for (int j = 0; j < V; ++j) oe[j] = swiglu_one<T>(ge[j], ue[j]);
+                store16_nt(out + i * V, o);
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_fwd_any(
+    const typename Elem<T>::store_t* __restrict__ gate, const typename Elem<T>::store_t* __restrict__ up,
+    typename Elem<T>::store_t* __restrict__ out, long first, long n) {
+    const long stride = static_cast<long>(gridDim.x) * kBlock;
+    for (long i = first + static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride)
+        out[i] = swiglu_one<T>(gate[i], up[i]);
+}
+
+// Backward (csrc/ops/fused_ops.cpp:218-226), fp64 as on the host:
+//   s = 1/(1+exp(-g)); dup = dy*g*s; dgate = dy*u*(s*(1+g*(1-s)))
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_any(
+    const typename Elem<T>::store_t* __restrict__ go, const typename Elem<T>::store_t* __restrict__ gate,
+    const typename Elem<T>::store_t* __restrict__ up, typename Elem<T>::store_t* __restrict__ ggate,
+    typename Elem<T>::store_t* __restrict__ gup, long n) {
+    using E = Elem<T>;
+    const long stride = static_cast<long>(gridDim.x) * kBlock;
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) {
+        const double dy = E::to_f64(go[i]);
+        const double g  = E::to_f64(gate[i]);
+        const double u  = E::to_f64(up[i]);
+        const double s  = 1.0 / (1.0 + exp(-g));
+        gup[i]   = E::from_f64(dy * g * s);
+        ggate[i] = E::from_f64(dy * u * (s * (1.0 + g * (1.0 - s))));
+    }
+}
+
+// rotate_half (csrc/ops/fused_ops.cpp:254-263, 290-299): out[.., c] takes
+// x[.., c+half] (negated for forward) when c < half, else x[.., c-half]
+// (negated for backward).  Negation flips the sign bit, which is what
+// -(double)v rounded back gives for every finite value and infinity; a NaN
+// stays a NaN.
+template <typename S>
+__global__ __launch_bounds__(kBlock) void rotate_half_any(const S* __restrict__ x, S* __restrict__ out,
+                                                          long n, long D, int backward) {
+    const long half = D / 2;
+    const long stride = static_cast<long>(gridDim.x) * kBlock;
+    constexpr S kSign = static_cast<S>(S{1} << (sizeof(S) * 8 - 1));
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) {
+        const long col = i % D;
+        const bool first = col < half;
+        const S v = x[first ? i + half : i - half];
+        const bool negate = backward ? !first : first;
+        out[i] = negate ? static_cast<S>(v ^ kSign) : v;
+    }
+}
+
+int stream_grid(long work_items_per_block_iter, long total) {
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto* st = DeviceContext::instance().device(dev);
+    const long cus = st ? st->compute_units : 256;
+    const long cap = cus * 8;
+    const long need = (total + work_items_per_block_iter - 1) / work_items_per_block_iter;
+    const long g = need < cap ? need : cap;
+    return static_cast<int>(g < 1 ? 1 : g);
+}
+
+template <typename T>
+int launch_swiglu_fwd(const void* gate, const void* up, void* out, long n, hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    constexpr int V = Elem<T>::kVec;
+    const auto* g = static_cast<const S*>(gate);
+    const auto* u = static_cast<const S*>(up);
+    auto* o = static_cast<S*>(out);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) |
+                           reinterpret_cast<uintptr_t>(out)) % 16) == 0;
+    long done = 0;
+    if (aligned && n >= V) {
+        const long nvec = n / V;
+        hipLaunchKernelGGL((swiglu_fwd_vec<T>), dim3(stream_grid(kBlock * kUnroll, nvec)), dim3(kBlock), 0,
+                           s, g, u, o, nvec);
+        PARAS_HIP_TRY(hipGetLastError());
+        done = nvec * V;
+    }
+    if (done < n) {
+        hipLaunchKernelGGL((swiglu_fwd_any<T>), dim3(stream_grid(kBlock, n - done)), dim3(kBlock), 0, s, g,
+                           u, o, done, n);
+        PARAS_HIP_TRY(hipGetLastError());
+    }
+    return PARAS_OK;
+}
+
+template <typename T>
+int launch_swiglu_bwd(const void* go, const void* gate, const void* up, void* ggate, void* gup, long n,
+                      hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    hipLaunchKernelGGL((swiglu_bwd_any<T>), dim3(stream_grid(kBlock, n)), dim3(kBlock), 0, s,
+                       static_cast<const S*>(go), static_cast<const S*>(gate), static_cast<const S*>(up),
+                       static_cast<S*>(ggate), static_cast<S*>(gup), n);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // namespace
+}  // namespace paras
+
+extern "C" {
+
+int paras_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(n >= 0, "paras_swiglu_fwd: negative size");
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(gate && up && out, "paras_swiglu_fwd: null pointer");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    switch (dtype) {
+        case PARAS_F32:  return launch_swiglu_fwd<float>(gate, up, out, n, s);
+        case PARAS_F64:  return launch_swiglu_fwd<double>(gate, up, out, n, s);
+        case PARAS_BF16: return launch_swiglu_fwd<bf16_t>(gate, up, out, n, s);
+        case PARAS_F16:  return launch_swiglu_fwd<f16_t>(gate, up, out, n, s);
+        default: return fail(PARAS_ERR_INVALID, "paras_swiglu_fwd: unknown dtype %d", dtype);
+    }
+}
+
+int paras_swiglu_bwd(const void* grad_out, const void* gate, const void* up, void* grad_gate,
+                     void* grad_up, int64_t n, int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(n >= 0, "paras_swiglu_bwd: negative size");
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(grad_out && gate && up && grad_gate && grad_up, "paras_swiglu_bwd: null pointer");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    switch (dtype) {
+        case PARAS_F32:  return launch_swiglu_bwd<float>(grad_out, gate, up, grad_gate, grad_up, n, s);
+        case PARAS_F64:  return launch_swiglu_bwd<double>(grad_out, gate, up, grad_gate, grad_up, n, s);
+        case PARAS_BF16: return launch_swiglu_bwd<bf16_t>(grad_out, gate, up, grad_gate, grad_up, n, s);
+        case PARAS_F16:  return launch_swiglu_bwd<f16_t>(grad_out, gate, up, grad_gate, grad_up, n, s);
+        default: return fail(PARAS_ERR_INVALID, "paras_swiglu_bwd: unknown dtype %d", dtype);
+    }
+}
+
+int paras_rotate_half(const void* x, void* out, int64_t rows, int64_t D, int backward, int dtype,
+                      void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(rows >= 0 && D >= 0, "paras_rotate_half: negative shape");
+    PARAS_REQUIRE(D % 2 == 0, "paras rotate_half: last dimension must be even");
+    const long n = rows * D;
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(x && out, "paras_rotate_half: null pointer");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    const dim3 grid(stream_grid(kBlock, n)), block(kBlock);
+    switch (dtype) {
+        case PARAS_F32:
+            hipLaunchKernelGGL((rotate_half_any<uint32_t>), grid, block, 0, s, static_cast<const uint32_t*>(x),
+                               static_cast<uint32_t*>(out), n, (long)D, backward);
+            break;
+        case PARAS_F64:
+            hipLaunchKernelGGL((rotate_half_any<uint64_t>), grid, block, 0, s, static_cast<const uint64_t*>(x),
+                               static_cast<uint64_t*>(out), n, (long)D, backward);
+            break;
+        case PARAS_BF16:
+        case PARAS_F16:
+            hipLaunchKernelGGL((rotate_half_any<uint16_t>), grid, block, 0, s, static_cast<const uint16_t*>(x),
+                               static_cast<uint16_t*>(out), n, (long)D, backward);
+            break;
+        default: return fail(PARAS_ERR_INVALID, "paras_rotate_half: unknown dtype %d", dtype);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // extern "C"

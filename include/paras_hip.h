@@ -1,0 +1,249 @@
+/*
+ * paras_hip.h -- C ABI of libparas_hip.so: the MI355X (gfx950) device layer
+ * behind the `paras` PyTorch device.
+ *
+ * Everything that crosses this boundary is a plain pointer, an integer or a
+ * double; no torch / ATen / C++ types appear.  All device pointers are plain
+ * HBM addresses obtained from paras_alloc() or from any other HIP allocation
+ * of the same process.  `stream` is a hipStream_t passed as void* and used as
+ * given on the calling thread's current HIP device (NULL is HIP's null
+ * stream); paras_stream(device) hands out the context's own stream.  Launches
+ * are asynchronous on that stream.
+ *
+ * Every function returns PARAS_OK (0) or a negative paras_status; the text of
+ * the last failure on the calling thread is returned by paras_last_error().
+ * Nothing here throws and nothing here falls back to the host: if no HIP
+ * device or no gfx950 code object is usable the call fails.
+ *
+ * The reference (Torch-ParaS) has no C ABI: its ops are C++ functions in
+ * anonymous namespaces registered with the PyTorch dispatcher, running on
+ * `compat::Queue`.  Each entry point below names the reference function whose
+ * arithmetic it replaces (paths relative to the reference tree).
+ */
+#ifndef PARAS_HIP_H
+#define PARAS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PARAS_API __attribute__((visibility("default")))
+
+typedef enum paras_status {
+    PARAS_OK              = 0,
+    PARAS_ERR_INVALID     = -1, /* bad argument (shape, dtype, null pointer)   */
+    PARAS_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for  */
+    PARAS_ERR_HIP         = -3, /* a HIP runtime call failed                   */
+    PARAS_ERR_NO_DEVICE   = -4, /* no usable HIP device                        */
+    PARAS_ERR_OOM         = -5  /* hipMalloc failed                            */
+} paras_status;
+
+/* Element types.  Values are part of the ABI. */
+typedef enum paras_dtype {
+    PARAS_F32  = 0,
+    PARAS_F16  = 1,
+    PARAS_BF16 = 2,
+    PARAS_F64  = 3
+} paras_dtype;
+
+/* ------------------------------------------------------------------------- */
+/* Library / error state                                                     */
+/* ------------------------------------------------------------------------- */
+
+/* Text of the last error raised on the calling thread ("" if none). */
+PARAS_API const char* paras_last_error(void);
+
+/* ABI version of this header (bumped on any incompatible change). */
+PARAS_API int paras_abi_version(void);
+
+/* ------------------------------------------------------------------------- */
+/* Device context (replaces compat::enumerate_devices / compat::Queue,        */
+/* csrc/compat/paras_compat.h:69-221, and Context, csrc/core/context.h:43-74) */
+/* Device i is HIP device i.  One non-blocking stream per device.            */
+/* ------------------------------------------------------------------------- */
+
+/* Number of HIP devices; 0 (never an error) when none is visible. */
+PARAS_API int paras_device_count(void);
+
+/* Copies the device's marketing name into buf (NUL-terminated, truncated). */
+PARAS_API int paras_device_name(int device, char* buf, size_t buflen);
+
+/* Compute-unit count and total HBM bytes of the device. */
+PARAS_API int paras_device_info(int device, int* compute_units, uint64_t* hbm_bytes);
+
+/* The context's stream for `device` (a hipStream_t), created on first use. */
+PARAS_API int paras_stream(int device, void** stream_out);
+
+/* 1 in a process forked after the context was built (HIP state does not
+ * survive fork; csrc/core/context.cpp:33-38, 106-109), else 0. */
+PARAS_API int paras_is_bad_fork(void);
+
+/* Blocks until all work queued on the context stream of `device` is done
+ * (Context::synchronize, csrc/core/context.cpp:69). */
+PARAS_API int paras_synchronize(int device);
+
+/* ------------------------------------------------------------------------- */
+/* Binned HBM allocator (replaces MemoryPool, csrc/core/allocator.cpp:53-122) */
+/* Same contract: request rounded up to a power of two, at least 256 bytes     */
+/* (above 1 GiB: to a multiple of 256 MiB); freed blocks are cached per size   */
+/* class unless PARAS_NO_CACHE=1; backing store is hipMalloc (device HBM,      */
+/* never managed memory).                                                      */
+/* ------------------------------------------------------------------------- */
+
+PARAS_API int paras_alloc(int device, size_t nbytes, void** ptr_out);
+/* Returns the block to the pool; an unknown pointer is PARAS_ERR_INVALID
+ * (csrc/core/allocator.cpp:92-94). */
+PARAS_API int paras_free(int device, void* ptr);
+/* Synchronizes the device, then hipFree()s every cached block
+ * (Context::empty_cache, csrc/core/context.cpp:96-100). */
+PARAS_API int paras_empty_cache(int device);
+/* Bytes held from hipMalloc (live + cached) and bytes sitting in the cache. */
+PARAS_API int paras_memory_stats(int device, uint64_t* allocated, uint64_t* cached);
+/* Size class a request of nbytes lands in (pure function, no device needed). */
+PARAS_API size_t paras_round_size(size_t nbytes);
+
+/* Copies (replace Queue::copy / Queue::memset, paras_compat.cpp:326-391).
+ * kind: 0 host->device, 1 device->host, 2 device->device.  Host->device and
+ * device->host copies return after the data has arrived; device->device
+ * copies are queued on the context stream. */
+PARAS_API int paras_memcpy(int device, void* dst, const void* src, size_t nbytes, int kind);
+PARAS_API int paras_memset(int device, void* dst, int value, size_t nbytes);
+
+/* ------------------------------------------------------------------------- */
+/* Fused RMSNorm (replaces ptsycl::rms_norm, csrc/ops/fused_ops.cpp:43-88)    */
+/*   ss = sum_j x[r][j]^2 ; rstd[r] = 1/sqrt(ss/H + eps)                      */
+/*   out[r][j] = T( x[r][j] * rstd[r] * w[j] )   (single rounding)            */
+/* x, out: [rows, H] contiguous, dtype T; w: [H] dtype T; rstd: [rows] fp32.  */
+/* rows == 0 or H == 0 is a no-op.                                            */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_rms_norm_fwd(const void* x, const void* w, void* out, float* rstd,
+                                 int64_t rows, int64_t H, double eps, int dtype,
+                                 void* stream);
+
+/* (replaces ptsycl::rms_norm_backward, csrc/ops/fused_ops.cpp:90-157)
+ *   dot = sum_j g*w*x ; dx = g*w*rstd - rstd^3/H * x * dot ;
+ *   dw[j] = sum_r g[r][j]*x[r][j]*rstd[r]
+ * `workspace` must hold paras_rms_norm_bwd_workspace(rows, H) bytes of device
+ * memory (partial column sums). */
+PARAS_API size_t paras_rms_norm_bwd_workspace(int64_t rows, int64_t H);
+PARAS_API int paras_rms_norm_bwd(const void* grad_out, const void* x, const void* w,
+                                 const float* rstd, void* grad_x, void* grad_w,
+                                 void* workspace, int64_t rows, int64_t H, int dtype,
+                                 void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Fused SwiGLU (replaces ptsycl::swiglu, csrc/ops/fused_ops.cpp:162-194)     */
+/*   out[i] = T( gate[i]/(1+exp(-gate[i])) * up[i] ), contiguous, n elements  */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n,
+                               int dtype, void* stream);
+
+/* (replaces ptsycl::swiglu_backward, csrc/ops/fused_ops.cpp:196-229)
+ *   s = sigmoid(g); dup = dy*g*s ; dgate = dy*u*s*(1+g*(1-s)) */
+PARAS_API int paras_swiglu_bwd(const void* grad_out, const void* gate, const void* up,
+                               void* grad_gate, void* grad_up, int64_t n, int dtype,
+                               void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* rotate_half (replaces ptsycl::rotate_half(+_backward),                     */
+/* csrc/ops/fused_ops.cpp:234-302): out = cat(-x2, x1) over the last dim D    */
+/* (backward: cat(g2, -g1)).  x, out: [rows, D] contiguous, D even.           */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_rotate_half(const void* x, void* out, int64_t rows, int64_t D,
+                                int backward, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Scaled dot-product attention forward                                       */
+/* (replaces ptsycl::sdpa_math, csrc/ops/attention_ops.cpp:71-136, with its   */
+/* GEMMs csrc/ops/vision_ops.cpp:398-406, its mask ops                        */
+/* csrc/ops/indexing_ops.cpp:574-579 / csrc/ops/scatter_ops.cpp:43-71 and its */
+/* softmax csrc/ops/pointwise_ops.cpp:926-981)                                */
+/*   out = softmax(q k^T * scale + mask) v                                    */
+/* Causal masking is top-left aligned: query i sees keys 0..i whatever Lk is  */
+/* (attention_ops.cpp:103-116).  GQA: query head h reads kv head              */
+/* h / (Hq/Hkv); K/V are never replicated.  A row whose keys are all masked   */
+/* yields NaN, as the reference's softmax does.                               */
+/* ------------------------------------------------------------------------- */
+typedef struct paras_sdpa_args {
+    const void* q;      /* [B, Hq,  Lq, D ]  last dim contiguous              */
+    const void* k;      /* [B, Hkv, Lk, D ]                                   */
+    const void* v;      /* [B, Hkv, Lk, Dv]                                   */
+    void*       out;    /* [B, Hq,  Lq, Dv]  contiguous                       */
+    void*       attn;   /* optional [B, Hq, Lq, Lk] contiguous, dtype of q:
+                           the softmax weights the math op returns; NULL
+                           skips them (needed for the flash kernels)          */
+    float*      lse;    /* optional [B, Hq, Lq] natural-log sum-exp; or NULL  */
+    const void* mask;   /* optional mask broadcast to [B, Hq, Lq, Lk]         */
+    int32_t     mask_kind;      /* 0 none, 1 bool (1 byte, nonzero = attend),
+                                   2 additive in the dtype of q               */
+    int32_t     is_causal;      /* mutually exclusive with mask               */
+    int32_t     dtype;          /* paras_dtype of q, k, v, out, attn          */
+    int32_t     reserved;
+    int64_t     B, Hq, Hkv, Lq, Lk, D, Dv;
+    int64_t     q_strides[3];   /* element strides of dims B, H, L            */
+    int64_t     k_strides[3];
+    int64_t     v_strides[3];
+    int64_t     mask_strides[4];/* element strides over B,Hq,Lq,Lk (0 = bcast)*/
+    double      scale;          /* multiplies q k^T exactly as given          */
+} paras_sdpa_args;
+
+/* Scratch bytes the chosen kernel needs for these shapes (0 for most). */
+PARAS_API size_t paras_sdpa_workspace(const paras_sdpa_args* args);
+/* `workspace` may be NULL when paras_sdpa_workspace() returned 0. */
+PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream);
+/* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma", "decode_split"
+ * or "generic". */
+PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
+
+/* ------------------------------------------------------------------------- */
+/* MoE routing.  No reference function; each step is defined by a reference   */
+/* primitive:                                                                 */
+/*   topk  (csrc/ops/pointwise_ops.cpp:1292-1381): k largest of E logits,     */
+/*         sorted descending, ties to the lower expert index;                 */
+/*   _softmax over the k kept logits in fp32 (pointwise_ops.cpp:926-981);     */
+/*   stable argsort of the flattened [T*k] expert ids                         */
+/*         (csrc/ops/sort_ops.cpp:129-166): expert-major, (token,slot) order  */
+/*         kept inside an expert;                                             */
+/*   counts / offsets = histogram and exclusive cumsum                        */
+/*         (pointwise_ops.cpp:1221-1265).                                     */
+/* logits: [T, E] dtype `dtype`; topi: [T, k] int64; topw: [T, k] fp32;       */
+/* order: [T*k] int64 (order[p] = t*k + slot of the p-th routed row);         */
+/* inv_order: [T*k] int64 (position of flat slot in `order`; may be NULL);    */
+/* counts: [E] int64; offsets: [E+1] int64.  1 <= k <= E <= 64.               */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k,
+                              int dtype, int64_t* topi, float* topw, int64_t* order,
+                              int64_t* inv_order, int64_t* counts, int64_t* offsets,
+                              void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* MoE grouped expert FFN with SwiGLU.  Per routed row p (expert e):          */
+/*   xp = x[order[p] / k]                                   (index_select,    */
+/*                                   csrc/ops/indexing_ops.cpp:98-152)        */
+/*   g = T(xp W_gate[e]^T), u = T(xp W_up[e]^T)             (mm_out,          */
+/*                                   csrc/ops/vision_ops.cpp:388-396)         */
+/*   h = T(silu(g) * u)                                     (fused_ops.cpp    */
+/*                                   :162-194)                                */
+/*   y = T(h W_down[e]^T)                                                     */
+/*   out[t] = T( sum_slot T(y[inv_order[t*k+slot]] * T(topw[t][slot])) )      */
+/*                                   (mul_out / sum_out,                      */
+/*                                    pointwise_ops.cpp:280-284,766-774)      */
+/* x: [T, H]; w_gate, w_up: [E, I, H]; w_down: [E, H, I]; out: [T, H];        */
+/* all dtype `dtype` (bf16 or f16), GEMMs accumulate in fp32.                 */
+/* `workspace`: paras_moe_ffn_workspace(T,k,H,I) bytes of device memory.      */
+/* ------------------------------------------------------------------------- */
+PARAS_API size_t paras_moe_ffn_workspace(int64_t T, int64_t k, int64_t H, int64_t I,
+                                         int dtype);
+PARAS_API int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up,
+                            const void* w_down, const float* topw, const int64_t* order,
+                            const int64_t* inv_order, const int64_t* offsets,
+                            void* out, void* workspace, int64_t T, int64_t E, int64_t k,
+                            int64_t H, int64_t I, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PARAS_HIP_H */

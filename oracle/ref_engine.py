@@ -1,0 +1,184 @@
+"""Loader for oracle/_ref/libparas_ref.so -- the reference's own CPU flavor
+(its `paras:0` host engine), compiled from the reference sources by
+oracle/Makefile.ref.
+
+TEST INFRASTRUCTURE ONLY.  It validates the C restatement (oracle/paras_oracle.c)
+and serves as bench.py's timed CPU baseline (cpu_baseline.kind == "reference").
+
+The library claims PyTorch's PrivateUse1 device for itself, and so does the
+product's torch_paras package; one process can hold only one of them.  Use
+``load()`` in a process that has not imported torch_paras, or ``run()`` to
+evaluate a function in a child process.
+
+Only the compiled C++ is used: the reference's Python package is not imported;
+the few lines below register the device module PyTorch wants for a renamed
+PrivateUse1 backend.
+"""
+from __future__ import annotations
+
+import os
+import pickle
+import subprocess
+import sys
+import tempfile
+import types
+from pathlib import Path
+
+import torch
+
+_HERE = Path(__file__).resolve().parent
+LIB = _HERE / "_ref" / "libparas_ref.so"
+DEVICE = "paras:0"
+_loaded = False
+
+
+def available() -> bool:
+    return LIB.exists()
+
+
+def load() -> None:
+    """Registers the reference engine as device `paras` in this process."""
+    global _loaded
+    if _loaded:
+        return
+    if "torch_paras" in sys.modules:
+        raise RuntimeError("the product's torch_paras already owns PrivateUse1 in this process")
+    torch.ops.load_library(str(LIB))
+    torch.utils.rename_privateuse1_backend("paras")
+    mod = types.ModuleType("torch.paras")
+    mod.device_count = lambda: 1
+    mod.is_available = lambda: True
+    mod.current_device = lambda: 0
+    mod.is_bad_fork = lambda: False
+    mod._is_in_bad_fork = lambda: False
+    mod.manual_seed_all = lambda seed: None
+    mod.get_amp_supported_dtype = lambda: [torch.float16, torch.float32]
+    torch._register_device_module("paras", mod)
+    _loaded = True
+
+
+# --- functions evaluated on the reference engine (inputs/outputs: CPU tensors) ---
+def _dev(t):
+    return t.to(DEVICE) if torch.is_tensor(t) else t
+
+
+def _cpu(x):
+    if torch.is_tensor(x):
+        return x.cpu()
+    if isinstance(x, (tuple, list)):
+        return tuple(_cpu(i) for i in x)
+    return x
+
+
+def rms_norm(x, w, eps):
+    return _cpu(torch.ops.paras.rms_norm(_dev(x), _dev(w), eps))
+
+
+def rms_norm_backward(go, x, w, rstd):
+    return _cpu(torch.ops.paras.rms_norm_backward(_dev(go), _dev(x), _dev(w), _dev(rstd)))
+
+
+def swiglu(gate, up):
+    return _cpu(torch.ops.paras.swiglu(_dev(gate), _dev(up)))
+
+
+def swiglu_backward(go, gate, up):
+    return _cpu(torch.ops.paras.swiglu_backward(_dev(go), _dev(gate), _dev(up)))
+
+
+def rotate_half(x, backward=False):
+    fn = torch.ops.paras.rotate_half_backward if backward else torch.ops.paras.rotate_half
+    return _cpu(fn(_dev(x)))
+
+
+def rms_norm_composed(x, normalized_shape, weight=None, eps=None):
+    return _cpu(torch.ops.aten.rms_norm(_dev(x), list(normalized_shape), _dev(weight), eps))
+
+
+def swiglu_composed(x, gate):
+    return _cpu(torch.ops.torch_paras.swiglu(_dev(x), _dev(gate)))
+
+
+def sdpa_math(q, k, v, attn_mask=None, is_causal=False, scale=None, enable_gqa=False):
+    return _cpu(torch.ops.aten._scaled_dot_product_attention_math(
+        _dev(q), _dev(k), _dev(v), _dev(attn_mask), 0.0, is_causal, None, scale=scale, enable_gqa=enable_gqa))
+
+
+def softmax_last(x, out_dtype=None):
+    half_to_float = out_dtype is not None and out_dtype != x.dtype
+    return _cpu(torch.ops.aten._softmax(_dev(x), -1, half_to_float))
+
+
+def topk_last(x, k, largest=True):
+    return _cpu(torch.topk(_dev(x), k, dim=-1, largest=largest, sorted=True))
+
+
+def argsort_stable(keys):
+    return _cpu(torch.argsort(_dev(keys), dim=-1, stable=True))
+
+
+def moe_route(logits, k):
+    """The canonical MoE routing composition, each step on the reference engine."""
+    d = _dev(logits)
+    T, E = logits.shape
+    topv, topi = torch.topk(d, k, dim=-1)
+    topw = torch.ops.aten._softmax(topv.float(), -1, False)
+    flat_e = topi.reshape(-1)
+    order = torch.argsort(flat_e, dim=-1, stable=True)
+    inv = torch.argsort(order, dim=-1, stable=True)
+    flat_cpu = flat_e.cpu()
+    counts = torch.bincount(flat_cpu, minlength=E).to(torch.int64)
+    offsets = torch.zeros(E + 1, dtype=torch.int64)
+    offsets[1:] = torch.cumsum(counts, 0)
+    return topi.cpu(), topw.cpu(), order.cpu(), inv.cpu(), counts, offsets
+
+
+def moe_ffn(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, k):
+    T, H = x.shape
+    E = w_gate.shape[0]
+    dx = _dev(x)
+    xp = torch.index_select(dx, 0, _dev(order // k))
+    ys = []
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi == lo:
+            continue
+        rows = xp[lo:hi]
+        g = torch.mm(rows, _dev(w_gate[e]).t())
+        u = torch.mm(rows, _dev(w_up[e]).t())
+        h = torch.ops.paras.swiglu(g, u)
+        ys.append(torch.mm(h, _dev(w_down[e]).t()))
+    y = torch.cat([t.cpu() for t in ys], 0).to(DEVICE)
+    yt = torch.index_select(y, 0, _dev(inv_order)).reshape(T, k, H)
+    wt = _dev(topw).to(x.dtype).reshape(T, k, 1)
+    return (yt * wt).sum(1).cpu()
+
+
+# --- child-process evaluation ----------------------------------------------------
+def run(fn_name: str, *args, threads: int | None = None, **kwargs):
+    """Evaluates ``ref_engine.<fn_name>(*args, **kwargs)`` in a child process and
+    returns its result (CPU tensors travel through a temporary file written
+    and read by this module only)."""
+    with tempfile.TemporaryDirectory() as td:
+        inp, outp = Path(td) / "in.pt", Path(td) / "out.pt"
+        torch.save({"fn": fn_name, "args": args, "kwargs": kwargs}, inp)
+        env = dict(os.environ)
+        if threads:
+            env["PTSYCL_CPU_THREADS"] = str(threads)
+            env["OMP_NUM_THREADS"] = str(threads)
+        proc = subprocess.run([sys.executable, str(Path(__file__).resolve()), str(inp), str(outp)],
+                              capture_output=True, text=True, env=env)
+        if proc.returncode != 0:
+            raise RuntimeError(f"reference engine failed:\n{proc.stdout}\n{proc.stderr}")
+        return torch.load(outp, weights_only=False)
+
+
+def _child(inp: str, outp: str) -> None:
+    load()
+    req = torch.load(inp, weights_only=False)
+    fn = globals()[req["fn"]]
+    torch.save(fn(*req["args"], **req["kwargs"]), outp)
+
+
+if __name__ == "__main__":
+    _child(sys.argv[1], sys.argv[2])
