@@ -1,0 +1,349 @@
+// MoE grouped expert FFN for gfx950: two grouped GEMMs on bf16/fp16 MFMA with
+// fp32 accumulation, and the weighted combine.
+//
+//   GEMM 1   h[p, :] = T( silu(T(xp W_gate[e]^T)) * T(xp W_up[e]^T) )
+//            xp = x[order[p] / k] is gathered inside the A-tile load (no
+//            permuted copy of x is ever written); gate and up columns of the
+//            same tile are accumulated side by side and the SwiGLU runs in
+//            the epilogue on the values already rounded to T, as the composed
+//            reference would see them (mm -> T, paras::swiglu -> T).
+//   GEMM 2   y[p, :] = T( h[p, :] W_down[e]^T )
+//   combine  out[t] = T( sum_slot T( y[inv_order[t*k+slot]] * T(topw[t][slot]) ) )
+//
+// Both products are "NT": A rows and weight rows are contiguous along the
+// contraction dim, which is exactly the 8-element-per-lane operand layout of
+// v_mfma_f32_32x32x16, so neither operand needs a transpose.
+//
+// Tiling: workgroup = 4 waves = 128 routed rows x two 128-column groups (gate
+// and up columns n0..n0+127 for GEMM 1; columns n0..n0+255 for GEMM 2), k-tile
+// 64, waves arranged 2x2 with 64x64 per column group each (128 fp32
+// accumulators per lane).  Global -> registers -> LDS with the next k-tile's
+// loads in flight during the MFMAs.  Rows of one expert are contiguous in the
+// routed order; m-tiles never straddle experts (the grid is sized for the
+// worst case and surplus workgroups exit).  The block index is unscrambled so
+// that the workgroups resident on one XCD cover all m-tiles of a few column
+// tiles: weight tiles are then shared through that XCD's L2.
+#include <hip/hip_runtime.h>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+#include "kernels/swiglu_math.h"
+
+namespace paras {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kBM = 128;
+constexpr int kBN = 128;          // columns per group; a workgroup computes two groups
+constexpr int kBK = 64;
+constexpr int kLS = kBK + 8;      // LDS row stride (elements): 16 consecutive rows hit distinct banks
+
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+
+struct FfnGemmParams {
+    const std::uint16_t* a;     // x [T, K] (gathered) or h [R, K]
+    const std::uint16_t* b;     // weights of column group 0, [E, Nw, K]
+    const std::uint16_t* b2;    // weights of column group 1 (same layout)
+    std::uint16_t* c;           // [R, N]
+    const long* order;          // gather index (routed row -> flat (token, slot)); null = direct rows
+    const long* offsets;        // [E+1]
+    long K, N, Nw, R;           // contraction, output columns, weight rows per expert, routed rows
+    int E, k;
+    int mt_total;               // upper bound on m-tiles
+    int n_units;                // column units (128 output columns for GEMM 1, 256 for GEMM 2)
+    int ngt;                    // column units an XCD sweeps together
+};
+
+template <typename T> struct MmaT;
+template <> struct MmaT<bf16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct MmaT<f16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+template <typename T, bool kSwiglu>
+__global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemmParams p) {
+    using El = Elem<T>;
+    __shared__ __attribute__((aligned(16))) std::uint16_t a_lds[kBM * kLS];
+    __shared__ __attribute__((aligned(16))) std::uint16_t b_lds[2][kBN * kLS];
+
+    // ---- tile coordinates.  Linear id L: xcd = L % 8 (hardware round-robin);
+    // within an XCD walk (column group, m-tile, column-in-group).
+    int mt, nu;
+    {
+        const long L = blockIdx.x;
+        const int xcd = static_cast<int>(L & 7);
+        const long j = L >> 3;
+        const long per_group = static_cast<long>(p.mt_total) * p.ngt;
+        const long g = j / per_group, rem = j % per_group;
+        mt = static_cast<int>(rem / p.ngt);
+        nu = static_cast<int>((g * 8 + xcd) * p.ngt + rem % p.ngt);
+        if (nu >= p.n_units) return;
+    }
+    // m-tile -> (expert, first row)
+    int e = 0;
+    long row0 = 0, row_end = 0;
+    {
+        int tiles_before = 0;
+        bool found = false;
+        for (int i = 0; i < p.E; ++i) {
+            const long lo = p.offsets[i], hi = p.offsets[i + 1];
+            const int tiles = static_cast<int>((hi - lo + kBM - 1) / kBM);
+            if (!found && mt < tiles_before + tiles) {
+                e = i;
+                row0 = lo + static_cast<long>(mt - tiles_before) * kBM;
+                row_end = hi;
+                found = true;
+            }
+            tiles_before += tiles;
+        }
+        if (!found) return;
+    }
+    const long n0 = static_cast<long>(nu) * (kSwiglu ? kBN : 2 * kBN);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lh = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- global -> register staging: 16-byte chunks, 8 per row of a k-tile
+    const std::uint16_t* a_ptr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + i * kThreads;
+        long prow = row0 + (c >> 3);
+        if (prow >= row_end) prow = row_end - 1;  // clamp: result rows beyond the expert are not stored
+        const long src = p.order ? p.order[prow] / p.k : prow;
+        a_ptr[i] = p.a + src * p.K + (c & 7) * 8;
+    }
+    const std::uint16_t* b_ptr[2][4];
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * kThreads;
+            long wrow = (kSwiglu ? n0 : n0 + g * kBN) + (c >> 3);
+            if (wrow >= p.Nw) wrow = p.Nw - 1;
+            const std::uint16_t* base = g == 0 ? p.b : p.b2;
+            b_ptr[g][i] = base + (static_cast<long>(e) * p.Nw + wrow) * p.K + (c & 7) * 8;
+        }
+    u32x4 a_st[4], b_st[2][4];
+    auto load_tile = [&](long k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_ptr[i] + k0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_ptr[g][i] + k0);
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * kThreads;
+            const int off = (c >> 3) * kLS + (c & 7) * 8;
+            *reinterpret_cast<u32x4*>(&a_lds[off]) = a_st[i];
+            *reinterpret_cast<u32x4*>(&b_lds[0][off]) = b_st[0][i];
+            *reinterpret_cast<u32x4*>(&b_lds[1][off]) = b_st[1][i];
+        }
+    };
+
+    float16_t acc[2][2][2];
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[g][mi][ni][r] = 0.f;
+
+    const int a_off = (wm * 64 + lr) * kLS + lh * 8;
+    const int b_off = (wn * 64 + lr) * kLS + lh * 8;
+    const long k_tiles = p.K / kBK;
+    load_tile(0);
+    store_tile();
+    __syncthreads();
+    for (long kt = 0; kt < k_tiles; ++kt) {
+        if (kt + 1 < k_tiles) load_tile((kt + 1) * kBK);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            i16x8 af[2], bf[2][2];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+                af[mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off + mi * 32 * kLS + ks * 16]);
+#pragma unroll
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    bf[g][ni] = *reinterpret_cast<const i16x8*>(&b_lds[g][b_off + ni * 32 * kLS + ks * 16]);
+#pragma unroll
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni)
+                        acc[g][mi][ni] = MmaT<T>::run(af[mi], bf[g][ni], acc[g][mi][ni]);
+        }
+        __syncthreads();
+        if (kt + 1 < k_tiles) {
+            store_tile();
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue.  Accumulator lane (column lr, half lh) holds rows (r/4)*8 + 4*lh + r%4.
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+            const long col = n0 + wn * 64 + ni * 32 + lr;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const long prow = row0 + wm * 64 + mi * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                if (prow >= row_end) continue;
+                if (kSwiglu) {
+                    if (col < p.N) {
+                        const auto g = El::from_f32(acc[0][mi][ni][r]);
+                        const auto u = El::from_f32(acc[1][mi][ni][r]);
+                        p.c[prow * p.N + col] = swiglu_one<T>(g, u);
+                    }
+                } else {
+                    if (col < p.N) p.c[prow * p.N + col] = El::from_f32(acc[0][mi][ni][r]);
+                    if (col + kBN < p.N) p.c[prow * p.N + col + kBN] = El::from_f32(acc[1][mi][ni][r]);
+                }
+            }
+        }
+}
+
+// out[t, :] = T( sum_slot T( y[inv[t*k+slot], :] * T(w[t, slot]) ) ), 8 columns per lane.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void moe_combine_kernel(const std::uint16_t* __restrict__ y,
+                                                              const float* __restrict__ topw,
+                                                              const long* __restrict__ inv_order,
+                                                              std::uint16_t* __restrict__ out, long T_, int k, long H) {
+    using El = Elem<T>;
+    const long hv = H / 8;
+    const long total = T_ * hv;
+    for (long i = static_cast<long>(blockIdx.x) * kThreads + threadIdx.x; i < total;
+         i += static_cast<long>(gridDim.x) * kThreads) {
+        const long t = i / hv, c = (i % hv) * 8;
+        double acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int s = 0; s < k; ++s) {
+            const long prow = inv_order[t * k + s];
+            const double w = El::to_f64(El::from_f32(topw[t * k + s]));  // w.to(T)
+            const u32x4 v = load16(y + prow * H + c);
+            const std::uint16_t* ve = reinterpret_cast<const std::uint16_t*>(&v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] += El::to_f64(El::from_f64(El::to_f64(ve[j]) * w));
+        }
+        u32x4 o;
+        std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) oe[j] = El::from_f64(acc[j]);
+        store16(out + t * H + c, o);
+    }
+}
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+template <typename T>
+int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
+            const long* order, const long* inv_order, const long* offsets, void* out, void* workspace, long T_,
+            int E, int k, long H, long I, hipStream_t s) {
+    const long R = T_ * k;
+    auto* h = static_cast<std::uint16_t*>(workspace);
+    auto* y = reinterpret_cast<std::uint16_t*>(static_cast<char*>(workspace) + align_up(static_cast<size_t>(R) * I * 2, 256));
+    const int mt_total = static_cast<int>((R + kBM - 1) / kBM) + E;
+
+    FfnGemmParams g1{};
+    g1.a = static_cast<const std::uint16_t*>(x);
+    g1.b = static_cast<const std::uint16_t*>(w_gate);
+    g1.b2 = static_cast<const std::uint16_t*>(w_up);
+    g1.c = h;
+    g1.order = order;
+    g1.offsets = offsets;
+    g1.K = H; g1.N = I; g1.Nw = I; g1.R = R; g1.E = E; g1.k = k;
+    g1.mt_total = mt_total;
+    g1.n_units = static_cast<int>((I + kBN - 1) / kBN);
+    // Column units an XCD sweeps together: up to 4, fewer when there are not
+    // enough units to keep all 8 XCDs busy.
+    auto plan = [](FfnGemmParams& g) {
+        int ngt = g.n_units / 8;
+        g.ngt = ngt < 1 ? 1 : (ngt > 4 ? 4 : ngt);
+    };
+    auto grid_of = [&](const FfnGemmParams& g) {
+        const long groups = (g.n_units + 8 * g.ngt - 1) / (8 * g.ngt);
+        return static_cast<unsigned>(groups * 8 * g.ngt * g.mt_total);
+    };
+    plan(g1);
+    hipLaunchKernelGGL((grouped_gemm_kernel<T, true>), dim3(grid_of(g1)), dim3(kThreads), 0, s, g1);
+    PARAS_HIP_TRY(hipGetLastError());
+
+    FfnGemmParams g2{};
+    g2.a = h;
+    g2.b = static_cast<const std::uint16_t*>(w_down);
+    g2.b2 = g2.b;  // column group 1 = the next 128 weight rows, selected through the row index
+    g2.c = y;
+    g2.order = nullptr;
+    g2.offsets = offsets;
+    g2.K = I; g2.N = H; g2.Nw = H; g2.R = R; g2.E = E; g2.k = k;
+    g2.mt_total = mt_total;
+    g2.n_units = static_cast<int>((H + 2 * kBN - 1) / (2 * kBN));
+    plan(g2);
+    hipLaunchKernelGGL((grouped_gemm_kernel<T, false>), dim3(grid_of(g2)), dim3(kThreads), 0, s, g2);
+    PARAS_HIP_TRY(hipGetLastError());
+
+    const long total = T_ * (H / 8);
+    long blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    hipLaunchKernelGGL((moe_combine_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, y, topw,
+                       inv_order, static_cast<std::uint16_t*>(out), T_, k, H);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // namespace
+}  // namespace paras
+
+extern "C" {
+
+size_t paras_moe_ffn_workspace(int64_t T, int64_t k, int64_t H, int64_t I, int dtype) {
+    (void)dtype;
+    if (T <= 0 || k <= 0 || H <= 0 || I <= 0) return 0;
+    const size_t R = static_cast<size_t>(T) * k;
+    return paras::align_up(R * I * 2, 256) + paras::align_up(R * H * 2, 256);
+}
+
+int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
+                  const int64_t* order, const int64_t* inv_order, const int64_t* offsets, void* out,
+                  void* workspace, int64_t T, int64_t E, int64_t k, int64_t H, int64_t I, int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(T >= 0 && E >= 1 && k >= 1 && H >= 1 && I >= 1, "paras_moe_ffn: bad shape");
+    if (T == 0) return PARAS_OK;
+    PARAS_REQUIRE(dtype == PARAS_BF16 || dtype == PARAS_F16, "paras_moe_ffn: dtype must be bf16 or f16");
+    if (H % kBK != 0 || I % kBK != 0)
+        return fail(PARAS_ERR_UNSUPPORTED, "paras_moe_ffn: hidden (%lld) and intermediate (%lld) sizes must be multiples of %d",
+                    (long long)H, (long long)I, kBK);
+    PARAS_REQUIRE(x && w_gate && w_up && w_down && topw && order && inv_order && offsets && out && workspace,
+                  "paras_moe_ffn: null pointer");
+    PARAS_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_gate) | reinterpret_cast<uintptr_t>(w_up) |
+                    reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0,
+                  "paras_moe_ffn: tensors must be 16-byte aligned");
+    PARAS_REQUIRE(T * k <= 0x3fffffffLL, "paras_moe_ffn: too many routed rows");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    const long* ord = reinterpret_cast<const long*>(order);
+    const long* inv = reinterpret_cast<const long*>(inv_order);
+    const long* off = reinterpret_cast<const long*>(offsets);
+    if (dtype == PARAS_BF16)
+        return run_ffn<bf16_t>(x, w_gate, w_up, w_down, topw, ord, inv, off, out, workspace, T, (int)E, (int)k, H, I, s);
+    return run_ffn<f16_t>(x, w_gate, w_up, w_down, topw, ord, inv, off, out, workspace, T, (int)E, (int)k, H, I, s);
+}
+
+}  // extern "C"

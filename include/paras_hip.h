@@ -213,11 +213,14 @@ PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 /* order: [T*k] int64 (order[p] = t*k + slot of the p-th routed row);         */
 /* inv_order: [T*k] int64 (position of flat slot in `order`; may be NULL);    */
 /* counts: [E] int64; offsets: [E+1] int64.  1 <= k <= E <= 64.               */
+/* `workspace`: paras_moe_route_workspace(T,E,k) bytes of device memory        */
+/* (per-workgroup histograms).                                                 */
 /* ------------------------------------------------------------------------- */
+PARAS_API size_t paras_moe_route_workspace(int64_t T, int64_t E, int64_t k);
 PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k,
                               int dtype, int64_t* topi, float* topw, int64_t* order,
                               int64_t* inv_order, int64_t* counts, int64_t* offsets,
-                              void* stream);
+                              void* workspace, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* MoE grouped expert FFN with SwiGLU.  Per routed row p (expert e):          */

@@ -17,7 +17,6 @@ PrivateUse1 backend.
 from __future__ import annotations
 
 import os
-import pickle
 import subprocess
 import sys
 import tempfile
@@ -171,6 +170,16 @@ def run(fn_name: str, *args, threads: int | None = None, **kwargs):
         if proc.returncode != 0:
             raise RuntimeError(f"reference engine failed:\n{proc.stdout}\n{proc.stderr}")
         return torch.load(outp, weights_only=False)
+
+
+def run_batch(jobs, threads: int | None = None):
+    """jobs: list of (fn_name, args, kwargs); one child process evaluates them
+    all and the list of results comes back in the same order."""
+    return run("_batch", jobs, threads=threads)
+
+
+def _batch(jobs):
+    return [globals()[name](*args, **kwargs) for name, args, kwargs in jobs]
 
 
 def _child(inp: str, outp: str) -> None:

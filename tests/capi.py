@@ -54,7 +54,8 @@ SIGNATURES = {
     "paras_sdpa_workspace": (sz, [C.POINTER(SdpaArgs)]),
     "paras_sdpa_fwd": (i32, [C.POINTER(SdpaArgs), vp, vp]),
     "paras_sdpa_kernel_name": (C.c_char_p, [C.POINTER(SdpaArgs)]),
-    "paras_moe_route": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp]),
+    "paras_moe_route_workspace": (sz, [i64, i64, i64]),
+    "paras_moe_route": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp]),
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
 }
@@ -196,8 +197,9 @@ def moe_route(logits, k):
     inv = torch.empty(T * k, dtype=torch.int64, device=dev)
     counts = torch.empty(E, dtype=torch.int64, device=dev)
     offsets = torch.empty(E + 1, dtype=torch.int64, device=dev)
+    ws = torch.empty(max(1, lib().paras_moe_route_workspace(T, E, k)), dtype=torch.uint8, device=dev)
     check(lib().paras_moe_route(_ptr(logits), T, E, k, DT[logits.dtype], _ptr(topi), _ptr(topw), _ptr(order),
-                                _ptr(inv), _ptr(counts), _ptr(offsets), _stream()))
+                                _ptr(inv), _ptr(counts), _ptr(offsets), _ptr(ws), _stream()))
     return topi, topw, order, inv, counts, offsets
 
 

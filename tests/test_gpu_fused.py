@@ -1,0 +1,141 @@
+"""GPU parity of the fused RMSNorm / SwiGLU / rotate_half kernels, through the
+C ABI, against the CPU oracle and the golden vectors.  Bar: bit-exact for
+fp32 / bf16 / fp16 (the kernels evaluate the host engine's fp64 formula);
+fp64 tensors within 1e-13 relative (summation order / exp last bit)."""
+import pytest
+import torch
+
+import capi
+import oracle as O
+from conftest import assert_bit_exact
+from golden_util import DTYPE_TAGS, case
+
+pytestmark = pytest.mark.gpu
+EXACT = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def dev(t):
+    return t.cuda()
+
+
+@pytest.mark.parametrize("tag", DTYPE_TAGS)
+def test_golden_vectors(tag):
+    c = case(f"rms_norm_{tag}")
+    out, rstd = capi.rms_norm(dev(c["x"]), dev(c["w"]), 1e-6)
+    assert_bit_exact(out, c["out"], "rms_norm")
+    assert_bit_exact(rstd, c["rstd"], "rstd")
+    gx, gw = capi.rms_norm_backward(dev(c["go"]), dev(c["x"]), dev(c["w"]), dev(c["rstd"]))
+    assert_bit_exact(gx, c["gx"], "grad_input")
+    if tag == "f32":
+        assert torch.allclose(gw.cpu(), c["gw"], rtol=1e-6, atol=1e-6)   # slab-wise column sums
+    else:
+        assert_bit_exact(gw, c["gw"], "grad_weight")
+    c = case(f"swiglu_{tag}")
+    assert_bit_exact(capi.swiglu(dev(c["gate"]), dev(c["up"])), c["out"], "swiglu")
+    gg, gu = capi.swiglu_backward(dev(c["go"]), dev(c["gate"]), dev(c["up"]))
+    assert_bit_exact(gg, c["ggate"], "grad_gate")
+    assert_bit_exact(gu, c["gup"], "grad_up")
+    c = case(f"rotate_half_{tag}")
+    assert_bit_exact(capi.rotate_half(dev(c["x"])), c["out"], "rotate_half")
+    assert_bit_exact(capi.rotate_half(dev(c["x"]), True), c["bwd"], "rotate_half_backward")
+
+
+@pytest.mark.parametrize("dtype", EXACT)
+@pytest.mark.parametrize("shape", [(7, 200), (33, 4096), (5, 8192), (3, 10000), (64, 1024), (2, 8), (1, 1), (300, 264)])
+def test_rms_norm_matches_oracle(dtype, shape):
+    x = torch.randn(*shape).to(dtype)
+    w = (1 + 0.02 * torch.randn(shape[1])).to(dtype)
+    out, rstd = capi.rms_norm(dev(x), dev(w), 1e-6)
+    want, wrstd = O.rms_norm(x, w, 1e-6)
+    assert_bit_exact(out, want, f"rms_norm {dtype} {shape}")
+    assert_bit_exact(rstd, wrstd, "rstd")
+
+
+def test_rms_norm_unaligned_and_3d():
+    base = torch.randn(4 * 6 * 40 + 3).bfloat16()
+    x = base[3:].view(4, 6, 40)            # data pointer not 16-byte aligned on the device copy below
+    w = torch.randn(40).bfloat16()
+    xd = dev(base)[3:].view(4, 6, 40)
+    out, rstd = capi.rms_norm(xd, dev(w), 1e-5)
+    want, wrstd = O.rms_norm(x.contiguous(), w, 1e-5)
+    assert_bit_exact(out, want, "unaligned rms_norm")
+    assert out.shape == (4, 6, 40) and rstd.shape == (24,)
+
+
+def test_rms_norm_fp64_and_empty():
+    x, w = torch.randn(9, 300, dtype=torch.float64), torch.randn(300, dtype=torch.float64)
+    out, rstd = capi.rms_norm(dev(x), dev(w), 1e-6)
+    want, _ = O.rms_norm(x, w, 1e-6)
+    assert torch.allclose(out.cpu(), want, rtol=1e-13, atol=1e-13)
+    out, rstd = capi.rms_norm(torch.empty(0, 8, device="cuda"), torch.ones(8, device="cuda"), 1e-6)
+    assert out.shape == (0, 8) and rstd.shape == (0,)
+
+
+@pytest.mark.parametrize("dtype", EXACT)
+@pytest.mark.parametrize("n", [1, 13, 4096, 100003])
+def test_swiglu_matches_oracle(dtype, n):
+    gate, up = (3 * torch.randn(n)).to(dtype), torch.randn(n).to(dtype)
+    assert_bit_exact(capi.swiglu(dev(gate), dev(up)), O.swiglu(gate, up), f"swiglu {dtype} n={n}")
+
+
+def test_swiglu_extreme_gates_take_the_exact_tier():
+    """Gates outside the range of the fp32 fast path, zeros, infinities, NaN."""
+    vals = [0.0, -0.0, 1e-30, -1e-30, -8.0, -8.5, -20.0, -60.0, -100.0, -700.0, 8.0, 60.0, 61.0, 100.0, 3e38,
+            float("inf"), float("-inf"), float("nan")]
+    gate = torch.tensor(vals).repeat_interleave(len(vals))
+    up = torch.tensor(vals).repeat(len(vals))
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        g, u = gate.to(dtype), up.to(dtype)
+        assert_bit_exact(capi.swiglu(dev(g), dev(u)), O.swiglu(g, u), f"swiglu extremes {dtype}")
+
+
+def test_swiglu_every_bf16_gate():
+    """All 65536 bf16 gate bit patterns against a few up values: the two-tier
+    evaluation equals the fp64-then-round definition everywhere."""
+    gate = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    for upv in (1.0, -0.3, 7.25, 1e-3):
+        up = torch.full_like(gate, upv)
+        assert_bit_exact(capi.swiglu(dev(gate), dev(up)), O.swiglu(gate, up), f"all gates, up={upv}")
+
+
+@pytest.mark.parametrize("dtype", EXACT)
+def test_backward_ops_match_oracle(dtype):
+    x, w, go = torch.randn(50, 320).to(dtype), torch.randn(320).to(dtype), torch.randn(50, 320).to(dtype)
+    _, rstd = O.rms_norm(x, w, 1e-6)
+    gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(rstd))
+    wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
+    assert_bit_exact(gx, wgx, "rms_norm grad_input")
+    if dtype == torch.float32:
+        assert torch.allclose(gw.cpu(), wgw, rtol=1e-6, atol=1e-6)
+    else:
+        assert_bit_exact(gw, wgw, "rms_norm grad_weight")
+    gate, up, g2 = torch.randn(1000).to(dtype), torch.randn(1000).to(dtype), torch.randn(1000).to(dtype)
+    gg, gu = capi.swiglu_backward(dev(g2), dev(gate), dev(up))
+    wgg, wgu = O.swiglu_backward(g2, gate, up)
+    assert_bit_exact(gg, wgg, "swiglu grad_gate")
+    assert_bit_exact(gu, wgu, "swiglu grad_up")
+    xr = torch.randn(6, 10).to(dtype)
+    assert_bit_exact(capi.rotate_half(dev(xr)), O.rotate_half(xr), "rotate_half")
+    with pytest.raises(capi.ParasError):
+        capi.rotate_half(torch.randn(4, 7, device="cuda"))          # odd last dim
+
+
+def test_full_size_rms_norm_and_swiglu_bf16():
+    """BASELINE config 2 at its real size, bit-exact against the oracle."""
+    x = torch.randn(16384, 4096).bfloat16()
+    w = (1 + 0.02 * torch.randn(4096)).bfloat16()
+    out, rstd = capi.rms_norm(dev(x), dev(w), 1e-6)
+    want, wrstd = O.rms_norm(x, w, 1e-6)
+    assert_bit_exact(out, want, "rms_norm 16384x4096")
+    assert_bit_exact(rstd, wrstd, "rstd")
+    del x, out, want
+    # SwiGLU: a 2048-row slab of the 16384 x 14336 tensor against the oracle,
+    # the whole tensor through size-independent properties
+    gate, up = torch.randn(16384, 14336).bfloat16(), torch.randn(16384, 14336).bfloat16()
+    gd, ud = dev(gate), dev(up)
+    res = capi.swiglu(gd, ud)
+    assert_bit_exact(res[:2048], O.swiglu(gate[:2048], up[:2048]), "swiglu slab")
+    assert_bit_exact(res[-64:], O.swiglu(gate[-64:], up[-64:]), "swiglu tail")
+    neg = capi.swiglu(gd, -ud)
+    assert torch.equal(neg.view(torch.int16) ^ res.view(torch.int16),
+                       torch.full_like(res.view(torch.int16), -32768))    # odd in `up`, bit for bit

@@ -1,0 +1,132 @@
+"""GPU parity of MoE routing (bit-exact integers) and the grouped expert FFN.
+
+FFN bar: bf16 / fp16 within 2e-2 absolute of the host-engine oracle, or one
+unit in the last place of the 16-bit result where that is larger (|y| >= 4 for
+bf16: a GEMM whose fp32 summation order differs from ATen's flips the final
+rounding of a few outputs, by exactly one ulp)."""
+import pytest
+import torch
+
+import capi
+import oracle as O
+from conftest import assert_bit_exact
+from golden_util import DTYPE_TAGS, case
+
+pytestmark = pytest.mark.gpu
+NAMES = ("topi", "topw", "order", "inv", "counts", "offsets")
+
+
+def ulp16(ref, dtype):
+    mant = 7 if dtype == torch.bfloat16 else 10
+    return 2.0 ** (torch.floor(torch.log2(ref.double().abs().clamp_min(1e-30))) - mant)
+
+
+def assert_ffn_close(out, ref, dtype):
+    """Per element: max(2e-2, one 16-bit ulp of the reference value).  A GEMM
+    whose fp32 summation order differs from ATen's flips the last bit of a few
+    intermediate y values; weighted and re-rounded they reach the output as at
+    most one ulp of the top binade of the outputs, for at most 1 element in
+    1000."""
+    err = (out.double().cpu() - ref.double()).abs()
+    tol = torch.maximum(torch.full_like(err, 2e-2), ulp16(ref, dtype) * 1.001)
+    frac = float((err > tol).double().mean())
+    top = float(ulp16(ref.double().abs().max() * 1.999, dtype))
+    assert frac <= 1e-3, f"{frac:.2e} of elements beyond max(2e-2, 1 ulp); worst {err.max().item():.3e}"
+    assert err.max().item() <= max(2e-2, top) * 1.001, f"worst {err.max().item():.3e} > one ulp of the top binade {top:.3e}"
+    return err
+
+
+@pytest.mark.parametrize("tag", DTYPE_TAGS)
+def test_route_golden(tag):
+    c = case(f"moe_route_{tag}")
+    got = capi.moe_route(c["logits"].cuda(), 2)
+    for name, g in zip(NAMES, got):
+        assert_bit_exact(g, c[name], f"moe_route {name}")
+
+
+@pytest.mark.parametrize("shape", [(1, 8, 2), (100, 8, 2), (1000, 8, 2), (777, 16, 4), (300, 64, 8), (5000, 3, 3),
+                                   (8192, 8, 2), (257, 1, 1), (4096, 8, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_route_matches_oracle(shape, dtype):
+    T, E, k = shape
+    logits = torch.randn(T, E).to(dtype)
+    if T > 10:
+        logits[3] = logits[3, 0]                       # every expert tied
+        logits[7, E // 2] = logits[7, 0]
+    got = capi.moe_route(logits.cuda(), k)
+    want = O.moe_route(logits, k)
+    for name, g, w in zip(NAMES, got, want):
+        assert_bit_exact(g, w, f"moe_route {name} T{T} E{E} k{k} {dtype}")
+
+
+def test_route_quantised_logits_many_ties_and_skew():
+    logits = torch.randint(-2, 3, (3000, 8)).float().bfloat16()     # 5 distinct values: ties everywhere
+    logits[:, 5] += 5                                                 # one hot expert: skewed counts
+    logits[:, 2] -= 9                                                 # one expert never chosen
+    got = capi.moe_route(logits.cuda(), 2)
+    want = O.moe_route(logits, 2)
+    for name, g, w in zip(NAMES, got, want):
+        assert_bit_exact(g, w, f"moe_route {name}")
+    assert got[4][2].item() == 0 and got[4][5].item() == 3000
+
+
+def test_route_errors_and_empty():
+    with pytest.raises(capi.ParasError, match="k out of range"):
+        capi.moe_route(torch.randn(4, 8, device="cuda"), 9)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(torch.empty(0, 8, device="cuda"), 2)
+    assert counts.tolist() == [0] * 8 and offsets.tolist() == [0] * 9
+
+
+def test_ffn_golden():
+    c = case("moe_ffn_bf16")
+    d = {k: v.cuda() for k, v in c.items()}
+    out = capi.moe_ffn(d["x"], d["wg"], d["wu"], d["wd"], d["topw"], d["order"], d["inv"], d["offsets"], 2)
+    assert_ffn_close(out, c["out"], torch.bfloat16)
+
+
+@pytest.mark.parametrize("shape", [(64, 4, 2, 128, 256), (300, 8, 2, 256, 512), (100, 8, 2, 128, 192), (257, 3, 1, 64, 64),
+                                   (500, 8, 4, 320, 448)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_ffn_matches_oracle(shape, dtype):
+    T, E, k, H, I = shape
+    x, logits = torch.randn(T, H).to(dtype), torch.randn(T, E).to(dtype)
+    logits[:, E - 1] -= 20                              # an expert that receives no token
+    wg, wu = (0.05 * torch.randn(E, I, H)).to(dtype), (0.05 * torch.randn(E, I, H)).to(dtype)
+    wd = (0.05 * torch.randn(E, H, I)).to(dtype)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    r = O.moe_route(logits, k)
+    want = O.moe_ffn(x, wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
+    err = assert_ffn_close(out, want, dtype)
+    assert err.mean().item() < 1e-3
+
+
+def test_ffn_rejects_unsupported_sizes():
+    T, E, k = 16, 2, 1
+    with pytest.raises(capi.ParasError, match="multiples of 64"):
+        z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
+        route = capi.moe_route(torch.randn(T, E, device="cuda").bfloat16(), k)
+        capi.moe_ffn(z(T, 72), z(E, 64, 72), z(E, 64, 72), z(E, 72, 64), route[1], route[2], route[3], route[5], k)
+
+
+def test_config5_routing_exact_and_sampled_tokens():
+    """BASELINE config 5 (T=8192 H=4096 E=8 top-2 I=14336 bf16) at full size:
+    routing bit-exact on all tokens, the FFN on 48 sampled tokens against the
+    oracle (a token's output depends only on its own row and routing)."""
+    T, H, E, k, I = 8192, 4096, 8, 2, 14336
+    dt = torch.bfloat16
+    logits, x = torch.randn(T, E).to(dt), torch.randn(T, H).to(dt)
+    wg, wu = (0.02 * torch.randn(E, I, H)).to(dt), (0.02 * torch.randn(E, I, H)).to(dt)
+    wd = (0.02 * torch.randn(E, H, I)).to(dt)
+    got = capi.moe_route(logits.cuda(), k)
+    want = O.moe_route(logits, k)
+    for name, g, w in zip(NAMES, got, want):
+        assert_bit_exact(g, w, f"config 5 moe_route {name}")
+    topi, topw, order, inv, counts, offsets = got
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    assert not bool(out.isnan().any())
+    sel = torch.randperm(T)[:48]
+    r = O.moe_route(logits[sel], k)
+    ref = O.moe_ffn(x[sel], wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
+    err = assert_ffn_close(out.cpu()[sel], ref, dt)
+    assert err.mean().item() < 5e-4

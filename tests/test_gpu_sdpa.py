@@ -1,0 +1,218 @@
+"""GPU parity of scaled-dot-product attention through the C ABI.
+
+Bars: fp32 within 1e-5 relative (max |a-b| / max |b|); bf16 / fp16 within 2e-2
+absolute of the host-engine oracle; the generic kernel additionally reproduces
+the host engine's softmax weights bit for bit (it narrows at the same points).
+"""
+import math
+
+import pytest
+import torch
+
+import capi
+import oracle as O
+from conftest import assert_bit_exact
+from golden_util import DTYPE_TAGS, case
+
+pytestmark = pytest.mark.gpu
+ABS_16BIT = 2e-2
+REL_F32 = 1e-5
+
+
+def run(q, k, v, **kw):
+    kw = {a: (b.cuda() if torch.is_tensor(b) else b) for a, b in kw.items()}
+    return capi.sdpa(q.cuda(), k.cuda(), v.cuda(), **kw)
+
+
+def rel_err(a, b):
+    return ((a.double().cpu() - b.double()).abs().max() / b.double().abs().max()).item()
+
+
+def max_abs(a, b):
+    return (a.double().cpu() - b.double()).abs().max().item()
+
+
+def test_config1_fp32_causal():
+    """BASELINE config 1: B=1 H=8 S=128 D=64 fp32, N(0,1), seed 0, scale 1/sqrt(D)."""
+    q, k, v = torch.randn(1, 8, 128, 64), torch.randn(1, 8, 128, 64), torch.randn(1, 8, 128, 64)
+    out, attn, lse, name = run(q, k, v, is_causal=True, want_attn=True, want_lse=True)
+    want, wattn = O.sdpa_math(q, k, v, is_causal=True, gemm="aten")
+    assert name == "generic" and out.shape == (1, 8, 128, 64)
+    assert rel_err(out, want) <= REL_F32
+    assert torch.allclose(out.cpu(), want, rtol=REL_F32, atol=REL_F32 * want.abs().max().item())
+    assert rel_err(attn, wattn) <= REL_F32
+    ref_lse = torch.logsumexp((q @ k.transpose(-1, -2) * 0.125).masked_fill(~torch.ones(128, 128).tril().bool(), -math.inf), -1)
+    assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("tag", DTYPE_TAGS)
+def test_golden_vectors_generic_kernel(tag):
+    """Small heads (D=16) with every mask variant: outputs and softmax weights of
+    the reference's host engine, bit for bit (fp32: 1e-5 relative, its GEMM is
+    ATen's)."""
+    c = case(f"sdpa_{tag}")
+    q, k, v = c["q"], c["k"], c["v"]
+    dtype = q.dtype
+    scale32 = O.round_to_dtype(1 / math.sqrt(32), dtype)   # the op layer narrows the scale (to_compute)
+    variants = {"plain": {}, "causal": dict(is_causal=True), "bool": dict(mask=c["mask"].bool()),
+                "bias": dict(mask=c["bias"]), "scale": dict(scale=scale32)}
+    for name, kw in variants.items():
+        out, attn, _, kern = run(q, k, v, want_attn=True, **kw)
+        assert kern == "generic"
+        if tag == "f32":
+            assert rel_err(out, c[f"out_{name}"]) <= REL_F32 and rel_err(attn, c[f"attn_{name}"]) <= REL_F32
+        else:
+            assert_bit_exact(attn, c[f"attn_{name}"], f"{tag} {name} weights")
+            one_ulp_of_the_gemm(out, c[f"out_{name}"])
+    out, _, _, _ = run(q, c["kg"], c["vg"])
+    if tag == "f32":
+        assert rel_err(out, c["out_gqa"]) <= REL_F32
+    else:
+        one_ulp_of_the_gemm(out, c["out_gqa"])
+
+
+@pytest.mark.parametrize("tag", ("bf16", "f16"))
+def test_golden_vectors_mfma_kernels(tag):
+    c = case(f"sdpa_d128_{tag}")
+    out, _, _, kern = run(c["q"], c["k"], c["v"], is_causal=True)
+    assert kern == "flash_mfma" and max_abs(out, c["out_causal"]) <= ABS_16BIT
+    out, _, _, kern = run(c["q"], c["k"], c["v"])
+    assert kern == "flash_mfma" and max_abs(out, c["out_plain"]) <= ABS_16BIT
+    d = case(f"sdpa_decode_{tag}")
+    out, _, _, kern = run(d["q"], c["k"], c["v"])
+    assert kern == "decode_split" and max_abs(out, d["out"]) <= ABS_16BIT
+
+
+def one_ulp_of_the_gemm(out, want):
+    """The output is a GEMM of the (bit-identical) weights with V: ATen sums in
+    fp32 in its own order, the kernel in fp64, so a few results land on the
+    other side of a 16-bit rounding boundary.  At most one ulp, at most 1 %."""
+    mant = 7 if want.dtype == torch.bfloat16 else 10
+    a, b = out.double().cpu(), want.double()
+    ulp = 2.0 ** (torch.floor(torch.log2(b.abs().clamp_min(1e-30))) - mant)
+    assert bool(((a - b).abs() <= ulp * 1.001).all())
+    assert float((a != b).double().mean()) <= 0.01
+
+
+FLASH_SHAPES = [  # B, Hq, Hkv, Lq, Lk, D, causal
+    (1, 2, 2, 128, 128, 128, True), (2, 4, 2, 200, 200, 128, True), (1, 2, 1, 130, 77, 64, False),
+    (1, 8, 8, 256, 256, 64, True), (1, 2, 2, 64, 300, 128, True), (1, 4, 4, 300, 64, 128, True),
+    (2, 2, 2, 512, 512, 128, False), (1, 1, 1, 17, 1, 128, False), (3, 5, 5, 129, 191, 64, True),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", FLASH_SHAPES)
+def test_flash_matches_oracle(dtype, shape):
+    B, Hq, Hkv, Lq, Lk, D, causal = shape
+    q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
+    out, _, lse, kern = run(q, k, v, is_causal=causal, want_lse=True)
+    want, _ = O.sdpa_math(q, k, v, is_causal=causal, enable_gqa=True, gemm="aten")
+    assert kern == "flash_mfma"
+    assert max_abs(out, want) <= ABS_16BIT, f"{shape} {dtype}"
+    rep = Hq // Hkv
+    s = (q.float() @ k.float().repeat_interleave(rep, 1).transpose(-1, -2)) / math.sqrt(D)
+    if causal:
+        s = s.masked_fill(~torch.ones(Lq, Lk).tril().bool(), -math.inf)
+    assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=1e-3, atol=1e-3)
+
+
+def test_flash_strided_inputs_and_explicit_scale():
+    """q/k/v as views of a packed [B, L, 3, H, D] projection (no copy)."""
+    B, L, H, D = 2, 160, 4, 128
+    qkv = torch.randn(B, L, 3, H, D).bfloat16()
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    dq = qkv.cuda()
+    dqv, dkv, dvv = (dq[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    out, _, _, kern = capi.sdpa(dqv, dkv, dvv, is_causal=True, scale=0.05)
+    want, _ = O.sdpa_math(q.contiguous(), k.contiguous(), v.contiguous(), is_causal=True, scale=0.05, gemm="aten")
+    assert kern == "flash_mfma" and max_abs(out, want) <= ABS_16BIT
+
+
+DECODE_SHAPES = [(2, 8, 2, 1, 1000), (1, 4, 4, 1, 77), (3, 32, 8, 1, 2048), (1, 8, 2, 2, 300), (2, 16, 1, 1, 129), (1, 2, 2, 8, 5000)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", DECODE_SHAPES)
+def test_decode_matches_oracle(dtype, shape):
+    B, Hq, Hkv, Lq, Lk = shape
+    q, k, v = torch.randn(B, Hq, Lq, 128).to(dtype), torch.randn(B, Hkv, Lk, 128).to(dtype), torch.randn(B, Hkv, Lk, 128).to(dtype)
+    out, _, lse, kern = run(q, k, v, want_lse=True)
+    want, _ = O.sdpa_math(q, k, v, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split"
+    assert max_abs(out, want) <= ABS_16BIT
+    s = (q.float() @ k.float().repeat_interleave(Hq // Hkv, 1).transpose(-1, -2)) / math.sqrt(128)
+    assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=1e-3, atol=1e-3)
+
+
+def test_generic_handles_odd_heads_masks_and_all_masked_rows():
+    q, k, v = torch.randn(1, 3, 5, 24), torch.randn(1, 3, 9, 24), torch.randn(1, 3, 9, 40)
+    out, attn, _, kern = run(q, k, v, want_attn=True)                # Dv != D
+    want, wattn = O.sdpa_math(q, k, v, gemm="aten")
+    assert kern == "generic" and out.shape == (1, 3, 5, 40) and rel_err(out, want) <= REL_F32
+    mask = torch.ones(5, 9, dtype=torch.bool)
+    mask[2] = False                                                    # a row with no visible key
+    out, attn, _, _ = run(q, k, v, mask=mask, want_attn=True)
+    want, wattn = O.sdpa_math(q, k, v, attn_mask=mask, gemm="aten")
+    assert bool(out[:, :, 2].isnan().all()) and bool(want[:, :, 2].isnan().all())   # NaN, as the host softmax gives
+    keep = [0, 1, 3, 4]
+    assert rel_err(out[:, :, keep], want[:, :, keep]) <= REL_F32
+    out, _, _, _ = run(q.double(), k.double(), v.double(), is_causal=True)
+    want, _ = O.sdpa_math(q.double(), k.double(), v.double(), is_causal=True)
+    assert rel_err(out, want) <= 1e-13
+
+
+def test_error_conventions():
+    q = torch.randn(1, 5, 4, 8, device="cuda")
+    k = torch.randn(1, 2, 4, 8, device="cuda")
+    with pytest.raises(capi.ParasError, match="multiple of key/value heads"):   # tests/test_attention_norm_ops.py:103-108
+        capi.sdpa(q, k, k)
+    q = torch.randn(1, 2, 4, 8, device="cuda")
+    with pytest.raises(capi.ParasError, match="mutually exclusive"):
+        capi.sdpa(q, k, k, mask=torch.ones(4, 4, dtype=torch.bool, device="cuda"), is_causal=True)
+    out, _, _, _ = capi.sdpa(q[:, :, :0], k, k)                                   # empty query
+    assert out.shape == (1, 2, 0, 8)
+
+
+def test_config3_shape_properties_and_slice():
+    """BASELINE config 3 (bf16 causal B=4 H=32 S=4096 D=128) at full size: a
+    slice against the oracle, the whole output through properties."""
+    B, H, S, D = 4, 32, 4096, 128
+    q, k, v = torch.randn(B, H, S, D).bfloat16(), torch.randn(B, H, S, D).bfloat16(), torch.randn(B, H, S, D).bfloat16()
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    out, _, lse, kern = capi.sdpa(qd, kd, vd, is_causal=True, want_lse=True)
+    assert kern == "flash_mfma"
+    want, _ = O.sdpa_math(q[:1, :2], k[:1, :2], v[:1, :2], is_causal=True, gemm="aten")
+    assert max_abs(out[:1, :2], want) <= ABS_16BIT
+    # rows 3000..3063 of the last head: causal == an explicit lower-triangular mask on those rows
+    full_rows = O.sdpa_math(q[3:, 31:, 3000:3064], k[3:, 31:], v[3:, 31:],
+                            attn_mask=torch.ones(S, S).tril().bool()[3000:3064], gemm="aten")[0]
+    assert max_abs(out[3:, 31:, 3000:3064], full_rows) <= ABS_16BIT
+    assert not bool(out.isnan().any())
+    assert torch.equal(out[:, :, 0].cpu(), v[:, :, 0])                       # causal row 0 sees key 0 only
+    ones, _, _, _ = capi.sdpa(qd, kd, torch.ones_like(vd), is_causal=True)   # weights sum to one
+    assert (ones.float() - 1).abs().max().item() <= 2 ** -7
+    # linearity in V: f(V1 + V2) == f(V1) + f(V2) up to 16-bit rounding of each term
+    v2 = torch.randn(B, H, S, D).bfloat16().cuda()
+    o2, _, _, _ = capi.sdpa(qd, kd, v2, is_causal=True)
+    o12, _, _, _ = capi.sdpa(qd, kd, (vd.float() + v2.float()).bfloat16(), is_causal=True)
+    assert (o12.float() - (out.float() + o2.float())).abs().max().item() <= 6e-2
+
+
+def test_config4_shape_slice_and_gqa_equivalence():
+    """BASELINE config 4 (bf16 GQA decode B=64 Hq=32 Hkv=8 Lk=8192 D=128)."""
+    B, Hq, Hkv, Lk = 64, 32, 8, 8192
+    q = torch.randn(B, Hq, 1, 128).bfloat16()
+    k, v = torch.randn(B, Hkv, Lk, 128).bfloat16(), torch.randn(B, Hkv, Lk, 128).bfloat16()
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    out, _, _, kern = capi.sdpa(qd, kd, vd)
+    assert kern == "decode_split"
+    want, _ = O.sdpa_math(q[:4], k[:4], v[:4], enable_gqa=True, gemm="aten")
+    assert max_abs(out[:4], want) <= ABS_16BIT
+    want, _ = O.sdpa_math(q[60:], k[60:], v[60:], enable_gqa=True, gemm="aten")
+    assert max_abs(out[60:], want) <= ABS_16BIT
+    # GQA by index mapping == explicit repeat_interleave of K/V (what the reference does)
+    rep, _, _, _ = capi.sdpa(qd[:8], kd[:8].repeat_interleave(4, 1), vd[:8].repeat_interleave(4, 1))
+    assert max_abs(out[:8], rep.cpu()) <= 4e-3
+    ones, _, _, _ = capi.sdpa(qd, kd, torch.ones_like(vd))
+    assert (ones.float() - 1).abs().max().item() <= 2 ** -7
