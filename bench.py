@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused transformer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Prints ONE JSON line.  The headline value is BASELINE.json's first metric:
+bf16 causal flash-attention forward at B=4, H=32, S=4096, D=128 (configs[2]) in
+TFLOP/s, counted with the causal-halved figure 4*B*H*S^2*D/2.  The same line
+carries, under "workloads", the other configurations the metric names
+(RMSNorm and SwiGLU of configs[1] in GB/s, the GQA decode of configs[3], the
+MoE layer of configs[4]), each with its own roofline object.
+
+A step is one pass of the workload's kernels over one batch of synthetic
+inputs (seeded N(0,1) / N(1,0.02) / N(0,0.02) as BASELINE.json states) that
+are resident in HBM before the timed region.  Kernels are called through the C
+ABI of libparas_hip.so on torch's current stream; per-launch durations come
+from HIP events recorded on that same stream.  The HBM-bound kernels rotate
+over enough buffers that no input is served from the 256 MB last-level cache.
+
+cpu_baseline times the reference's own CPU flavor (oracle/_ref, "reference")
+-- or, if that library is absent, the oracle's C restatement ("port") -- on a
+bounded sample of the headline workload in a child process on this box's host
+cores.  It is a reported baseline, not a target.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT / "tests", ROOT / "oracle"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+HBM_PEAK_GBS = 8000.0         # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
+METRIC = "SDPA TFLOP/s (% MFMA peak); RMSNorm/SwiGLU GB/s (% HBM peak) at 1 GPU"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def load_traffic() -> dict:
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE),
+    recorded next to the profile summaries."""
+    path = ROOT / "profiles" / "hbm_traffic.json"
+    if path.exists():
+        return json.loads(path.read_text())
+    return {}
+
+
+class Timer:
+    """HIP events on the launch stream: average launch duration in ms."""
+
+    def __init__(self, torch):
+        self.torch = torch
+
+    def run(self, fn, steps, warmup):
+        torch = self.torch
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            fn(warmup + i)
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        return e0.elapsed_time(e1) / steps, wall_ms
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build targets one GPU; --gpus must be 1 (nothing here shards across GPUs)", file=sys.stderr)
+        return 2
+
+    import torch
+    import capi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    L = capi.lib()                       # raises if libparas_hip.so is missing: no fallback
+    assert L.paras_device_count() >= 1
+    torch.manual_seed(0)
+    dev = "cuda:0"
+    bf = torch.bfloat16
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    timer = Timer(torch)
+    traffic = load_traffic()
+    steps, warmup = args.steps, args.warmup
+    want = lambda name: args.workload in ("all", name)
+    results = {}
+
+    def must(rc):
+        if rc != 0:
+            raise RuntimeError(L.paras_last_error().decode())
+
+    def roofline(bound, achieved, key):
+        peak = HBM_PEAK_GBS if bound == "hbm" else MFMA_BF16_PEAK_TFLOPS
+        return {"bound": bound, "achieved": round(achieved, 2), "peak": peak,
+                "unit": "GB/s" if bound == "hbm" else "TFLOP/s", "frac": round(achieved / peak, 4),
+                "traffic": traffic.get(key)}
+
+    # ------------------------------------------------------------------ configs[2]
+    if want("sdpa_prefill"):
+        B, H, S, D = 4, 32, 4096, 128
+        q, k, v = (torch.randn(B, H, S, D, device=dev).to(bf) for _ in range(3))
+        out = torch.empty_like(q)
+        a = capi.sdpa_args(q, k, v, out, is_causal=True)
+        assert L.paras_sdpa_kernel_name(C.byref(a)) == b"flash_mfma"
+        ms, wall = timer.run(lambda i: must(L.paras_sdpa_fwd(C.byref(a), None, st)), steps, warmup)
+        flops = 4 * B * H * S * S * D / 2          # causal-halved
+        tf = flops / ms / 1e9
+        results["sdpa_prefill"] = {
+            "workload": "bf16 causal flash-attention fwd B=4 H=32 S=4096 D=128 (configs[2])",
+            "value": round(tf, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall, 4),
+            "kernel": "flash_fwd_kernel<bf16,128,causal>", "algorithmic_flops_per_launch": flops,
+            "roofline": roofline("mfma", tf, "flash_fwd_kernel"),
+        }
+        log(f"sdpa_prefill: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s  ({tf / MFMA_BF16_PEAK_TFLOPS:.1%} of dense bf16 peak)")
+        del q, k, v, out
+
+    # ------------------------------------------------------------------ configs[1]
+    if want("rmsnorm_swiglu"):
+        rows, Hd, I = 16384, 4096, 14336
+        nrot = 4                                  # 4 x 268 MB of RMSNorm traffic between reuses of a buffer
+        xs = [torch.randn(rows, Hd, device=dev).to(bf) for _ in range(nrot)]
+        outs = [torch.empty_like(x) for x in xs]
+        w = (1 + 0.02 * torch.randn(Hd, device=dev)).to(bf)
+        rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+
+        def rms(i):
+            j = i % nrot
+            must(L.paras_rms_norm_fwd(xs[j].data_ptr(), w.data_ptr(), outs[j].data_ptr(), rstd.data_ptr(), rows, Hd,
+                                      1e-6, capi.BF16, st))
+        ms_r, _ = timer.run(rms, steps, warmup)
+        bytes_r = 2 * rows * Hd * 2 + Hd * 2 + rows * 4
+        gbs_r = bytes_r / ms_r / 1e6
+        del xs, outs
+        gate = torch.randn(rows, I, device=dev).to(bf)
+        up = torch.randn(rows, I, device=dev).to(bf)
+        so = torch.empty_like(gate)
+        n = rows * I
+        ms_s, _ = timer.run(lambda i: must(L.paras_swiglu_fwd(gate.data_ptr(), up.data_ptr(), so.data_ptr(), n, capi.BF16, st)),
+                            steps, warmup)
+        bytes_s = 3 * n * 2
+        gbs_s = bytes_s / ms_s / 1e6
+        results["rmsnorm_swiglu"] = {
+            "workload": "bf16 fused RMSNorm 16384x4096 (eps 1e-6) then SwiGLU 16384x14336 (configs[1])",
+            "value": round((bytes_r + bytes_s) / (ms_r + ms_s) / 1e6, 1), "unit": "GB/s",
+            "ms_per_step": round(ms_r + ms_s, 4),
+            "rms_norm": {"ms": round(ms_r, 4), "algorithmic_bytes_per_launch": bytes_r, "kernel": "rms_norm_fwd_vec<bf16,2>",
+                         "roofline": roofline("hbm", gbs_r, "rms_norm_fwd_vec")},
+            "swiglu": {"ms": round(ms_s, 4), "algorithmic_bytes_per_launch": bytes_s, "kernel": "swiglu_fwd_vec<bf16>",
+                       "roofline": roofline("hbm", gbs_s, "swiglu_fwd_vec")},
+        }
+        log(f"rms_norm: {ms_r * 1e3:.1f} us  {gbs_r:.0f} GB/s ({gbs_r / HBM_PEAK_GBS:.1%})   "
+            f"swiglu: {ms_s * 1e3:.1f} us  {gbs_s:.0f} GB/s ({gbs_s / HBM_PEAK_GBS:.1%})")
+        del gate, up, so
+
+    # ------------------------------------------------------------------ configs[3]
+    if want("sdpa_decode"):
+        B, Hq, Hkv, Lk, D = 64, 32, 8, 8192, 128
+        q = torch.randn(B, Hq, 1, D, device=dev).to(bf)
+        k, v = torch.randn(B, Hkv, Lk, D, device=dev).to(bf), torch.randn(B, Hkv, Lk, D, device=dev).to(bf)
+        out = torch.empty_like(q)
+        a = capi.sdpa_args(q, k, v, out)
+        assert L.paras_sdpa_kernel_name(C.byref(a)) == b"decode_split"
+        ws = torch.empty(max(1, L.paras_sdpa_workspace(C.byref(a))), dtype=torch.uint8, device=dev)
+        ms, _ = timer.run(lambda i: must(L.paras_sdpa_fwd(C.byref(a), C.c_void_p(ws.data_ptr()), st)), steps, warmup)
+        nbytes = 2 * B * Hkv * Lk * D * 2 + 2 * B * Hq * D * 2
+        gbs = nbytes / ms / 1e6
+        results["sdpa_decode"] = {
+            "workload": "bf16 GQA decode SDPA B=64 Hq=32 Hkv=8 Lq=1 Lk=8192 D=128 (configs[3])",
+            "value": round(gbs, 1), "unit": "GB/s", "ms_per_step": round(ms, 4),
+            "tokens_per_s": round(B / ms * 1e3, 1), "kernel": "decode_split_kernel<bf16> + decode_combine_kernel",
+            "algorithmic_bytes_per_launch": nbytes, "roofline": roofline("hbm", gbs, "decode_split_kernel"),
+        }
+        log(f"sdpa_decode: {ms * 1e3:.1f} us  {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS:.1%})")
+        del q, k, v, out, ws
+
+    # ------------------------------------------------------------------ configs[4]
+    if want("moe"):
+        T, Hd, E, kk, I = 8192, 4096, 8, 2, 14336
+        x = torch.randn(T, Hd, device=dev).to(bf)
+        logits = torch.randn(T, E, device=dev).to(bf)
+        wg = (0.02 * torch.randn(E, I, Hd, device=dev)).to(bf)
+        wu = (0.02 * torch.randn(E, I, Hd, device=dev)).to(bf)
+        wd = (0.02 * torch.randn(E, Hd, I, device=dev)).to(bf)
+        topi = torch.empty(T, kk, dtype=torch.int64, device=dev)
+        topw = torch.empty(T, kk, dtype=torch.float32, device=dev)
+        order = torch.empty(T * kk, dtype=torch.int64, device=dev)
+        inv = torch.empty_like(order)
+        counts = torch.empty(E, dtype=torch.int64, device=dev)
+        offsets = torch.empty(E + 1, dtype=torch.int64, device=dev)
+        rws = torch.empty(max(1, L.paras_moe_route_workspace(T, E, kk)), dtype=torch.uint8, device=dev)
+        fws = torch.empty(L.paras_moe_ffn_workspace(T, kk, Hd, I, capi.BF16), dtype=torch.uint8, device=dev)
+        out = torch.empty(T, Hd, dtype=bf, device=dev)
+
+        def route(i):
+            must(L.paras_moe_route(logits.data_ptr(), T, E, kk, capi.BF16, topi.data_ptr(), topw.data_ptr(), order.data_ptr(),
+                                   inv.data_ptr(), counts.data_ptr(), offsets.data_ptr(), rws.data_ptr(), st))
+
+        def ffn(i):
+            must(L.paras_moe_ffn(x.data_ptr(), wg.data_ptr(), wu.data_ptr(), wd.data_ptr(), topw.data_ptr(), order.data_ptr(),
+                                 inv.data_ptr(), offsets.data_ptr(), out.data_ptr(), fws.data_ptr(), T, E, kk, Hd, I, capi.BF16, st))
+        msteps, mwarm = max(3, steps // 5), max(1, warmup // 5)
+        ms_route, _ = timer.run(route, msteps, mwarm)
+        ms_ffn, _ = timer.run(ffn, msteps, mwarm)
+        ms_all, _ = timer.run(lambda i: (route(i), ffn(i)), msteps, mwarm)
+        flops = T * kk * 3 * 2 * Hd * I
+        tf = flops / ms_ffn / 1e9
+        results["moe"] = {
+            "workload": "bf16 MoE layer T=8192 H=4096 E=8 top-2 I=14336: routing + grouped expert FFN (configs[4])",
+            "value": round(T / ms_all * 1e3, 1), "unit": "tokens/s", "ms_per_step": round(ms_all, 4),
+            "route_ms": round(ms_route, 4), "ffn_ms": round(ms_ffn, 4), "ffn_tflops": round(tf, 2),
+            "kernel": "grouped_gemm_kernel<bf16> (gate-up+SwiGLU, down) + moe_combine_kernel",
+            "algorithmic_flops_per_launch": flops, "roofline": roofline("mfma", tf, "grouped_gemm_kernel"),
+        }
+        log(f"moe: route {ms_route * 1e3:.1f} us, ffn {ms_ffn * 1e3:.1f} us = {tf:.1f} TFLOP/s ({tf / MFMA_BF16_PEAK_TFLOPS:.1%}), "
+            f"layer {ms_all * 1e3:.1f} us = {T / ms_all * 1e3:.0f} tokens/s")
+        del x, wg, wu, wd, fws, out
+
+    # ------------------------------------------------------------------ cpu baseline
+    head_name = "sdpa_prefill" if "sdpa_prefill" in results else next(iter(results))
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(head_name)
+
+    head = results[head_name]
+    line = {
+        "metric": METRIC,
+        "value": head["value"],
+        "unit": head["unit"],
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": head["workload"], "device": torch.cuda.get_device_name(0),
+                   "timing": "HIP events on the launch stream, inputs resident in HBM"},
+        "roofline": head.get("roofline") or head["rms_norm"]["roofline"],
+        "cpu_baseline": cpu,
+        "workloads": results,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def cpu_baseline(name: str):
+    """Times a bounded sample of the workload on the host cores: the reference's
+    own CPU flavor when oracle/_ref is present, else the oracle's restatement."""
+    import ref_engine as R
+    samples = {
+        "sdpa_prefill": ({"B": 1, "H": 16, "S": 4096, "D": 128}, lambda s: 4 * s["B"] * s["H"] * s["S"] ** 2 * s["D"] / 2 / 1e12, "TFLOP/s",
+                         "B=1, H=16 of the 4x32 heads at S=4096, D=128 (1/8 of the workload)"),
+        "rmsnorm_swiglu": ({"rows": 2048, "H": 4096, "I": 14336}, lambda s: (2 * s["rows"] * s["H"] * 2 + 3 * s["rows"] * s["I"] * 2) / 1e9, "GB/s",
+                           "2048 of the 16384 rows (1/8 of the workload)"),
+        "sdpa_decode": ({"B": 2, "Hq": 32, "Hkv": 8, "Lk": 8192, "D": 128}, lambda s: 2 * s["B"] * s["Hkv"] * s["Lk"] * s["D"] * 2 / 1e9, "GB/s",
+                        "B=2 of 64 sequences (1/32 of the workload)"),
+        "moe": ({"T": 128, "H": 4096, "E": 8, "k": 2, "I": 14336}, lambda s: s["T"] / 1.0, "tokens/s",
+                "128 of the 8192 tokens, all 8 experts' weights"),
+    }
+    sample, work, unit, text = samples[name]
+    try:
+        if R.available():
+            res = R.run("time_workload", name, sample)
+            threads = R.run("host_threads")
+            kind = "reference"
+        else:
+            res, threads, kind = port_baseline(name, sample)
+        val = work(sample) / res["seconds"]
+        log(f"cpu_baseline[{kind}] {name}: sample took {res['seconds']:.2f} s on {threads} threads -> {val:.4g} {unit}")
+        return {"value": float(f"{val:.4g}"), "unit": unit, "cores": threads, "kind": kind,
+                "sample": f"{text}; {res['seconds']:.2f} s of CPU work, scaled linearly", "detail": res}
+    except Exception as e:  # the baseline is informative; its failure must not hide the GPU result
+        log(f"cpu_baseline failed: {e}")
+        return {"value": None, "unit": unit, "cores": os.cpu_count(), "kind": "unavailable", "sample": str(e)[:200]}
+
+
+def port_baseline(name, sample):
+    import torch
+    import oracle as O
+    torch.manual_seed(0)
+    bf = torch.bfloat16
+    if name != "sdpa_prefill":
+        raise RuntimeError("oracle/_ref missing and the port baseline covers sdpa_prefill only")
+    B, H, S, D = sample["B"], sample["H"], sample["S"], sample["D"]
+    q, k, v = (torch.randn(B, H, S, D).to(bf) for _ in range(3))
+    t0 = time.perf_counter()
+    O.sdpa_math(q, k, v, is_causal=True, gemm="aten")
+    return {"seconds": time.perf_counter() - t0}, O.get_threads(), "port"
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -67,6 +67,11 @@ template <> struct Elem<bf16_t> {
     __device__ static __forceinline__ float  to_f32(std::uint16_t v) { return bf16_bits_to_f32(v); }
     __device__ static __forceinline__ double to_f64(std::uint16_t v) { return static_cast<double>(bf16_bits_to_f32(v)); }
     __device__ static __forceinline__ std::uint16_t from_f32(float v) { return f32_to_bf16_bits(v); }
+    // Same rounding through v_cvt_pk_bf16_f32, for values known not to be NaN
+    // (the hardware keeps a NaN's payload, the host canonicalises it).
+    __device__ static __forceinline__ std::uint16_t from_f32_finite(float v) {
+        return __builtin_bit_cast(std::uint16_t, static_cast<__bf16>(v));
+    }
     // The host path converts double -> float -> bf16 (c10::BFloat16 has only a
     // float constructor), i.e. two roundings; keep both.
     __device__ static __forceinline__ std::uint16_t from_f64(double v) { return f32_to_bf16_bits(static_cast<float>(v)); }
@@ -77,6 +82,7 @@ template <> struct Elem<f16_t> {
     __device__ static __forceinline__ float  to_f32(std::uint16_t v) { return f16_bits_to_f32(v); }
     __device__ static __forceinline__ double to_f64(std::uint16_t v) { return static_cast<double>(f16_bits_to_f32(v)); }
     __device__ static __forceinline__ std::uint16_t from_f32(float v) { return f32_to_f16_bits(v); }
+    __device__ static __forceinline__ std::uint16_t from_f32_finite(float v) { return f32_to_f16_bits(v); }
     // Two roundings as on the host (double -> float -> half).  The empty asm
     // keeps the compiler from merging them into one double -> half rounding.
     __device__ static __forceinline__ std::uint16_t from_f64(double v) {

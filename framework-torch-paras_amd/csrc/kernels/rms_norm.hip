@@ -1,21 +1,24 @@
 // Fused RMSNorm forward/backward for gfx950.
 //
 // Arithmetic follows the reference's host engine (csrc/ops/fused_ops.cpp:67-85,
-// 105-156): everything is evaluated in fp64 and rounded once to the tensor
-// dtype (double -> float -> T).  fp64 FMA runs at the same per-lane rate as
-// unpacked fp32 on CDNA4 and these kernels are HBM-bound, so the wide math is
-// free; it makes the result agree with the host engine bit for bit except
-// where the summation order changes the last bit of the fp64 sum.
+// 105-156): everything is evaluated in fp64 and narrowed once to the tensor
+// dtype (double -> float -> T).
 //
-// Forward: one 256-thread workgroup per row at a time, grid-stride over rows.
-// Each thread owns NV 16-byte vectors of the row (kept in registers between
-// the sum-of-squares pass and the scaling pass, so x is read from HBM once),
-// the four wave sums meet in LDS.
+// Forward: one 256-thread workgroup per row (grid = rows, so tens of
+// thousands of independent workgroups keep HBM requests in flight).  Each
+// thread owns NV 16-byte vectors of the row, loaded once with non-temporal
+// loads and kept in registers between the sum-of-squares pass and the scaling
+// pass; the four wave sums meet in LDS.  The sum of squares and rstd are fp64
+// (the fp32 rstd output then matches the host bit for bit); the scaled outputs
+// of 16-bit tensors take the fp32 fast tier of kernels/swiglu_math.h and fall
+// back to the fp64 product only next to a rounding boundary, so they too are
+// bit-identical to the host engine's.
 #include <hip/hip_runtime.h>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
+#include "kernels/swiglu_math.h"
 
 namespace paras {
 namespace {
@@ -37,12 +40,27 @@ __device__ __forceinline__ double block_sum(double v, double* slots) {
     return t;
 }
 
+// 1/sqrt(v) in fp64 from the hardware estimate and two Newton steps (error of a
+// few 1e-16 relative: the fp32 rstd and every narrowed output are what the
+// correctly rounded 1.0/sqrt(v) gives, since neither can see the last bit of
+// a double).  Zero, infinite, NaN and subnormal arguments take the plain form.
+__device__ __forceinline__ double rsqrt_f64(double v) {
+    if (!(v > 1e-300 && v < 1e300)) return 1.0 / sqrt(v);
+    double r = __builtin_amdgcn_rsq(v);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const double e = fma(-v * r, r, 1.0);
+        r = fma(0.5 * r, e, r);
+    }
+    return r;
+}
+
 // Register-resident row: H == vectors per row * kVec, vectors per row <= kBlock*NV.
 template <typename T, int NV>
-__global__ __launch_bounds__(kBlock) void rms_norm_fwd_vec(
+__global__ __launch_bounds__(kBlock, 8) void rms_norm_fwd_vec(
     const typename Elem<T>::store_t* __restrict__ x, const typename Elem<T>::store_t* __restrict__ w,
     typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, int H,
-    double eps) {
+    double eps, double inv_h) {
     using E = Elem<T>;
     using S = typename E::store_t;
     constexpr int V = E::kVec;
@@ -53,9 +71,8 @@ __global__ __launch_bounds__(kBlock) void rms_norm_fwd_vec(
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int c = threadIdx.x + i * kBlock;
-        if (c < nvec) wv[i] = load16(w + static_cast<long>(c) * V);
+        if (c < nvec) wv[i] = load16(w + static_cast<long>(c) * V);  // shared by every row: an L2 hit
     }
-
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         const S* xr = x + r * H;
         S* outr = out + r * H;
@@ -79,20 +96,35 @@ __global__ __launch_bounds__(kBlock) void rms_norm_fwd_vec(
             }
         }
         ss = block_sum(ss, slots);
-        const double rs = 1.0 / sqrt(ss / static_cast<double>(H) + eps);
-        if (threadIdx.x == 0) rstd[r] = static_cast<float>(rs);
+        // 16-bit tensors: mean by the reciprocal and the refined rsqrt (outputs
+        // cannot see the difference); fp32 / fp64 tensors: the host's own form.
+        const double rs = sizeof(S) == 2 ? rsqrt_f64(fma(ss, inv_h, eps)) : 1.0 / sqrt(ss / static_cast<double>(H) + eps);
+        const float rs32 = static_cast<float>(rs);
+        if (threadIdx.x == 0) rstd[r] = rs32;
+        if constexpr (sizeof(S) == 2) {
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int c = threadIdx.x + i * kBlock;
-            if (c < nvec) {
-                const S* e  = reinterpret_cast<const S*>(&xv[i]);
-                const S* we = reinterpret_cast<const S*>(&wv[i]);
-                u32x4 o;
-                S* oe = reinterpret_cast<S*>(&o);
+            for (int i = 0; i < NV; ++i) {
+                const int c = threadIdx.x + i * kBlock;
+                if (c < nvec) {
+                    bool fix;
+                    u32x4 o = scale_vec16_fast<T>(xv[i], wv[i], rs32, fix);
+                    if (__builtin_expect(fix, 0)) o = scale_vec16_fix<T>(xv[i], wv[i], o, rs32, rs);
+                    store16_nt(outr + static_cast<long>(c) * V, o);
+                }
+            }
+        } else {
 #pragma unroll
-                for (int j = 0; j < V; ++j)
-                    oe[j] = E::from_f64(E::to_f64(e[j]) * rs * E::to_f64(we[j]));
-                store16_nt(outr + static_cast<long>(c) * V, o);
+            for (int i = 0; i < NV; ++i) {
+                const int c = threadIdx.x + i * kBlock;
+                if (c < nvec) {
+                    const S* e  = reinterpret_cast<const S*>(&xv[i]);
+                    const S* we = reinterpret_cast<const S*>(&wv[i]);
+                    u32x4 o;
+                    S* oe = reinterpret_cast<S*>(&o);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) oe[j] = scale_one<T>(e[j], rs32, rs, we[j]);
+                    store16_nt(outr + static_cast<long>(c) * V, o);
+                }
             }
         }
     }
@@ -186,7 +218,7 @@ int grid_for_rows(long rows) {
     (void)hipGetDevice(&dev);
     auto* st = DeviceContext::instance().device(dev);
     const long cus = st ? st->compute_units : 256;
-    const long cap = cus * 8;  // eight 256-thread workgroups fill a CU
+    const long cap = cus * 256;  // far more workgroups than fit at once: the dispatcher keeps every CU fed
     return static_cast<int>(rows < cap ? rows : cap);
 }
 
@@ -203,11 +235,11 @@ int launch_fwd(const void* x, const void* w, void* out, float* rstd, long rows, 
                                            reinterpret_cast<uintptr_t>(out)) % 16 == 0);
     const long nvec = H / V;
     if (aligned && nvec <= kBlock * 1 && H <= INT32_MAX)
-        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 1>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps);
+        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 1>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps, 1.0 / static_cast<double>(H));
     else if (aligned && nvec <= kBlock * 2)
-        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps);
+        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps, 1.0 / static_cast<double>(H));
     else if (aligned && nvec <= kBlock * 4)
-        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 4>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps);
+        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 4>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps, 1.0 / static_cast<double>(H));
     else
         hipLaunchKernelGGL((rms_norm_fwd_any<T>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, H, eps);
     PARAS_HIP_TRY(hipGetLastError());

@@ -4,7 +4,9 @@
 // kernels/swiglu_math.h for how the fp64 definition is met at fp32 cost).
 //
 // Layout: flat contiguous streams, 16 bytes per lane per access, kUnroll
-// independent accesses in flight per lane, grid-stride.
+// independent non-temporal accesses per stream in flight per lane, one chunk
+// per workgroup (tens of thousands of short workgroups stream better here
+// than a persistent grid-stride loop).
 #include <hip/hip_runtime.h>
 
 #include "core/device_context.h"
@@ -16,7 +18,7 @@ namespace paras {
 namespace {
 
 constexpr int kBlock  = 256;
-constexpr int kUnroll = 2;  // 16-byte vectors per stream per lane per iteration
+constexpr int kUnroll = 4;  // 16-byte vectors per stream per lane per iteration
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void swiglu_fwd_vec(
@@ -124,8 +126,9 @@ int launch_swiglu_fwd(const void* gate, const void* up, void* out, long n, hipSt
     long done = 0;
     if (aligned && n >= V) {
         const long nvec = n / V;
-        hipLaunchKernelGGL((swiglu_fwd_vec<T>), dim3(stream_grid(kBlock * kUnroll, nvec)), dim3(kBlock), 0,
-                           s, g, u, o, nvec);
+        long blocks = (nvec + kBlock * kUnroll - 1) / (kBlock * kUnroll);
+        if (blocks > 0x7fffffffL) blocks = 0x7fffffffL;  // the kernel grid-strides beyond that
+        hipLaunchKernelGGL((swiglu_fwd_vec<T>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, s, g, u, o, nvec);
         PARAS_HIP_TRY(hipGetLastError());
         done = nvec * V;
     }

@@ -1,17 +1,19 @@
-// silu(gate) * up for one element, with the rounding of the reference's host
-// engine: fp64 evaluation, then double -> float -> T
-// (csrc/ops/fused_ops.cpp:185-190).  Shared by the streaming SwiGLU kernel and
-// the MoE expert GEMM epilogue.
+// Element math shared by the streaming kernels: results that equal the
+// reference host engine's "evaluate in fp64, narrow double -> float -> T"
+// (csrc/ops/fused_ops.cpp:72-84,185-190) at fp32 cost.
 //
-// For the 16-bit dtypes the value is computed in two tiers:
-//   fast  fp32 evaluation with a proven relative error bound kFastRelErr; the
-//         result is accepted when both ends of the error interval round to
-//         the same 16-bit value, which means the fp64 result rounds there too;
-//   exact the fp64 formula, taken by the few lanes whose interval straddles a
-//         rounding boundary (about 1 element in 1000) or whose gate lies
-//         outside the range the bound was derived for.
-// The output therefore equals the fp64-then-round definition everywhere, not
-// only within a tolerance.  fp32/fp64 tensors use the fp64 formula directly.
+// Two tiers for the 16-bit dtypes:
+//   fast   the value is computed in fp32 with a proven relative error bound.
+//          If the fp32 result is further from every 16-bit rounding boundary
+//          than that bound, the fp64 result narrows to the same 16-bit value,
+//          so the fp32 result is narrowed and used.
+//   exact  otherwise (about 1 element in 1000) the fp64 formula is evaluated.
+// The output therefore equals the fp64-then-narrow definition everywhere, not
+// only within a tolerance.  fp32 / fp64 tensors use the fp64 formula directly.
+//
+// The distance test works on the bits of the fp32 result: a 16-bit type with
+// M explicit mantissa bits drops the low (23-M) bits; the rounding boundary
+// sits at half of that field.  `ulps` is the error bound in fp32 ulps.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -20,13 +22,37 @@
 
 namespace paras {
 
-// Bound on |fast - exact| / |exact| for gate in [kFastGateMin, kFastGateMax]:
-// the exponent argument g*log2(e) carries at most |g*log2e| * 2^-23 absolute
-// error (product rounding + constant), i.e. <= 8.1e-7 relative on exp for
-// g >= -8 (for g > 0 the term exp(-g) <= 1 is damped by 1/(1+e)); v_exp_f32,
-// the add, v_rcp_f32 and the two multiplies add < 5e-7.  2^-19 = 1.9e-6
-// covers the sum with margin.
-constexpr float kFastRelErr  = 1.9073486328125e-06f;  // 2^-19
+template <typename T> struct Narrow16;
+template <> struct Narrow16<bf16_t> {
+    static constexpr std::uint32_t kMask = 0xFFFFu, kHalf = 0x8000u;
+    // normal range of the result in which the dropped field has fixed width
+    static constexpr float kMinNormal = 1e-30f, kMaxFinite = 3.0e38f;
+};
+template <> struct Narrow16<f16_t> {
+    static constexpr std::uint32_t kMask = 0x1FFFu, kHalf = 0x1000u;
+    static constexpr float kMinNormal = 6.2e-5f /* > 2^-14 */, kMaxFinite = 65000.0f;
+};
+
+// True when narrowing `y` (fp32, relative error <= ulps fp32 ulps) to T is safe.
+template <typename T>
+__device__ __forceinline__ bool narrow_is_safe(float y, std::uint32_t ulps) {
+    const std::uint32_t b = __builtin_bit_cast(std::uint32_t, y);
+    const std::uint32_t f = b & Narrow16<T>::kMask;
+    const bool near = (f - (Narrow16<T>::kHalf - ulps)) <= 2u * ulps;  // unsigned wrap: one compare
+    const float a = fabsf(y);
+    const bool ranged = (a >= Narrow16<T>::kMinNormal) && (a <= Narrow16<T>::kMaxFinite);  // false for NaN
+    return !near && ranged;
+}
+
+// ---- SwiGLU ------------------------------------------------------------------
+// Error of the fp32 evaluation for gate in [kFastGateMin, kFastGateMax]: the
+// exponent argument g*log2(e) carries at most |g*log2e| * 2^-23 absolute error
+// (product rounding + constant), i.e. <= 8.1e-7 relative on exp for g >= -8
+// (for g > 0 the term exp(-g) <= 1 is damped by 1/(1+e)); v_exp_f32, the add,
+// v_rcp_f32 and the two multiplies add < 5e-7.  2^-19 = 1.9e-6 relative covers
+// the sum with margin; that is 16 fp32 ulps at the bottom of a binade and 32
+// at the top, so 32 is used.
+constexpr std::uint32_t kSwigluUlps = 32;
 constexpr float kFastGateMin = -8.0f;
 constexpr float kFastGateMax = 60.0f;
 
@@ -46,23 +72,97 @@ __device__ __forceinline__ typename Elem<T>::store_t swiglu_one(typename Elem<T>
         const float u = E::to_f32(us);
         const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
         const float y = g * __builtin_amdgcn_rcpf(1.0f + e) * u;
-        const auto lo = E::from_f32(y * (1.0f - kFastRelErr));
-        const auto hi = E::from_f32(y * (1.0f + kFastRelErr));
-        // NaN gates fail the range test and take the exact tier.  A result in
-        // fp32's denormal range has no relative bound, so it is only accepted
-        // when it is an exact zero (zero gate or zero up).
-        const bool sized = (fabsf(y) >= 1e-30f) || (g == 0.0f) || (u == 0.0f);
-        const bool ok = (lo == hi) && (g >= kFastGateMin) && (g <= kFastGateMax) && sized;
-        // Return the rounding of y itself: it lies between lo and hi, and unlike
-        // them it keeps the sign of a zero result (the compiler may form lo/hi
-        // with a fused multiply-add-convert whose +0 addend drops it).
-        if (__builtin_expect(ok, 1)) return E::from_f32(y);
+        // |g - 26| <= 34  <=>  -8 <= g <= 60; false for a NaN gate.
+        const bool ok = narrow_is_safe<T>(y, kSwigluUlps) && (fabsf(g - 26.0f) <= 34.0f);
+        if (__builtin_expect(ok, 1)) return E::from_f32_finite(y);
+        // A zero gate or zero up gives an exact signed zero (or NaN against an
+        // infinity) in fp32 as in fp64; keep zero padding off the fp64 path.
+        if (y == 0.0f && (g == 0.0f || u == 0.0f)) return E::from_f32(y);
         return swiglu_exact<T>(g, u);
     } else {
         const double g = E::to_f64(gs);
         const double s = g / (1.0 + exp(-g));
         return E::from_f64(s * E::to_f64(us));
     }
+}
+
+// ---- RMSNorm output ------------------------------------------------------------
+// out = T(x * rstd * w).  fp32: fl(fl(x*fl(rstd))*w) is within 3 * 2^-24
+// relative of the exact product (three roundings), i.e. at most 3 fp32 ulps; 4 is used.
+constexpr std::uint32_t kScaleUlps = 4;
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::store_t scale_one(typename Elem<T>::store_t xs, float rs32, double rs64,
+                                                                 typename Elem<T>::store_t ws) {
+    using E = Elem<T>;
+    if constexpr (sizeof(typename E::store_t) == 2) {
+        const float x = E::to_f32(xs), w = E::to_f32(ws);
+        const float y = x * rs32 * w;
+        if (__builtin_expect(narrow_is_safe<T>(y, kScaleUlps), 1)) return E::from_f32_finite(y);
+        if (y == 0.0f && (x == 0.0f || w == 0.0f)) return E::from_f32(y);  // exact signed zero
+        return E::from_f64(static_cast<double>(x) * rs64 * static_cast<double>(w));
+    } else {
+        return E::from_f64(E::to_f64(xs) * rs64 * E::to_f64(ws));
+    }
+}
+
+
+// Eight 16-bit elements at once (one 16-byte vector of x and of w), fast tier
+// only, straight-line: returns the packed fp32-path results and sets `fix` when
+// any element sits next to a rounding boundary or outside the normal range.
+// The caller passes flagged vectors through scale_vec16_fix before storing.
+template <typename T>
+__device__ __forceinline__ u32x4 scale_vec16_fast(u32x4 xv, u32x4 wv, float rs32, bool& fix) {
+    using E = Elem<T>;
+    static_assert(sizeof(typename E::store_t) == 2, "16-bit dtypes only");
+    // distance of the dropped field from the rounding boundary, biased so that
+    // "within kScaleUlps" reads (field + bias) & mask <= 2*kScaleUlps; the
+    // smallest of the eight decides for the vector
+    constexpr std::uint32_t kBias = kScaleUlps - Narrow16<T>::kHalf;
+    u32x4 o;
+    float amin = 1.0f, amax = 1.0f;
+    std::uint32_t dmin = 0xFFFFu;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const float y0 = E::to_f32(static_cast<std::uint16_t>(xv[p])) * rs32 * E::to_f32(static_cast<std::uint16_t>(wv[p]));
+        const float y1 = E::to_f32(static_cast<std::uint16_t>(xv[p] >> 16)) * rs32 * E::to_f32(static_cast<std::uint16_t>(wv[p] >> 16));
+        const std::uint32_t d0 = (__builtin_bit_cast(std::uint32_t, y0) + kBias) & Narrow16<T>::kMask;
+        const std::uint32_t d1 = (__builtin_bit_cast(std::uint32_t, y1) + kBias) & Narrow16<T>::kMask;
+        dmin = min(dmin, min(d0, d1));
+        amin = fminf(amin, fminf(fabsf(y0), fabsf(y1)));
+        amax = fmaxf(amax, fmaxf(fabsf(y0), fabsf(y1)));
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        if constexpr (sizeof(T) == sizeof(bf16_t) && __is_same(T, bf16_t)) {
+            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+            o[p] = __builtin_bit_cast(std::uint32_t, __builtin_convertvector((f32x2){y0, y1}, bf16x2));
+        } else {
+            typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+            o[p] = __builtin_bit_cast(std::uint32_t, __builtin_convertvector((f32x2){y0, y1}, f16x2));
+        }
+    }
+    fix = (dmin <= 2 * kScaleUlps) || !(amin >= Narrow16<T>::kMinNormal && amax <= Narrow16<T>::kMaxFinite);
+    return o;
+}
+
+// Replaces the elements of one result vector whose fp32 value was not safe to
+// narrow with the exact fp64 product.  Rare (about one vector in a thousand
+// per lane), so it is written as a rolled loop over the 8 elements: one exact
+// product is live at a time and the hot loop keeps its registers.
+template <typename T>
+__device__ __forceinline__ u32x4 scale_vec16_fix(u32x4 xv, u32x4 wv, u32x4 o, float rs32, double rs64) {
+    using E = Elem<T>;
+#pragma unroll 1
+    for (int j = 0; j < 8; ++j) {
+        const int p = j >> 1, sh = (j & 1) * 16;
+        const std::uint16_t xs = static_cast<std::uint16_t>(xv[p] >> sh), ws = static_cast<std::uint16_t>(wv[p] >> sh);
+        const float x = E::to_f32(xs), w = E::to_f32(ws);
+        const float y = x * rs32 * w;
+        if (narrow_is_safe<T>(y, kScaleUlps)) continue;
+        const bool zero = (y == 0.0f) && (x == 0.0f || w == 0.0f);  // an exact signed zero needs no fp64
+        const std::uint32_t r = zero ? E::from_f32(y) : E::from_f64(static_cast<double>(x) * rs64 * static_cast<double>(w));
+        o[p] = (o[p] & ~(0xFFFFu << sh)) | (r << sh);
+    }
+    return o;
 }
 
 }  // namespace paras

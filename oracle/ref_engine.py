@@ -153,6 +153,59 @@ def moe_ffn(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, k):
     return (yt * wt).sum(1).cpu()
 
 
+# --- timed samples for bench.py's cpu_baseline leg (run in a child process) --------
+def time_workload(name: str, sample: dict) -> dict:
+    """Builds seeded inputs of the sampled shape, runs the workload once on the
+    reference engine (after one small warm-up call), returns wall seconds."""
+    import time
+    torch.manual_seed(0)
+    bf = torch.bfloat16
+    if name == "sdpa_prefill":
+        B, H, S, D = sample["B"], sample["H"], sample["S"], sample["D"]
+        q, k, v = (torch.randn(B, H, S, D).to(bf) for _ in range(3))
+        sdpa_math(q[:, :1, :64], k[:, :1, :64], v[:, :1, :64], is_causal=True)
+        dq, dk, dv = _dev(q), _dev(k), _dev(v)
+        t0 = time.perf_counter()
+        out = torch.ops.aten._scaled_dot_product_attention_math(dq, dk, dv, None, 0.0, True, None, scale=None, enable_gqa=False)[0]
+        out.cpu()
+        return {"seconds": time.perf_counter() - t0}
+    if name == "rmsnorm_swiglu":
+        rows, H, I = sample["rows"], sample["H"], sample["I"]
+        x, w = torch.randn(rows, H).to(bf), (1 + 0.02 * torch.randn(H)).to(bf)
+        gate, up = torch.randn(rows, I).to(bf), torch.randn(rows, I).to(bf)
+        rms_norm(x[:4], w, 1e-6)
+        dx, dw, dg, du = _dev(x), _dev(w), _dev(gate), _dev(up)
+        t0 = time.perf_counter()
+        torch.ops.paras.rms_norm(dx, dw, 1e-6)
+        t1 = time.perf_counter()
+        torch.ops.paras.swiglu(dg, du)
+        t2 = time.perf_counter()
+        return {"seconds": t2 - t0, "rms_norm_seconds": t1 - t0, "swiglu_seconds": t2 - t1}
+    if name == "sdpa_decode":
+        B, Hq, Hkv, Lk, D = sample["B"], sample["Hq"], sample["Hkv"], sample["Lk"], sample["D"]
+        q, k, v = torch.randn(B, Hq, 1, D).to(bf), torch.randn(B, Hkv, Lk, D).to(bf), torch.randn(B, Hkv, Lk, D).to(bf)
+        dq, dk, dv = _dev(q), _dev(k), _dev(v)
+        t0 = time.perf_counter()
+        torch.ops.aten._scaled_dot_product_attention_math(dq, dk, dv, None, 0.0, False, None, scale=None, enable_gqa=True)[0].cpu()
+        return {"seconds": time.perf_counter() - t0}
+    if name == "moe":
+        T, H, E, k, I = sample["T"], sample["H"], sample["E"], sample["k"], sample["I"]
+        x, logits = torch.randn(T, H).to(bf), torch.randn(T, E).to(bf)
+        wg, wu = (0.02 * torch.randn(E, I, H)).to(bf), (0.02 * torch.randn(E, I, H)).to(bf)
+        wd = (0.02 * torch.randn(E, H, I)).to(bf)
+        t0 = time.perf_counter()
+        topi, topw, order, inv, counts, offsets = moe_route(logits, k)
+        moe_ffn(x, wg, wu, wd, topw, order, inv, offsets, k)
+        return {"seconds": time.perf_counter() - t0}
+    raise ValueError(name)
+
+
+def host_threads() -> int:
+    """Threads the reference's host pool uses (csrc/compat/paras_compat.cpp:70-82)."""
+    env = os.environ.get("PTSYCL_CPU_THREADS")
+    return int(env) if env and int(env) > 0 else torch.get_num_threads()
+
+
 # --- child-process evaluation ----------------------------------------------------
 def run(fn_name: str, *args, threads: int | None = None, **kwargs):
     """Evaluates ``ref_engine.<fn_name>(*args, **kwargs)`` in a child process and
