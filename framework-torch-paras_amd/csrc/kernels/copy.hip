@@ -1,0 +1,289 @@
+// Tensor plumbing kernels for the `paras` device: strided copy with optional
+// float-type conversion, strided fill, and the two "composed" ops whose
+// reference implementations narrow to the tensor dtype after every step.
+// None of these is a performance target; they keep whole expressions on the
+// device so that the hot-path kernels are not surrounded by host bounces.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+
+namespace paras {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMaxDims = 8;  // the reference's StridedSpec limit (csrc/core/kernels.h:31)
+
+struct Strided {
+    int  ndim;
+    long sizes[kMaxDims];
+    long src_strides[kMaxDims];
+    long dst_strides[kMaxDims];
+};
+
+__device__ __forceinline__ void offsets(const Strided& s, long flat, long* so, long* d_o) {
+    long a = 0, b = 0;
+    for (int d = s.ndim - 1; d >= 0; --d) {
+        const long c = flat % s.sizes[d];
+        flat /= s.sizes[d];
+        a += c * s.src_strides[d];
+        b += c * s.dst_strides[d];
+    }
+    *so = a;
+    *d_o = b;
+}
+
+template <typename W>
+__global__ __launch_bounds__(kBlock) void copy_same_kernel(const W* __restrict__ src, W* __restrict__ dst, long n,
+                                                           const Strided s) {
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * kBlock) {
+        long a, b;
+        offsets(s, i, &a, &b);
+        dst[b] = src[a];
+    }
+}
+
+// Conversion between the four float storage types goes through double, which
+// holds every source value exactly, then narrows as the host does.
+template <typename TS, typename TD>
+__global__ __launch_bounds__(kBlock) void copy_convert_kernel(const typename Elem<TS>::store_t* __restrict__ src,
+                                                              typename Elem<TD>::store_t* __restrict__ dst, long n,
+                                                              const Strided s) {
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * kBlock) {
+        long a, b;
+        offsets(s, i, &a, &b);
+        if constexpr (sizeof(typename Elem<TS>::store_t) == 8)
+            dst[b] = Elem<TD>::from_f64(Elem<TS>::to_f64(src[a]));
+        else
+            dst[b] = Elem<TD>::from_f32(Elem<TS>::to_f32(src[a]));   // float -> T: one narrowing, as static_cast<T>(float)
+    }
+}
+
+template <typename W>
+__global__ __launch_bounds__(kBlock) void fill_kernel(W* __restrict__ dst, long n, const Strided s, W value) {
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * kBlock) {
+        long a, b;
+        offsets(s, i, &a, &b);
+        dst[b] = value;
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ double narrow(double v) { return Elem<T>::to_f64(Elem<T>::from_f64(v)); }
+
+// aten::rms_norm as the reference composes it (csrc/ops/rms_swiglu_ops.cpp:66-73):
+// pow(2) -> mean(keepdim) [sum, then * 1/n] -> + eps -> rsqrt -> x * inv -> * w,
+// each step narrowed to T.  One workgroup per row.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rms_norm_composed_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                                   const typename Elem<T>::store_t* __restrict__ w,
+                                                                   typename Elem<T>::store_t* __restrict__ out, long rows,
+                                                                   long H, double eps_narrowed) {
+    using E = Elem<T>;
+    __shared__ double slots[kBlock / kWave];
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        const auto* xr = x + r * H;
+        double acc = 0.0;
+        for (long j = threadIdx.x; j < H; j += kBlock) {
+            const double v = E::to_f64(xr[j]);
+            acc += narrow<T>(v * v);
+        }
+        acc = wave_sum(acc);
+        __syncthreads();
+        if ((threadIdx.x & (kWave - 1)) == 0) slots[threadIdx.x / kWave] = acc;
+        __syncthreads();
+        double sum = 0.0;
+        for (int i = 0; i < kBlock / kWave; ++i) sum += slots[i];
+        const double s = narrow<T>(sum);
+        const double m = narrow<T>(s * (H > 0 ? 1.0 / static_cast<double>(H) : 0.0));
+        const double a = narrow<T>(m + 1.0 * eps_narrowed);
+        const double inv = narrow<T>(1.0 / sqrt(a));
+        for (long j = threadIdx.x; j < H; j += kBlock) {
+            double y = narrow<T>(E::to_f64(xr[j]) * inv);
+            if (w != nullptr) y = narrow<T>(y * E::to_f64(w[j]));
+            out[r * H + j] = E::from_f64(y);
+        }
+    }
+}
+
+// torch_paras::swiglu(x, gate) = x * silu(gate), silu narrowed first
+// (csrc/ops/rms_swiglu_ops.cpp:83-86, csrc/ops/pointwise_ops.cpp:460-464).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_composed_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                                 const typename Elem<T>::store_t* __restrict__ gate,
+                                                                 typename Elem<T>::store_t* __restrict__ out, long n) {
+    using E = Elem<T>;
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * kBlock) {
+        const double g = E::to_f64(gate[i]);
+        const double s = narrow<T>(g / (1.0 + exp(-g)));
+        out[i] = E::from_f64(E::to_f64(x[i]) * s);
+    }
+}
+
+unsigned grid_for(long n) {
+    long g = (n + kBlock - 1) / kBlock;
+    if (g > 65536) g = 65536;
+    return static_cast<unsigned>(g < 1 ? 1 : g);
+}
+
+int make_spec(int ndim, const int64_t* sizes, const int64_t* ss, const int64_t* ds, Strided* s, long* n) {
+    PARAS_REQUIRE(ndim >= 0 && ndim <= kMaxDims, "paras: tensor rank %d exceeds kernel limit of %d", ndim, kMaxDims);
+    s->ndim = ndim;
+    long total = 1;
+    for (int d = 0; d < ndim; ++d) {
+        PARAS_REQUIRE(sizes[d] >= 0, "paras: negative size");
+        s->sizes[d] = sizes[d];
+        s->src_strides[d] = ss ? ss[d] : 0;
+        s->dst_strides[d] = ds ? ds[d] : 0;
+        total *= sizes[d];
+    }
+    *n = total;
+    return PARAS_OK;
+}
+
+template <typename TS>
+int convert_from(const void* src, void* dst, long n, const Strided& s, int dst_dtype, hipStream_t st) {
+    using SS = typename Elem<TS>::store_t;
+    const auto* sp = static_cast<const SS*>(src);
+    const dim3 g(grid_for(n)), b(kBlock);
+    switch (dst_dtype) {
+        case PARAS_F32:  hipLaunchKernelGGL((copy_convert_kernel<TS, float>), g, b, 0, st, sp, static_cast<float*>(dst), n, s); break;
+        case PARAS_F64:  hipLaunchKernelGGL((copy_convert_kernel<TS, double>), g, b, 0, st, sp, static_cast<double*>(dst), n, s); break;
+        case PARAS_BF16: hipLaunchKernelGGL((copy_convert_kernel<TS, bf16_t>), g, b, 0, st, sp, static_cast<uint16_t*>(dst), n, s); break;
+        case PARAS_F16:  hipLaunchKernelGGL((copy_convert_kernel<TS, f16_t>), g, b, 0, st, sp, static_cast<uint16_t*>(dst), n, s); break;
+        default: return fail(PARAS_ERR_INVALID, "paras_copy_strided: unknown dtype %d", dst_dtype);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // namespace
+}  // namespace paras
+
+extern "C" {
+
+int paras_copy_strided(const void* src, void* dst, int ndim, const int64_t* sizes, const int64_t* src_strides,
+                       const int64_t* dst_strides, int elem_size, int src_dtype, int dst_dtype, void* stream) {
+    using namespace paras;
+    Strided s;
+    long n = 0;
+    int rc = make_spec(ndim, sizes, src_strides, dst_strides, &s, &n);
+    if (rc != PARAS_OK) return rc;
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(src && dst, "paras_copy_strided: null pointer");
+    hipStream_t st = nullptr;
+    rc = resolve_stream(stream, &st);
+    if (rc != PARAS_OK) return rc;
+    const dim3 g(grid_for(n)), b(kBlock);
+    if (src_dtype == dst_dtype) {
+        switch (elem_size) {
+            case 1: hipLaunchKernelGGL((copy_same_kernel<uint8_t>), g, b, 0, st, static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), n, s); break;
+            case 2: hipLaunchKernelGGL((copy_same_kernel<uint16_t>), g, b, 0, st, static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), n, s); break;
+            case 4: hipLaunchKernelGGL((copy_same_kernel<uint32_t>), g, b, 0, st, static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), n, s); break;
+            case 8: hipLaunchKernelGGL((copy_same_kernel<uint64_t>), g, b, 0, st, static_cast<const uint64_t*>(src), static_cast<uint64_t*>(dst), n, s); break;
+            default: return fail(PARAS_ERR_UNSUPPORTED, "paras_copy_strided: element size %d", elem_size);
+        }
+        PARAS_HIP_TRY(hipGetLastError());
+        return PARAS_OK;
+    }
+    switch (src_dtype) {
+        case PARAS_F32:  return convert_from<float>(src, dst, n, s, dst_dtype, st);
+        case PARAS_F64:  return convert_from<double>(src, dst, n, s, dst_dtype, st);
+        case PARAS_BF16: return convert_from<bf16_t>(src, dst, n, s, dst_dtype, st);
+        case PARAS_F16:  return convert_from<f16_t>(src, dst, n, s, dst_dtype, st);
+        default: return fail(PARAS_ERR_UNSUPPORTED, "paras_copy_strided: conversion from dtype %d", src_dtype);
+    }
+}
+
+int paras_fill_strided(void* dst, int ndim, const int64_t* sizes, const int64_t* strides, int elem_size,
+                       uint64_t value_bits, void* stream) {
+    using namespace paras;
+    Strided s;
+    long n = 0;
+    int rc = make_spec(ndim, sizes, nullptr, strides, &s, &n);
+    if (rc != PARAS_OK) return rc;
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(dst != nullptr, "paras_fill_strided: null pointer");
+    hipStream_t st = nullptr;
+    rc = resolve_stream(stream, &st);
+    if (rc != PARAS_OK) return rc;
+    const dim3 g(grid_for(n)), b(kBlock);
+    switch (elem_size) {
+        case 1: hipLaunchKernelGGL((fill_kernel<uint8_t>), g, b, 0, st, static_cast<uint8_t*>(dst), n, s, static_cast<uint8_t>(value_bits)); break;
+        case 2: hipLaunchKernelGGL((fill_kernel<uint16_t>), g, b, 0, st, static_cast<uint16_t*>(dst), n, s, static_cast<uint16_t>(value_bits)); break;
+        case 4: hipLaunchKernelGGL((fill_kernel<uint32_t>), g, b, 0, st, static_cast<uint32_t*>(dst), n, s, static_cast<uint32_t>(value_bits)); break;
+        case 8: hipLaunchKernelGGL((fill_kernel<uint64_t>), g, b, 0, st, static_cast<uint64_t*>(dst), n, s, value_bits); break;
+        default: return fail(PARAS_ERR_UNSUPPORTED, "paras_fill_strided: element size %d", elem_size);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+int paras_rms_norm_composed_fwd(const void* x, const void* w, void* out, int64_t rows, int64_t H, double eps,
+                                int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(rows >= 0 && H >= 0, "paras_rms_norm_composed_fwd: negative shape");
+    if (rows == 0 || H == 0) return PARAS_OK;
+    PARAS_REQUIRE(x && out, "paras_rms_norm_composed_fwd: null pointer");
+    hipStream_t st = nullptr;
+    int rc = resolve_stream(stream, &st);
+    if (rc != PARAS_OK) return rc;
+    const dim3 g(static_cast<unsigned>(rows < 65536 ? rows : 65536)), b(kBlock);
+    switch (dtype) {
+        case PARAS_F32:
+            hipLaunchKernelGGL((rms_norm_composed_kernel<float>), g, b, 0, st, static_cast<const float*>(x), static_cast<const float*>(w),
+                               static_cast<float*>(out), (long)rows, (long)H, static_cast<double>(static_cast<float>(eps)));
+            break;
+        case PARAS_F64:
+            hipLaunchKernelGGL((rms_norm_composed_kernel<double>), g, b, 0, st, static_cast<const double*>(x), static_cast<const double*>(w),
+                               static_cast<double*>(out), (long)rows, (long)H, eps);
+            break;
+        case PARAS_BF16: {
+            // eps narrowed to bf16 on the host exactly as c10::BFloat16(float(eps)) would
+            const float ef = static_cast<float>(eps);
+            uint32_t u;
+            __builtin_memcpy(&u, &ef, 4);
+            u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+            float en;
+            __builtin_memcpy(&en, &u, 4);
+            hipLaunchKernelGGL((rms_norm_composed_kernel<bf16_t>), g, b, 0, st, static_cast<const uint16_t*>(x),
+                               static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), (long)rows, (long)H,
+                               static_cast<double>(en));
+            break;
+        }
+        case PARAS_F16: {
+            const double en = static_cast<double>(static_cast<float>(static_cast<_Float16>(static_cast<float>(eps))));
+            hipLaunchKernelGGL((rms_norm_composed_kernel<f16_t>), g, b, 0, st, static_cast<const uint16_t*>(x),
+                               static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), (long)rows, (long)H, en);
+            break;
+        }
+        default: return fail(PARAS_ERR_INVALID, "paras_rms_norm_composed_fwd: unknown dtype %d", dtype);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+int paras_swiglu_composed_fwd(const void* x, const void* gate, void* out, int64_t n, int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(n >= 0, "paras_swiglu_composed_fwd: negative size");
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(x && gate && out, "paras_swiglu_composed_fwd: null pointer");
+    hipStream_t st = nullptr;
+    int rc = resolve_stream(stream, &st);
+    if (rc != PARAS_OK) return rc;
+    const dim3 g(grid_for(n)), b(kBlock);
+    switch (dtype) {
+        case PARAS_F32:  hipLaunchKernelGGL((swiglu_composed_kernel<float>), g, b, 0, st, static_cast<const float*>(x), static_cast<const float*>(gate), static_cast<float*>(out), (long)n); break;
+        case PARAS_F64:  hipLaunchKernelGGL((swiglu_composed_kernel<double>), g, b, 0, st, static_cast<const double*>(x), static_cast<const double*>(gate), static_cast<double*>(out), (long)n); break;
+        case PARAS_BF16: hipLaunchKernelGGL((swiglu_composed_kernel<bf16_t>), g, b, 0, st, static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(out), (long)n); break;
+        case PARAS_F16:  hipLaunchKernelGGL((swiglu_composed_kernel<f16_t>), g, b, 0, st, static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(out), (long)n); break;
+        default: return fail(PARAS_ERR_INVALID, "paras_swiglu_composed_fwd: unknown dtype %d", dtype);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // extern "C"

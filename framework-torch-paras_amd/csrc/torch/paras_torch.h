@@ -1,0 +1,63 @@
+// Shared definitions of the PyTorch side of the `paras` device.
+//
+// This translation-unit group (compiled by g++, no HIP headers) owns the
+// dispatcher registrations and tensor bookkeeping; everything that touches
+// the GPU goes through the C ABI of libparas_hip.so (include/paras_hip.h).
+#pragma once
+
+#include <ATen/ATen.h>
+#include <c10/core/Device.h>
+#include <c10/util/Exception.h>
+#include <torch/library.h>
+
+#include "paras_hip.h"
+
+namespace paras_torch {
+
+constexpr c10::DeviceType kParas = c10::DeviceType::PrivateUse1;
+
+// Converts a C-ABI status into the reference's error convention: a c10::Error
+// (RuntimeError in Python) carrying the library's message.
+inline void check(int rc) {
+    TORCH_CHECK(rc == PARAS_OK, paras_last_error());
+}
+
+inline bool is_paras(const at::Tensor& t) { return t.device().type() == kParas; }
+
+// paras_dtype code of a floating tensor type, or -1.
+inline int float_code(c10::ScalarType t) {
+    switch (t) {
+        case c10::kFloat:    return PARAS_F32;
+        case c10::kHalf:     return PARAS_F16;
+        case c10::kBFloat16: return PARAS_BF16;
+        case c10::kDouble:   return PARAS_F64;
+        default:             return -1;
+    }
+}
+
+inline int require_float_code(const at::Tensor& t, const char* op) {
+    const int c = float_code(t.scalar_type());
+    TORCH_CHECK(c >= 0, op, ": unsupported dtype ", t.scalar_type());
+    return c;
+}
+
+// Makes `index` the calling thread's HIP device and returns the context
+// stream every `paras` op of that device is queued on.
+void* stream_for(c10::DeviceIndex index);
+inline void* stream_for(const at::Tensor& t) { return stream_for(t.device().index()); }
+
+// Thread-local current device index (the device guard's state).
+c10::DeviceIndex current_device();
+
+// Fresh tensor on the `paras` device.
+at::Tensor empty_paras(c10::IntArrayRef sizes, c10::ScalarType dtype, c10::Device device);
+
+// Device scratch memory for one op call (returned to the pool when it dies).
+at::Tensor workspace(size_t nbytes, c10::Device device);
+
+// Value of a double after one trip through `dtype` (double -> float -> T), the
+// narrowing the reference applies to a wrapped scalar (to_compute,
+// csrc/ops/pointwise_ops.cpp:55-60).
+double narrow_scalar(double v, c10::ScalarType dtype);
+
+}  // namespace paras_torch

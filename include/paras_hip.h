@@ -112,6 +112,19 @@ PARAS_API size_t paras_round_size(size_t nbytes);
 PARAS_API int paras_memcpy(int device, void* dst, const void* src, size_t nbytes, int kind);
 PARAS_API int paras_memset(int device, void* dst, int value, size_t nbytes);
 
+/* Strided copy of an n-dimensional view (ndim <= 8), element strides, on the
+ * given stream (replaces device_to_device_copy, csrc/ops/tensor_ops.cpp:
+ * 211-250).  src_dtype == dst_dtype copies elem_size-byte elements of any
+ * type; otherwise both must be paras_dtype float types and the copy narrows /
+ * widens as static_cast does on the host. */
+PARAS_API int paras_copy_strided(const void* src, void* dst, int ndim, const int64_t* sizes,
+                                 const int64_t* src_strides, const int64_t* dst_strides,
+                                 int elem_size, int src_dtype, int dst_dtype, void* stream);
+/* Strided fill with one elem_size-byte value given as its bit pattern
+ * (replaces fill_, csrc/ops/tensor_ops.cpp:333-370). */
+PARAS_API int paras_fill_strided(void* dst, int ndim, const int64_t* sizes, const int64_t* strides,
+                                 int elem_size, uint64_t value_bits, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Fused RMSNorm (replaces ptsycl::rms_norm, csrc/ops/fused_ops.cpp:43-88)    */
 /*   ss = sum_j x[r][j]^2 ; rstd[r] = 1/sqrt(ss/H + eps)                      */
@@ -146,6 +159,17 @@ PARAS_API int paras_swiglu_fwd(const void* gate, const void* up, void* out, int6
 PARAS_API int paras_swiglu_bwd(const void* grad_out, const void* gate, const void* up,
                                void* grad_gate, void* grad_up, int64_t n, int dtype,
                                void* stream);
+
+/* The composed forms, which narrow to the tensor dtype after every step:
+ * aten::rms_norm over the trailing H elements of each row, w may be NULL
+ * (replaces ptsycl::rms_norm, csrc/ops/rms_swiglu_ops.cpp:43-75:
+ * pow(2) -> mean -> + eps -> rsqrt -> x * inv -> * w), and
+ * torch_paras::swiglu(x, gate) = x * T(silu(gate))
+ * (csrc/ops/rms_swiglu_ops.cpp:83-86). */
+PARAS_API int paras_rms_norm_composed_fwd(const void* x, const void* w, void* out, int64_t rows,
+                                          int64_t H, double eps, int dtype, void* stream);
+PARAS_API int paras_swiglu_composed_fwd(const void* x, const void* gate, void* out, int64_t n,
+                                        int dtype, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* rotate_half (replaces ptsycl::rotate_half(+_backward),                     */

@@ -45,6 +45,10 @@ SIGNATURES = {
     "paras_round_size": (sz, [sz]),
     "paras_memcpy": (i32, [i32, vp, vp, sz, i32]),
     "paras_memset": (i32, [i32, vp, i32, sz]),
+    "paras_copy_strided": (i32, [vp, vp, i32, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64), i32, i32, i32, vp]),
+    "paras_fill_strided": (i32, [vp, i32, C.POINTER(i64), C.POINTER(i64), i32, C.c_uint64, vp]),
+    "paras_rms_norm_composed_fwd": (i32, [vp, vp, vp, i64, i64, f64, i32, vp]),
+    "paras_swiglu_composed_fwd": (i32, [vp, vp, vp, i64, i32, vp]),
     "paras_rms_norm_fwd": (i32, [vp, vp, vp, vp, i64, i64, f64, i32, vp]),
     "paras_rms_norm_bwd_workspace": (sz, [i64, i64]),
     "paras_rms_norm_bwd": (i32, [vp, vp, vp, vp, vp, vp, vp, i64, i64, i32, vp]),

@@ -1,0 +1,303 @@
+"""The drop-in surface: `import torch_paras`, the `paras` device, the aten /
+paras:: / torch_paras:: ops, driven the way the reference's own tests drive
+them (tests/test_attention_norm_ops.py, tests/test_fused_ops.py, copy tests of
+tests/test_attention_norm_ops.py:172-216) -- device result against torch-CPU at
+the reference's tolerance, plus the oracle for the 16-bit dtypes."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle as O
+from conftest import assert_bit_exact
+
+pytestmark = pytest.mark.gpu
+ATOL = RTOL = 1e-4  # reference tests/common.py:7-8
+
+
+@pytest.fixture(scope="module")
+def device():
+    import torch_paras
+    assert torch_paras.is_available() and torch_paras.backend_name() == "paras-hip"
+    return "paras:0"
+
+
+def assert_close(actual, expected, msg=""):
+    actual, expected = actual.cpu(), expected.cpu()
+    assert actual.dtype == expected.dtype, f"{msg}: dtype {actual.dtype} vs {expected.dtype}"
+    assert actual.shape == expected.shape, f"{msg}: shape {tuple(actual.shape)} vs {tuple(expected.shape)}"
+    if actual.dtype.is_floating_point:
+        assert torch.allclose(actual, expected, atol=ATOL, rtol=RTOL, equal_nan=True), msg
+    else:
+        assert torch.equal(actual, expected), msg
+
+
+def _qkv(device, B=2, H=4, Lq=8, Lk=8, E=16, dtype=torch.float32):
+    q, k, v = torch.randn(B, H, Lq, E, dtype=dtype), torch.randn(B, H, Lk, E, dtype=dtype), torch.randn(B, H, Lk, E, dtype=dtype)
+    return q, k, v, q.to(device), k.to(device), v.to(device)
+
+
+# ---- module surface -----------------------------------------------------------
+def test_module_surface(device):
+    import torch_paras
+    assert torch_paras.device_count() >= 1 and torch.paras.is_available()
+    assert isinstance(torch_paras.device_name(0), str) and torch_paras.is_gpu_device(0)
+    assert torch_paras.get_amp_supported_dtype() == [torch.float16, torch.float32]
+    assert torch.paras._is_in_bad_fork() is False
+    x = torch.randn(1000, 1000).to(device)
+    assert x.is_paras and x.device == torch.device("paras", 0)
+    assert torch_paras.memory_allocated(0) >= 4_000_000
+    del x
+    torch_paras.synchronize()
+    torch_paras.empty_cache()
+    assert torch_paras.memory_cached(0) == 0
+    torch_paras.manual_seed(0)
+    with pytest.raises(RuntimeError):
+        torch.randn(2).to("paras:7")
+
+
+# ---- scaled dot-product attention (reference tests/test_attention_norm_ops.py:35-108)
+def test_sdpa_basic(device):
+    q, k, v, dq, dk, dv = _qkv(device)
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv), F.scaled_dot_product_attention(q, k, v), "sdpa_basic")
+
+
+def test_sdpa_explicit_scale(device):
+    q, k, v, dq, dk, dv = _qkv(device, E=16)
+    s = 1.0 / math.sqrt(32)
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, scale=s), F.scaled_dot_product_attention(q, k, v, scale=s), "scale")
+
+
+def test_sdpa_causal(device):
+    q, k, v, dq, dk, dv = _qkv(device)
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, is_causal=True),
+                 F.scaled_dot_product_attention(q, k, v, is_causal=True), "causal")
+
+
+def test_sdpa_causal_unequal_lengths(device):
+    q, k, v, dq, dk, dv = _qkv(device, Lq=4, Lk=8)
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, is_causal=True),
+                 F.scaled_dot_product_attention(q, k, v, is_causal=True), "causal Lq != Lk")
+
+
+def test_sdpa_bool_mask(device):
+    q, k, v, dq, dk, dv = _qkv(device)
+    mask = torch.rand(2, 4, 8, 8) > 0.3
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, attn_mask=mask.to(device)),
+                 F.scaled_dot_product_attention(q, k, v, attn_mask=mask), "bool mask")
+    m2 = torch.rand(8, 8) > 0.3            # broadcast over batch and heads
+    m2[:, 0] = True
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, attn_mask=m2.to(device)),
+                 F.scaled_dot_product_attention(q, k, v, attn_mask=m2), "broadcast bool mask")
+
+
+def test_sdpa_additive_mask(device):
+    q, k, v, dq, dk, dv = _qkv(device)
+    bias = torch.randn(2, 4, 8, 8) * 0.1
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, attn_mask=bias.to(device)),
+                 F.scaled_dot_product_attention(q, k, v, attn_mask=bias), "additive mask")
+
+
+def test_sdpa_gqa(device):
+    B, Lq, Lk, E = 2, 8, 8, 16
+    q, k, v = torch.randn(B, 4, Lq, E), torch.randn(B, 2, Lk, E), torch.randn(B, 2, Lk, E)
+    ref, ref_w = torch.ops.aten._scaled_dot_product_attention_math(q, k, v, None, 0.0, False, None, scale=None, enable_gqa=True)
+    out, w = torch.ops.aten._scaled_dot_product_attention_math(q.to(device), k.to(device), v.to(device), None, 0.0, False,
+                                                               None, scale=None, enable_gqa=True)
+    assert_close(out, ref, "sdpa_gqa")
+    assert_close(w, ref_w, "sdpa_gqa weights")
+    assert_close(F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), enable_gqa=True), ref, "F.sdpa gqa")
+
+
+def test_sdpa_mismatched_gqa_heads_raises(device):
+    q, k, v = torch.randn(1, 5, 4, 8).to(device), torch.randn(1, 2, 4, 8).to(device), torch.randn(1, 2, 4, 8).to(device)
+    with pytest.raises(RuntimeError):
+        torch.ops.aten._scaled_dot_product_attention_math(q, k, v, None, 0.0, False, None, scale=None, enable_gqa=True)
+    with pytest.raises(RuntimeError):
+        torch.ops.aten._scaled_dot_product_attention_math(q, k, v, torch.ones(4, 4, dtype=torch.bool).to(device), 0.0, True, None)
+
+
+def test_sdpa_math_op_returns_host_engine_weights(device):
+    """bf16: the math op's weights equal the host engine's bit for bit."""
+    q, k, v = (torch.randn(2, 4, 8, 16).bfloat16() for _ in range(3))
+    out, w = torch.ops.aten._scaled_dot_product_attention_math(q.to(device), k.to(device), v.to(device), None, 0.0, True, None)
+    want, want_w = O.sdpa_math(q, k, v, is_causal=True, gemm="aten")
+    assert_bit_exact(w.cpu(), want_w, "weights")
+    assert (out.cpu().float() - want.float()).abs().max().item() <= 2 ** -7
+
+
+def test_sdpa_bf16_takes_the_flash_and_decode_kernels(device):
+    q, k, v = (torch.randn(2, 8, 256, 128).bfloat16() for _ in range(3))
+    out = F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), is_causal=True)
+    want, _ = O.sdpa_math(q, k, v, is_causal=True, gemm="aten")
+    assert out.dtype == torch.bfloat16 and (out.cpu().float() - want.float()).abs().max().item() <= 2e-2
+    q1, k1, v1 = torch.randn(2, 8, 1, 128).bfloat16(), torch.randn(2, 2, 777, 128).bfloat16(), torch.randn(2, 2, 777, 128).bfloat16()
+    out = F.scaled_dot_product_attention(q1.to(device), k1.to(device), v1.to(device), enable_gqa=True)
+    want, _ = O.sdpa_math(q1, k1, v1, enable_gqa=True, gemm="aten")
+    assert (out.cpu().float() - want.float()).abs().max().item() <= 2e-2
+    q3 = torch.randn(4, 64, 128).bfloat16()                      # 3-D input
+    out = F.scaled_dot_product_attention(q3.to(device), q3.to(device), q3.to(device))
+    want, _ = O.sdpa_math(q3, q3, q3, gemm="aten")
+    assert out.shape == (4, 64, 128) and (out.cpu().float() - want.float()).abs().max().item() <= 2e-2
+
+
+# ---- aten::rms_norm / torch_paras::swiglu (reference tests/test_attention_norm_ops.py:115-165)
+def test_rms_norm_no_weight(device):
+    x = torch.randn(4, 6, 32)
+    assert_close(torch.ops.aten.rms_norm(x.to(device), [32], None, None), torch.ops.aten.rms_norm(x, [32], None, 1e-6), "no weight")
+
+
+def test_rms_norm_with_weight(device):
+    x, w = torch.randn(4, 6, 32), torch.randn(32)
+    assert_close(torch.ops.aten.rms_norm(x.to(device), [32], w.to(device), 1e-5), torch.ops.aten.rms_norm(x, [32], w, 1e-5), "weight")
+
+
+def test_rms_norm_multi_dim_normalized_shape(device):
+    x = torch.randn(3, 4, 5)
+    assert_close(torch.ops.aten.rms_norm(x.to(device), [4, 5], None, None), torch.ops.aten.rms_norm(x, [4, 5], None, 1e-6), "multi-dim")
+
+
+def test_rms_norm_shape_mismatch_raises(device):
+    with pytest.raises(RuntimeError):
+        torch.ops.aten.rms_norm(torch.randn(4, 6, 32).to(device), [32], torch.randn(16).to(device), None)
+
+
+def test_composed_ops_narrow_like_the_host_engine(device):
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        x, w = torch.randn(37, 200).to(dt), (1 + 0.02 * torch.randn(200)).to(dt)
+        got = torch.ops.aten.rms_norm(x.to(device), [200], w.to(device), 1e-5)
+        assert_bit_exact(got.cpu(), O.rms_norm_composed(x, [200], w, 1e-5), f"aten::rms_norm {dt}")
+        g = (3 * torch.randn(33, 70)).to(dt)
+        u = torch.randn(33, 70).to(dt)
+        got = torch.ops.torch_paras.swiglu(u.to(device), g.to(device))
+        assert_bit_exact(got.cpu(), O.swiglu_composed(u, g), f"torch_paras::swiglu {dt}")
+
+
+def test_swiglu(device):
+    x, gate = torch.randn(4, 32), torch.randn(4, 32)
+    assert_close(torch.ops.torch_paras.swiglu(x.to(device), gate.to(device)), torch.ops.torch_paras.swiglu(x, gate), "swiglu")
+    assert_close(torch.ops.torch_paras.swiglu(x.to(device), gate.to(device)), x * F.silu(gate), "swiglu manual")
+    b = torch.randn(32)
+    assert_close(torch.ops.torch_paras.swiglu(b.to(device), gate.to(device)), b * F.silu(gate), "swiglu broadcast")
+
+
+# ---- fused ops with autograd (reference tests/test_fused_ops.py:8-70) --------------
+def test_fused_forward_and_backward(device):
+    from torch_paras import nn as paras_nn
+    x = torch.randn(4, 8, requires_grad=True)
+    w = torch.randn(8, requires_grad=True)
+    ref = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+    ref.sum().backward()
+    xd, wd = x.detach().to(device).requires_grad_(), w.detach().to(device).requires_grad_()
+    out = paras_nn.rms_norm(xd, wd, 1e-6)
+    out.sum().backward()
+    assert_close(out.detach(), ref.detach(), "rms_norm")
+    assert_close(xd.grad, x.grad, "rms_norm.grad_input")
+    assert_close(wd.grad, w.grad, "rms_norm.grad_weight")
+
+    gate, up = torch.randn(4, 8, requires_grad=True), torch.randn(4, 8, requires_grad=True)
+    (F.silu(gate) * up).sum().backward()
+    gd, ud = gate.detach().to(device).requires_grad_(), up.detach().to(device).requires_grad_()
+    res = paras_nn.swiglu(gd, ud)
+    res.sum().backward()
+    assert_close(res.detach(), (F.silu(gate) * up).detach(), "swiglu")
+    assert_close(gd.grad, gate.grad, "swiglu.grad_gate")
+    assert_close(ud.grad, up.grad, "swiglu.grad_up")
+
+    r = torch.randn(4, 8, requires_grad=True)
+    x1, x2 = r.chunk(2, dim=-1)
+    torch.cat((-x2, x1), dim=-1).sum().backward()
+    rd = r.detach().to(device).requires_grad_()
+    rot = paras_nn.rotate_half(rd)
+    rot.sum().backward()
+    assert_close(rot.detach(), torch.cat((-x2, x1), dim=-1).detach(), "rotate_half")
+    assert_close(rd.grad, r.grad, "rotate_half.grad")
+    with pytest.raises(RuntimeError):
+        paras_nn.swiglu(torch.randn(4, 8).to(device), torch.randn(4, 9).to(device))
+    with pytest.raises(RuntimeError):
+        paras_nn.rms_norm(torch.randn(4, 8).to(device), torch.randn(7).to(device))
+
+
+def test_fused_ops_bf16_match_host_engine(device):
+    from torch_paras import nn as paras_nn
+    x, w = torch.randn(300, 4096).bfloat16(), (1 + 0.02 * torch.randn(4096)).bfloat16()
+    out, rstd = torch.ops.paras.rms_norm(x.to(device), w.to(device), 1e-6)
+    want, wrstd = O.rms_norm(x, w, 1e-6)
+    assert_bit_exact(out.cpu(), want, "paras::rms_norm")
+    assert_bit_exact(rstd.cpu(), wrstd, "rstd")
+    g, u = torch.randn(64, 14336).bfloat16(), torch.randn(64, 14336).bfloat16()
+    assert_bit_exact(paras_nn.swiglu(g.to(device), u.to(device)).cpu(), O.swiglu(g, u), "paras::swiglu")
+    xs = torch.randn(64, 256).bfloat16().to(device)[:, ::2]           # strided input is made contiguous
+    assert_bit_exact(torch.ops.paras.swiglu(xs, xs).cpu(), O.swiglu(xs.cpu().contiguous(), xs.cpu().contiguous()), "strided")
+
+
+# ---- MoE --------------------------------------------------------------------------
+def test_moe_layer(device):
+    from torch_paras import nn as paras_nn
+    T, E, k, H, I = 300, 8, 2, 256, 512
+    dt = torch.bfloat16
+    x, logits = torch.randn(T, H).to(dt), torch.randn(T, E).to(dt)
+    wg, wu, wd = (0.05 * torch.randn(E, I, H)).to(dt), (0.05 * torch.randn(E, I, H)).to(dt), (0.05 * torch.randn(E, H, I)).to(dt)
+    route = paras_nn.moe_route(logits.to(device), k)
+    want = O.moe_route(logits, k)
+    for g, w_ in zip(route, want):
+        assert_bit_exact(g.cpu(), w_, "moe_route")
+    out = paras_nn.moe_layer(x.to(device), logits.to(device), wg.to(device), wu.to(device), wd.to(device), k)
+    ref = O.moe_ffn(x, wg, wu, wd, want[1], want[2], want[3], want[5], k, gemm="aten")
+    assert out.shape == (T, H) and (out.cpu().float() - ref.float()).abs().max().item() <= 2e-2
+
+
+# ---- copies and plumbing (reference tests/test_attention_norm_ops.py:172-216) -----
+def test_copy_same_shape_dtype_cast_and_host(device):
+    a, src = torch.randn(4, 5), torch.randn(4, 5)
+    assert_close(a.to(device).clone().copy_(src.to(device)), a.clone().copy_(src), "copy_same_shape")
+    h = torch.randn(4, 5).half()
+    assert_close(a.to(device).clone().copy_(h.to(device)), a.clone().copy_(h), "copy_dtype_cast")
+    d = torch.randn(4, 5).to(device)
+    s = torch.randn(4, 5)
+    d.copy_(s)
+    assert_close(d.cpu(), s, "copy_from_host")
+    with pytest.raises(RuntimeError):                    # device-to-device broadcast copy is refused, as in the reference
+        torch.randn(4, 5).to(device).clone().copy_(torch.randn(5).to(device))
+
+
+def test_views_strides_fill_item_and_fallback(device):
+    x = torch.randn(6, 8, 10)
+    d = x.to(device)
+    assert_close(d.permute(2, 0, 1).contiguous(), x.permute(2, 0, 1).contiguous(), "permute+contiguous")
+    assert_close(d[:, 2:6, ::3], x[:, 2:6, ::3], "slice to host")
+    assert_close(d.transpose(0, 2).reshape(10, 48), x.transpose(0, 2).reshape(10, 48), "reshape copy")
+    assert_close(d.view(48, 10).t(), x.view(48, 10).t(), "view/t")
+    assert_close(d.to(torch.bfloat16), x.to(torch.bfloat16), "to bf16 on device")
+    assert_close(d.double().float(), x, "round trip through double")
+    z = torch.empty(3, 4, device=device).fill_(2.5)
+    assert_close(z, torch.full((3, 4), 2.5), "fill_")
+    assert_close(torch.zeros(5, dtype=torch.int64, device=device), torch.zeros(5, dtype=torch.int64), "zeros int64")
+    z[:, 1].zero_()
+    assert z.cpu()[:, 1].abs().sum().item() == 0 and z.cpu()[:, 0].sum().item() == 7.5
+    assert d[1, 2, 3].item() == x[1, 2, 3].item()
+    assert_close(torch.relu(d) + 1, torch.relu(x) + 1, "CPU fallback ops")           # unregistered ops bounce through the host
+    assert_close((d @ d.transpose(1, 2)), x @ x.transpose(1, 2), "matmul fallback")
+    i = torch.arange(12, device=device).view(3, 4)
+    assert_close(i.t().contiguous(), torch.arange(12).view(3, 4).t().contiguous(), "int64 strided copy")
+
+
+def test_threads_dispatch_concurrently(device):
+    import threading
+    errs = []
+
+    def work():
+        try:
+            x = torch.randn(64, 512).bfloat16()
+            w = torch.ones(512).bfloat16()
+            for _ in range(20):
+                out, _ = torch.ops.paras.rms_norm(x.to(device), w.to(device), 1e-6)
+            want, _ = O.rms_norm(x, w, 1e-6)
+            assert torch.equal(out.cpu().view(torch.int16), want.view(torch.int16))
+        except Exception as e:  # noqa: BLE001
+            errs.append(e)
+    ts = [threading.Thread(target=work) for _ in range(4)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert not errs, errs

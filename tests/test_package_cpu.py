@@ -1,0 +1,40 @@
+"""Without a GPU: the package imports, registers the `paras` device and its op
+schemas, reports no device, and refuses to run instead of falling back."""
+import pytest
+import torch
+
+
+def test_import_registers_device_and_schemas():
+    import torch_paras
+    assert torch_paras.backend_name() == "paras-hip"
+    assert torch._C._get_privateuse1_backend_name() == "paras"
+    assert hasattr(torch, "paras") and callable(torch.paras.is_available)
+    for name in ("rms_norm", "rms_norm_backward", "swiglu", "swiglu_backward", "rotate_half", "rotate_half_backward",
+                 "moe_route", "moe_ffn"):
+        assert hasattr(torch.ops.paras, name)
+    s = str(torch.ops.paras.rms_norm.default._schema)
+    assert s == "paras::rms_norm(Tensor input, Tensor weight, float eps) -> (Tensor, Tensor)"      # fused_ops.cpp:308
+    assert str(torch.ops.torch_paras.swiglu.default._schema) == "torch_paras::swiglu(Tensor x, Tensor gate) -> Tensor"
+    for op in ("aten::_scaled_dot_product_attention_math", "aten::rms_norm", "aten::_copy_from", "aten::empty.memory_format"):
+        assert torch._C._dispatch_has_kernel_for_dispatch_key(op, "PrivateUse1"), op
+    for fn in ("device_count", "is_available", "synchronize", "manual_seed", "manual_seed_all", "empty_cache", "device_name",
+               "backend_name", "is_gpu_device", "memory_allocated", "memory_cached", "get_amp_supported_dtype"):
+        assert callable(getattr(torch_paras, fn))
+    assert {"rms_norm", "swiglu", "rotate_half"} <= set(torch_paras.nn.__all__)
+
+
+def test_cpu_kernel_of_torch_paras_swiglu():
+    import torch_paras  # noqa: F401
+    x, g = torch.randn(4, 32), torch.randn(4, 32)
+    assert torch.equal(torch.ops.torch_paras.swiglu(x, g), x * torch.nn.functional.silu(g))
+
+
+def test_no_device_means_error_not_fallback():
+    import torch_paras
+    if torch_paras.device_count() > 0:
+        pytest.skip("a GPU is visible: covered by the gpu tests")
+    assert not torch_paras.is_available() and not torch.paras.is_available()
+    with pytest.raises(RuntimeError, match="invalid device index"):
+        torch.randn(4).to("paras")
+    with pytest.raises(RuntimeError):
+        torch.empty(4, device="paras:0")
