@@ -131,17 +131,43 @@ unsigned grid_for(long n) {
 
 int make_spec(int ndim, const int64_t* sizes, const int64_t* ss, const int64_t* ds, Strided* s, long* n) {
     PARAS_REQUIRE(ndim >= 0 && ndim <= kMaxDims, "paras: tensor rank %d exceeds kernel limit of %d", ndim, kMaxDims);
-    s->ndim = ndim;
+    // Size-1 dimensions are dropped and a dimension whose stride on both sides
+    // equals the extent of the next one is merged into it, so a contiguous tensor
+    // of any rank arrives at the kernels as one dimension of stride 1.
     long total = 1;
+    int m = 0;
     for (int d = 0; d < ndim; ++d) {
         PARAS_REQUIRE(sizes[d] >= 0, "paras: negative size");
-        s->sizes[d] = sizes[d];
-        s->src_strides[d] = ss ? ss[d] : 0;
-        s->dst_strides[d] = ds ? ds[d] : 0;
         total *= sizes[d];
+        if (sizes[d] == 1) continue;
+        s->sizes[m] = sizes[d];
+        s->src_strides[m] = ss ? ss[d] : 0;
+        s->dst_strides[m] = ds ? ds[d] : 0;
+        ++m;
     }
+    for (int d = m - 2; d >= 0 && total > 0; --d) {
+        if (s->src_strides[d] == s->src_strides[d + 1] * s->sizes[d + 1] &&
+            s->dst_strides[d] == s->dst_strides[d + 1] * s->sizes[d + 1]) {
+            s->sizes[d] *= s->sizes[d + 1];
+            s->src_strides[d] = s->src_strides[d + 1];
+            s->dst_strides[d] = s->dst_strides[d + 1];
+            for (int e = d + 1; e + 1 < m; ++e) {
+                s->sizes[e] = s->sizes[e + 1];
+                s->src_strides[e] = s->src_strides[e + 1];
+                s->dst_strides[e] = s->dst_strides[e + 1];
+            }
+            --m;
+        }
+    }
+    s->ndim = m;
     *n = total;
     return PARAS_OK;
+}
+
+// Both sides dense: a plain stream of 16-byte vectors, one per thread, past the cache.
+__global__ __launch_bounds__(kBlock) void copy_dense_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, long nvec) {
+    const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < nvec) store16_nt(dst + i, load16_nt(src + i));
 }
 
 template <typename TS>
@@ -179,6 +205,22 @@ int paras_copy_strided(const void* src, void* dst, int ndim, const int64_t* size
     if (rc != PARAS_OK) return rc;
     const dim3 g(grid_for(n)), b(kBlock);
     if (src_dtype == dst_dtype) {
+        const bool dense = s.ndim == 0 || (s.ndim == 1 && s.src_strides[0] == 1 && s.dst_strides[0] == 1);
+        const long bytes = n * elem_size;
+        if (dense && bytes >= 16 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0) {
+            const long nvec = bytes / 16;
+            hipLaunchKernelGGL(copy_dense_kernel, dim3(static_cast<unsigned>((nvec + kBlock - 1) / kBlock)), b, 0, st,
+                               static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), nvec);
+            PARAS_HIP_TRY(hipGetLastError());
+            const long done = nvec * 16 / elem_size;
+            if (done == n) return PARAS_OK;
+            // tail of fewer than 16 bytes: the element kernel on what is left
+            src = static_cast<const char*>(src) + nvec * 16;
+            dst = static_cast<char*>(dst) + nvec * 16;
+            n -= done;
+            s.ndim = 1; s.sizes[0] = n; s.src_strides[0] = 1; s.dst_strides[0] = 1;
+        }
+        const dim3 g(grid_for(n));
         switch (elem_size) {
             case 1: hipLaunchKernelGGL((copy_same_kernel<uint8_t>), g, b, 0, st, static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), n, s); break;
             case 2: hipLaunchKernelGGL((copy_same_kernel<uint16_t>), g, b, 0, st, static_cast<const uint16_t*>(src), static_cast<uint16_t*>(dst), n, s); break;

@@ -22,7 +22,14 @@
 //                  A = V^T read from the row-major V tile with
 //                  ds_read_b64_tr_b16, which transposes 4 keys x 16 d per
 //                  16-lane group in the LDS crossbar
-//   rescaling O by exp(m_old - m_new) is a per-lane scalar multiply.
+//   rescaling O by exp(m_old - m_new) is a per-lane scalar multiply, and it
+//                  is lazy: the running max is only raised (and O, l rescaled)
+//                  when a tile's row max exceeds it by more than 2^8 in the
+//                  exponent domain, so after the first tile the rescale is
+//                  skipped almost always; the same (possibly stale) max is used
+//                  for P and for the row sum, so out = O / l is unchanged.
+//   row sums       v_dot2_f32_{bf16,f16} on the packed 16-bit P (two elements
+//                  per instruction, and exactly the values the PV product uses)
 //
 // v_mfma_f32_32x32x16_{bf16,f16}: 32 MFMAs per wave per 64-key tile at D=128.
 #include <hip/hip_runtime.h>
@@ -72,6 +79,12 @@ template <> struct Mma<bf16_t> {
         const f32x2 v = {lo, hi};
         return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, bf16x2));
     }
+    // acc + both halves of a packed pair
+    __device__ static __forceinline__ float add_pair(std::uint32_t pk, float acc) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        const bf16x2 ones = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), ones, acc, false);
+    }
 };
 template <> struct Mma<f16_t> {
     __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
@@ -83,6 +96,11 @@ template <> struct Mma<f16_t> {
         typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
         const f32x2 v = {lo, hi};
         return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, f16x2));
+    }
+    __device__ static __forceinline__ float add_pair(std::uint32_t pk, float acc) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        const f16x2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), ones, acc, false);
     }
 };
 
@@ -143,7 +161,8 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
     const int b = bh / p.Hq, hq = bh % p.Hq;
     const int hkv = hq / (p.Hq / p.Hkv);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps per-wave branches scalar
     const int lq = lane & 31, lh = lane >> 5;
     const int q0 = qblock * kBM + wave * 32;  // first query of this wave
     const int my_q = q0 + lq;
@@ -170,19 +189,33 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
     }
 
     // ---- tile staging: each thread moves LOADS 16-byte chunks of K and of V.
+    // Addresses are a wave-uniform tile base plus a per-thread 32-bit offset
+    // that never changes, so the loop spends no vector ALU on addressing.
     u32x4 kst[LOADS], vst[LOADS];
-    auto load_tile = [&](int t) {
+    unsigned koff[LOADS], voff[LOADS];
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = tid + i * kThreads;
-            const int row = c / CHUNKS, col = (c % CHUNKS) * 8;
-            const int key = t * kBN + row;
-            if (key < p.Lk) {
-                kst[i] = load16(kbase + static_cast<long>(key) * p.ks_l + col);
-                vst[i] = load16(vbase + static_cast<long>(key) * p.vs_l + col);
-            } else {
-                kst[i] = u32x4{0, 0, 0, 0};
-                vst[i] = u32x4{0, 0, 0, 0};
+    for (int i = 0; i < LOADS; ++i) {
+        const int c = tid + i * kThreads;
+        const int row = c / CHUNKS, col = (c % CHUNKS) * 8;
+        koff[i] = static_cast<unsigned>(row * p.ks_l + col);
+        voff[i] = static_cast<unsigned>(row * p.vs_l + col);
+    }
+    auto load_tile = [&](int t) {
+        const std::uint16_t* kt = kbase + static_cast<long>(t) * kBN * p.ks_l;
+        const std::uint16_t* vt = vbase + static_cast<long>(t) * kBN * p.vs_l;
+        if ((t + 1) * kBN <= p.Lk) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                kst[i] = load16(kt + koff[i]);
+                vst[i] = load16(vt + voff[i]);
+            }
+        } else {  // last, partial tile: rows past the end read as zero
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                const int row = (tid + i * kThreads) / CHUNKS;
+                const bool live = t * kBN + row < p.Lk;
+                kst[i] = live ? load16(kt + koff[i]) : u32x4{0, 0, 0, 0};
+                vst[i] = live ? load16(vt + voff[i]) : u32x4{0, 0, 0, 0};
             }
         }
     };
@@ -213,89 +246,94 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
     const int grp = lane >> 4, m16 = lane & 15;
     const int v_off = (4 * lh + (m16 >> 2)) * VS + 16 * (grp & 1) + 4 * (m16 & 3);  // + (kb*32+16s(+8))*VS + db*32
 
+    // Raise the running max only when a tile exceeds it by more than this much
+    // (raw score units): exp2((s - m) * scale_log2) then stays below 2^8.
+    const float lazy_margin = 8.0f / p.scale_log2;
+
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
         if (t + 1 < n_tiles) load_tile(t + 1);
-
-        // ---- S^T = K Q^T for the two 32-key blocks of the tile
-        float16_t sacc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                const i16x8 a = *reinterpret_cast<const i16x8*>(&k_lds[buf][k_off + kb * 32 * KS + ks * 16]);
-                sacc[kb] = Mma<T>::run(a, qreg[ks], sacc[kb]);
-            }
-        }
-
-        // ---- masking (only tiles that touch the diagonal or the end of K)
         const int key0 = t * kBN;
-        const bool need_mask = (kCausal && key0 + kBN - 1 > q0) || (key0 + kBN > p.Lk);
-        if (need_mask) {
+        // A causal tile that lies entirely above this wave's queries contributes nothing.
+        const bool wave_has_work = !kCausal || key0 <= q0 + 31;
+        if (wave_has_work) {
+            // ---- S^T = K Q^T for the two 32-key blocks of the tile
+            float16_t sacc[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) {
+                    const i16x8 a = *reinterpret_cast<const i16x8*>(&k_lds[buf][k_off + kb * 32 * KS + ks * 16]);
+                    sacc[kb] = Mma<T>::run(a, qreg[ks], sacc[kb]);
+                }
+            }
+
+            // ---- masking (only tiles that touch the diagonal or the end of K):
+            // element (kb, r) sits at key offset kb*32 + (r/4)*8 + r%4 from this lane's
+            // first key; it is dead when that offset exceeds `rel`.
+            const bool need_mask = (kCausal && key0 + kBN - 1 > q0) || (key0 + kBN > p.Lk);
+            if (need_mask) {
+                const int last_visible = kCausal ? min(my_q, p.Lk - 1) : p.Lk - 1;
+                const int rel = last_visible - key0 - 4 * lh;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (kb * 32 + (r >> 2) * 8 + (r & 3) > rel) sacc[kb][r] = -INFINITY;
+            }
+
+            // ---- online softmax with a lazily raised running max
+            float mloc = sacc[0][0];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int key = key0 + kb * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
-                    const bool dead = (kCausal && key > my_q) || key >= p.Lk;
-                    if (dead) sacc[kb][r] = -INFINITY;
+                for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
+            mloc = half_swap_max(mloc);
+            if (__builtin_amdgcn_ballot_w64(mloc > m_run + lazy_margin) != 0) {  // wave-uniform
+                const float m_new = fmaxf(m_run, mloc);
+                const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2);
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+            }
+            const float mc = m_run * p.scale_log2;
+
+            // ---- P^T as MFMA B operands (two k-steps of 16 keys per 32-key block)
+            i16x8 pb[2][2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                    u32x4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float e0 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][8 * s2 + 2 * e], p.scale_log2, -mc));
+                        const float e1 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][8 * s2 + 2 * e + 1], p.scale_log2, -mc));
+                        w[e] = Mma<T>::pack2(e0, e1);
+                        l_run = Mma<T>::add_pair(w[e], l_run);
+                    }
+                    pb[kb][s2] = __builtin_bit_cast(i16x8, w);
                 }
+
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        const std::uint16_t* vp = &v_lds[buf][v_off + (kb * 32 + 16 * s2) * VS + db * 32];
+                        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+                        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * VS));
+                        const i16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        oacc[db] = Mma<T>::run(a, pb[kb][s2], oacc[db]);
+                    }
         }
-
-        // ---- online softmax
-        float mloc = sacc[0][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
-        mloc = half_swap_max(mloc);
-        const float m_new = fmaxf(m_run, mloc);
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2);
-        const float mc = m_new * p.scale_log2;
-        m_run = m_new;
-        float lsum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e = __builtin_amdgcn_exp2f(fmaf(sacc[kb][r], p.scale_log2, -mc));
-                sacc[kb][r] = e;
-                lsum += e;
-            }
-        l_run = l_run * alpha + lsum;
-#pragma unroll
-        for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-
-        // ---- P^T as MFMA B operands (two k-steps of 16 keys per 32-key block)
-        i16x8 pb[2][2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                u32x4 w;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    w[e] = Mma<T>::pack2(sacc[kb][8 * s + 2 * e], sacc[kb][8 * s + 2 * e + 1]);
-                pb[kb][s] = __builtin_bit_cast(i16x8, w);
-            }
-
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int db = 0; db < DBLK; ++db)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    const std::uint16_t* vp = &v_lds[buf][v_off + (kb * 32 + 16 * s) * VS + db * 32];
-                    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
-                    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * VS));
-                    const i16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    oacc[db] = Mma<T>::run(a, pb[kb][s], oacc[db]);
-                }
 
         // ---- publish the next tile
         if (t + 1 < n_tiles) store_tile(buf ^ 1);

@@ -114,7 +114,12 @@ def test_flash_matches_oracle(dtype, shape):
     s = (q.float() @ k.float().repeat_interleave(rep, 1).transpose(-1, -2)) / math.sqrt(D)
     if causal:
         s = s.masked_fill(~torch.ones(Lq, Lk).tril().bool(), -math.inf)
-    assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=1e-3, atol=1e-3)
+    # The kernel sums the row denominator from the probabilities as rounded to the
+    # 16-bit MFMA operand (so numerator and denominator see the same rounding):
+    # one probability carries up to 2^-9 (bf16) / 2^-12 (f16) relative error, and
+    # a row dominated by one key passes that on to exp(lse).
+    tol = 4e-3 if dtype == torch.bfloat16 else 1e-3
+    assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=tol, atol=tol)
 
 
 def test_flash_strided_inputs_and_explicit_scale():
