@@ -7,7 +7,10 @@
 // Work decomposition
 //   workgroup = 4 wavefronts = 128 queries of one (batch, head); each wave owns
 //   32 queries.  K/V are streamed in tiles of 64 keys through LDS (double
-//   buffered, one barrier per tile), shared by the 4 waves.
+//   buffered, one barrier per tile), shared by the 4 waves.  Tiles go from
+//   global memory straight into LDS (global_load_lds_dwordx4: no staging
+//   registers, no LDS store instructions); rows are unpadded and the 16-byte
+//   chunks of a row are XOR-swizzled so that operand reads stay conflict free.
 //
 // The products are formed transposed so that a lane always owns ONE query:
 //   S^T = K Q^T    A = K tile from LDS (lane: key l%32, 8 consecutive d),
@@ -44,9 +47,6 @@
 namespace paras {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves   = 4;
-constexpr int kBM      = 128;  // queries per workgroup
 constexpr int kBN      = 64;   // keys per tile
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -129,17 +129,29 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return lo + hi;
 }
 
-template <typename T, int D, bool kCausal>
-__global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParams p) {
-    constexpr int KS     = D + 8;    // K row stride in LDS (elements): 16-byte reads of 16 keys hit 64 distinct banks
-    constexpr int VS     = D + 32;   // V row stride: 4 consecutive keys x 64 bytes tile all 64 banks
+template <typename T, int D, bool kCausal, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void flash_fwd_kernel(const FlashParams p) {
+    constexpr int kThreads = NW * 64;  // NW waves of 32 queries share each K/V tile
+    constexpr int kBM      = NW * 32;
     constexpr int KSTEPS = D / 16;   // MFMA k-steps over the head dim
     constexpr int DBLK   = D / 32;   // 32-wide blocks of the output head dim
     constexpr int CHUNKS = D / 8;    // 16-byte chunks per row
-    constexpr int LOADS  = kBN * CHUNKS / kThreads;  // chunks per thread per tile
+    // Tiles are written by direct global->LDS loads: one wave instruction lays
+    // 64 x 16 bytes down contiguously, so rows are unpadded (D elements) and bank
+    // conflicts are avoided by XOR-ing the chunk index with a function of the row
+    // (the lane picks which global chunk it fetches for its fixed LDS slot).
+    //   K: slot = chunk ^ ksw(row): 16 consecutive rows at one chunk index cover all 64 banks
+    //      for the 16-byte operand reads;
+    //   V: slot = chunk ^ vsw(row): 4 consecutive rows x 64 bytes cover all 64 banks for the
+    //      transposed 8-byte reads.
+    constexpr int RPI    = 64 / CHUNKS;              // rows one wave instruction fills (1 KiB)
+    constexpr int NI     = kBN / (RPI * NW);         // instructions per wave per matrix per tile
+    static_assert(NI >= 1 && NI * RPI * NW == kBN, "tile does not split over the waves");
+    auto ksw = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto vsw = [](int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
 
-    __shared__ __attribute__((aligned(16))) std::uint16_t k_lds[2][kBN * KS];
-    __shared__ __attribute__((aligned(16))) std::uint16_t v_lds[2][kBN * VS];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds[2][kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds[2][kBN * D];
 
     // ---- which (batch, head, query block): heavy causal blocks first, and all
     // query blocks of one head on one XCD so its K/V stay in that XCD's L2.
@@ -188,45 +200,47 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
         n_tiles = (need + kBN - 1) / kBN;
     }
 
-    // ---- tile staging: each thread moves LOADS 16-byte chunks of K and of V.
-    // Addresses are a wave-uniform tile base plus a per-thread 32-bit offset
-    // that never changes, so the loop spends no vector ALU on addressing.
-    u32x4 kst[LOADS], vst[LOADS];
-    unsigned koff[LOADS], voff[LOADS];
-#pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        const int c = tid + i * kThreads;
-        const int row = c / CHUNKS, col = (c % CHUNKS) * 8;
-        koff[i] = static_cast<unsigned>(row * p.ks_l + col);
-        voff[i] = static_cast<unsigned>(row * p.vs_l + col);
-    }
-    auto load_tile = [&](int t) {
+    // ---- tile staging.  Wave w, instruction i fills rows i*RPI*NW + w*RPI .. +RPI-1;
+    // RPI*NW is a multiple of 16, so a lane's swizzle (and its global offset
+    // apart from a uniform row step) is the same for every i.
+    const int srow = wave * RPI + lane / CHUNKS;     // row within the first group
+    const int slot = lane % CHUNKS;
+    const unsigned koff = static_cast<unsigned>(srow * p.ks_l + ((slot ^ ksw(srow)) * 8));
+    const unsigned voff = static_cast<unsigned>(srow * p.vs_l + ((slot ^ vsw(srow)) * 8));
+    typedef __attribute__((address_space(1))) const void* gptr_t;
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    auto stage_tile = [&](int t, int buf) {
         const std::uint16_t* kt = kbase + static_cast<long>(t) * kBN * p.ks_l;
         const std::uint16_t* vt = vbase + static_cast<long>(t) * kBN * p.vs_l;
         if ((t + 1) * kBN <= p.Lk) {
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                kst[i] = load16(kt + koff[i]);
-                vst[i] = load16(vt + voff[i]);
+            for (int i = 0; i < NI; ++i) {
+                const int r0 = i * RPI * NW;                      // uniform row step
+                __builtin_amdgcn_global_load_lds((gptr_t)(kt + static_cast<long>(r0) * p.ks_l + koff),
+                                                 (lptr_t)&k_lds[buf][(r0 + wave * RPI) * D], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(vt + static_cast<long>(r0) * p.vs_l + voff),
+                                                 (lptr_t)&v_lds[buf][(r0 + wave * RPI) * D], 16, 0, 0);
             }
-        } else {  // last, partial tile: rows past the end read as zero
+        } else {  // last, partial tile: rows past the end of K/V read as zero
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                const int row = (tid + i * kThreads) / CHUNKS;
-                const bool live = t * kBN + row < p.Lk;
-                kst[i] = live ? load16(kt + koff[i]) : u32x4{0, 0, 0, 0};
-                vst[i] = live ? load16(vt + voff[i]) : u32x4{0, 0, 0, 0};
+            for (int i = 0; i < NI; ++i) {
+                const int r0 = i * RPI * NW;
+                std::uint16_t* kd = &k_lds[buf][(r0 + wave * RPI) * D];
+                std::uint16_t* vd = &v_lds[buf][(r0 + wave * RPI) * D];
+                if (t * kBN + r0 + srow < p.Lk) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(kt + static_cast<long>(r0) * p.ks_l + koff), (lptr_t)kd, 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((gptr_t)(vt + static_cast<long>(r0) * p.vs_l + voff), (lptr_t)vd, 16, 0, 0);
+                } else {
+                    *reinterpret_cast<u32x4*>(kd + lane * 8) = u32x4{0, 0, 0, 0};
+                    *reinterpret_cast<u32x4*>(vd + lane * 8) = u32x4{0, 0, 0, 0};
+                }
             }
         }
     };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            const int c = tid + i * kThreads;
-            const int row = c / CHUNKS, col = (c % CHUNKS) * 8;
-            *reinterpret_cast<u32x4*>(&k_lds[buf][row * KS + col]) = kst[i];
-            *reinterpret_cast<u32x4*>(&v_lds[buf][row * VS + col]) = vst[i];
-        }
+    // Direct loads land in LDS asynchronously: drain them before the barrier that publishes the tile.
+    auto publish = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     };
 
     float16_t oacc[DBLK];
@@ -237,26 +251,38 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
     float m_run = -INFINITY;  // running max of raw scores (before scaling)
     float l_run = 0.f;        // this half-wave's share of the running sum
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
+    stage_tile(0, 0);
+    publish();
 
-    // Per-lane LDS offsets.
-    const int k_off = lq * KS + lh * 8;                                        // + kb*32*KS + ks*16
+    // Per-lane LDS read offsets (elements).  K operand of k-step ks: row lq (+32 kb),
+    // chunk 2ks+lh; V^T operand of d-block db: row 4lh + m16/4 (+ 32kb + 16s2 [+8]),
+    // chunk 4db + 2(grp&1) + (m16&3)/2, 8-byte half (m16&1).  Row offsets that are
+    // multiples of 16 (K: 32) leave the swizzle unchanged, so they stay immediates.
     const int grp = lane >> 4, m16 = lane & 15;
-    const int v_off = (4 * lh + (m16 >> 2)) * VS + 16 * (grp & 1) + 4 * (m16 & 3);  // + (kb*32+16s(+8))*VS + db*32
+    int k_rd[KSTEPS], v_rd[DBLK];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) k_rd[ks] = lq * D + (((2 * ks + lh) ^ ksw(lq)) * 8);
+    {
+        const int vrow = 4 * lh + (m16 >> 2);
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+            v_rd[db] = vrow * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
+    }
 
     // Raise the running max only when a tile exceeds it by more than this much
     // (raw score units): exp2((s - m) * scale_log2) then stays below 2^8.
     const float lazy_margin = 8.0f / p.scale_log2;
 
-    for (int t = 0; t < n_tiles; ++t) {
+    // Tiles this wave computes on: a causal tile that lies entirely above the
+    // wave's queries contributes nothing.  The wave still helps stage those tiles
+    // for the others (second loop below).
+    const int wave_tiles = kCausal ? min(n_tiles, (q0 + 31) / kBN + 1) : n_tiles;
+
+    for (int t = 0; t < wave_tiles; ++t) {
         const int buf = t & 1;
-        if (t + 1 < n_tiles) load_tile(t + 1);
+        if (t + 1 < n_tiles) stage_tile(t + 1, buf ^ 1);
         const int key0 = t * kBN;
-        // A causal tile that lies entirely above this wave's queries contributes nothing.
-        const bool wave_has_work = !kCausal || key0 <= q0 + 31;
-        if (wave_has_work) {
+        {
             // ---- S^T = K Q^T for the two 32-key blocks of the tile
             float16_t sacc[2];
 #pragma unroll
@@ -265,7 +291,7 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
                 for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const i16x8 a = *reinterpret_cast<const i16x8*>(&k_lds[buf][k_off + kb * 32 * KS + ks * 16]);
+                    const i16x8 a = *reinterpret_cast<const i16x8*>(&k_lds[buf][k_rd[ks] + kb * 32 * D]);
                     sacc[kb] = Mma<T>::run(a, qreg[ks], sacc[kb]);
                 }
             }
@@ -327,17 +353,20 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int s2 = 0; s2 < 2; ++s2) {
-                        const std::uint16_t* vp = &v_lds[buf][v_off + (kb * 32 + 16 * s2) * VS + db * 32];
+                        const std::uint16_t* vp = &v_lds[buf][v_rd[db] + (kb * 32 + 16 * s2) * D];
                         const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
-                        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * VS));
+                        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
                         const i16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                         oacc[db] = Mma<T>::run(a, pb[kb][s2], oacc[db]);
                     }
         }
 
         // ---- publish the next tile
-        if (t + 1 < n_tiles) store_tile(buf ^ 1);
-        __syncthreads();
+        publish();
+    }
+    for (int t = wave_tiles; t < n_tiles; ++t) {
+        if (t + 1 < n_tiles) stage_tile(t + 1, (t & 1) ^ 1);
+        publish();
     }
 
     // ---- epilogue: normalise and store O[q][d]; lane holds 4 consecutive d per (db, r/4)
@@ -360,15 +389,23 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(const FlashParam
     }
 }
 
-template <typename T, int D>
-int launch_t(const FlashParams& p, bool causal, hipStream_t s) {
+template <typename T, int D, int NW>
+int launch_nw(FlashParams p, bool causal, hipStream_t s) {
+    p.n_qblocks = (p.Lq + NW * 32 - 1) / (NW * 32);
     const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
     if (causal)
-        hipLaunchKernelGGL((flash_fwd_kernel<T, D, true>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_fwd_kernel<T, D, true, NW>), dim3(static_cast<unsigned>(blocks)), dim3(NW * 64), 0, s, p);
     else
-        hipLaunchKernelGGL((flash_fwd_kernel<T, D, false>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((flash_fwd_kernel<T, D, false, NW>), dim3(static_cast<unsigned>(blocks)), dim3(NW * 64), 0, s, p);
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
+}
+
+template <typename T, int D>
+int launch_t(const FlashParams& p, bool causal, hipStream_t s) {
+    // 4 waves (128 queries) per workgroup: 8 waves sharing each tile halve the L2 -> LDS
+    // traffic but measured 9 % slower (more waves idle at each barrier and on the causal diagonal).
+    return launch_nw<T, D, 4>(p, causal, s);
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -384,7 +421,7 @@ bool flash_supported(const paras_sdpa_args& a) {
     if (!(a.scale > 0.0) || !std::isfinite(a.scale)) return false;  // the running max is taken on raw scores
     if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.out)) return false;
     if (!mult8(a.q_strides) || !mult8(a.k_strides) || !mult8(a.v_strides)) return false;
-    const int64_t nq = (a.Lq + kBM - 1) / kBM;
+    const int64_t nq = (a.Lq + 127) / 128;
     if (a.B * a.Hq * nq > 0x7fffffffLL || a.Lq > 0x3fffffff || a.Lk > 0x3fffffff) return false;
     return true;
 }
@@ -401,7 +438,7 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     p.vs_b = a.v_strides[0]; p.vs_h = a.v_strides[1]; p.vs_l = a.v_strides[2];
     p.B = static_cast<int>(a.B); p.Hq = static_cast<int>(a.Hq); p.Hkv = static_cast<int>(a.Hkv);
     p.Lq = static_cast<int>(a.Lq); p.Lk = static_cast<int>(a.Lk);
-    p.n_qblocks = static_cast<int>((a.Lq + kBM - 1) / kBM);
+    p.n_qblocks = 0;  // set by the launcher for the workgroup size it picks
     p.scale = static_cast<float>(a.scale);
     p.scale_log2 = static_cast<float>(a.scale * 1.4426950408889634);
     const bool causal = a.is_causal != 0;
