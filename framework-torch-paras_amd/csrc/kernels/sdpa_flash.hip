@@ -6,11 +6,11 @@
 //
 // Work decomposition
 //   workgroup = 4 wavefronts = 128 queries of one (batch, head); each wave owns
-//   32 queries.  K/V are streamed in tiles of 64 keys through LDS (double
-//   buffered, one barrier per tile), shared by the 4 waves.  Tiles go from
-//   global memory straight into LDS (global_load_lds_dwordx4: no staging
-//   registers, no LDS store instructions); rows are unpadded and the 16-byte
-//   chunks of a row are XOR-swizzled so that operand reads stay conflict free.
+//   32 queries.  K/V are streamed in tiles of 64 keys through LDS (two buffers
+//   each, one barrier per tile), shared by the 4 waves.  Tiles go from global
+//   memory straight into LDS (global_load_lds_dwordx4: no staging registers, no
+//   LDS store instructions); rows are unpadded and the 16-byte chunks of a row
+//   are XOR-swizzled so that operand reads stay conflict free.
 //
 // The products are formed transposed so that a lane always owns ONE query:
 //   S^T = K Q^T    A = K tile from LDS (lane: key l%32, 8 consecutive d),
@@ -27,17 +27,31 @@
 //                  16-lane group in the LDS crossbar
 //   rescaling O by exp(m_old - m_new) is a per-lane scalar multiply, and it
 //                  is lazy: the running max is only raised (and O, l rescaled)
-//                  when a tile's row max exceeds it by more than 2^8 in the
-//                  exponent domain, so after the first tile the rescale is
+//                  when a block's row max exceeds it by more than 2^8 in the
+//                  exponent domain, so after the first block the rescale is
 //                  skipped almost always; the same (possibly stale) max is used
 //                  for P and for the row sum, so out = O / l is unchanged.
 //   row sums       v_dot2_f32_{bf16,f16} on the packed 16-bit P (two elements
 //                  per instruction, and exactly the values the PV product uses)
 //
+// Software pipeline inside a wave: the unit of work is a 32-key block and the
+// score MFMAs run one block ahead,
+//
+//   block j:   [ S(j+1) = K(j+1) Q^T  MFMAs  |  exp / pack / row-sum of S(j) ]   one fenced schedule,
+//              [ O^T += V(j)^T P(j)^T MFMAs  |  in-lane row max of S(j+1)    ]   an MFMA per slot
+//              mask S(j+1) on the diagonal / at the end of K; raise the running max if needed (rare branch)
+//
+// so the matrix pipe has independent work in flight under the softmax VALU
+// work of the same wave.  K is staged half a tile ahead of V: K tile u holds
+// keys [64u-32, 64u+32), so the two blocks whose scores are computed during V
+// tile t (blocks 2t+1, 2t+2) both live in K tile t+1, and K and V need only two
+// LDS buffers each with a single barrier per tile.
+//
 // v_mfma_f32_32x32x16_{bf16,f16}: 32 MFMAs per wave per 64-key tile at D=128.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
@@ -47,7 +61,8 @@
 namespace paras {
 namespace {
 
-constexpr int kBN      = 64;   // keys per tile
+constexpr int kBN = 64;    // keys per tile
+constexpr int kBM = 128;   // queries per workgroup: 4 waves x 32
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
@@ -114,7 +129,7 @@ template <> struct Mma<f16_t> {
 // hazard recognizer cannot see inside an asm block.
 __device__ __forceinline__ void half_swap(float x, float& lo, float& hi) {
     float a = x, b = x;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
     lo = a;
     hi = b;
 }
@@ -129,38 +144,40 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return lo + hi;
 }
 
-template <typename T, int D, bool kCausal, int NW>
-__global__ __launch_bounds__(NW * 64, 8 / NW) void flash_fwd_kernel(const FlashParams p) {
-    constexpr int kThreads = NW * 64;  // NW waves of 32 queries share each K/V tile
-    constexpr int kBM      = NW * 32;
-    constexpr int KSTEPS = D / 16;   // MFMA k-steps over the head dim
-    constexpr int DBLK   = D / 32;   // 32-wide blocks of the output head dim
-    constexpr int CHUNKS = D / 8;    // 16-byte chunks per row
-    // Tiles are written by direct global->LDS loads: one wave instruction lays
-    // 64 x 16 bytes down contiguously, so rows are unpadded (D elements) and bank
-    // conflicts are avoided by XOR-ing the chunk index with a function of the row
-    // (the lane picks which global chunk it fetches for its fixed LDS slot).
-    //   K: slot = chunk ^ ksw(row): 16 consecutive rows at one chunk index cover all 64 banks
-    //      for the 16-byte operand reads;
-    //   V: slot = chunk ^ vsw(row): 4 consecutive rows x 64 bytes cover all 64 banks for the
-    //      transposed 8-byte reads.
-    constexpr int RPI    = 64 / CHUNKS;              // rows one wave instruction fills (1 KiB)
-    constexpr int NI     = kBN / (RPI * NW);         // instructions per wave per matrix per tile
-    static_assert(NI >= 1 && NI * RPI * NW == kBN, "tile does not split over the waves");
+template <typename T, int D, bool kCausal>
+__global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) {
+    // 32-query blocks per wave.  The code is written for any QB; 2 halves the LDS operand
+    // traffic per query but needs one wave per SIMD and measured 30 % slower (nothing hides
+    // LDS / barrier latency then), so 1 it is: two waves per SIMD, 256 registers each.
+    constexpr int QB     = 1;
+    constexpr int NW     = 4;
+    constexpr int WQ     = 32 * QB;          // queries per wave
+    static_assert(kBM == NW * WQ, "workgroup shape");
+    constexpr int KSTEPS = D / 16;
+    constexpr int DBLK   = D / 32;
+    constexpr int CHUNKS = D / 8;
+    constexpr int RPI    = 64 / CHUNKS;
+    constexpr int NI     = kBN / (RPI * NW);
     auto ksw = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
     auto vsw = [](int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
 
-    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds[2][kBN * D];
-    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds[2][kBN * D];
+    // LDS ring: NST tiles each of K and V (2 x 32 KiB per workgroup, two workgroups per CU).
+    constexpr int NST = 2;
+    constexpr int LA  = NST - 1;             // tiles of lookahead
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds[NST][kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds[NST][kBN * D];
 
-    // ---- which (batch, head, query block): heavy causal blocks first, and all
-    // query blocks of one head on one XCD so its K/V stay in that XCD's L2.
     const int nq = p.n_qblocks;
     const int BH = p.B * p.Hq;
     int bh, qi;
     {
         const int idx = blockIdx.x;
-        if (BH % 8 == 0) {
+        if (BH % 16 == 0) {
+            const int xcd = idx & 7, j = idx >> 3;
+            const int g = j / (2 * nq), r = j % (2 * nq);
+            bh = (2 * g + (r & 1)) * 8 + xcd;
+            qi = r >> 1;
+        } else if (BH % 8 == 0) {
             const int xcd = idx & 7, j = idx >> 3;
             bh = (j / nq) * 8 + xcd;
             qi = j % nq;
@@ -174,90 +191,99 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_fwd_kernel(const FlashP
     const int hkv = hq / (p.Hq / p.Hkv);
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps per-wave branches scalar
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lq = lane & 31, lh = lane >> 5;
-    const int q0 = qblock * kBM + wave * 32;  // first query of this wave
-    const int my_q = q0 + lq;
+    const int q0 = qblock * kBM + wave * WQ;   // first query of this wave; query block qb starts at q0 + 32 qb
 
-    // ---- Q^T operand: this lane's query row, 8 d-values per k-step.
-    i16x8 qreg[KSTEPS];
-    {
+    i16x8 qreg[QB][KSTEPS];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int my_q = q0 + 32 * qb + lq;
         const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
         const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks)
-            qreg[ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
+        for (int ks = 0; ks < KSTEPS; ++ks) qreg[qb][ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
     }
 
     const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
     const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
 
-    // Number of key tiles this workgroup needs.
     int n_tiles = (p.Lk + kBN - 1) / kBN;
     if (kCausal) {
-        const int last_q = min(qblock * kBM + kBM, p.Lq) - 1;  // keys 0..last_q
-        const int need = min(last_q + 1, p.Lk);
-        n_tiles = (need + kBN - 1) / kBN;
+        const int last_q = min(qblock * kBM + kBM, p.Lq) - 1;
+        n_tiles = (min(last_q + 1, p.Lk) + kBN - 1) / kBN;
     }
+    const int wave_tiles = kCausal ? min(n_tiles, (q0 + WQ - 1) / kBN + 1) : n_tiles;
 
-    // ---- tile staging.  Wave w, instruction i fills rows i*RPI*NW + w*RPI .. +RPI-1;
-    // RPI*NW is a multiple of 16, so a lane's swizzle (and its global offset
-    // apart from a uniform row step) is the same for every i.
-    const int srow = wave * RPI + lane / CHUNKS;     // row within the first group
+    // ---- staging: 64 LDS rows <- global rows first .. first+63 (rows outside [0, Lk) read as zero)
+    const int srow = wave * RPI + lane / CHUNKS;
     const int slot = lane % CHUNKS;
     const unsigned koff = static_cast<unsigned>(srow * p.ks_l + ((slot ^ ksw(srow)) * 8));
     const unsigned voff = static_cast<unsigned>(srow * p.vs_l + ((slot ^ vsw(srow)) * 8));
     typedef __attribute__((address_space(1))) const void* gptr_t;
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto stage_tile = [&](int t, int buf) {
-        const std::uint16_t* kt = kbase + static_cast<long>(t) * kBN * p.ks_l;
-        const std::uint16_t* vt = vbase + static_cast<long>(t) * kBN * p.vs_l;
-        if ((t + 1) * kBN <= p.Lk) {
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int r0 = i * RPI * NW;                      // uniform row step
-                __builtin_amdgcn_global_load_lds((gptr_t)(kt + static_cast<long>(r0) * p.ks_l + koff),
-                                                 (lptr_t)&k_lds[buf][(r0 + wave * RPI) * D], 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((gptr_t)(vt + static_cast<long>(r0) * p.vs_l + voff),
-                                                 (lptr_t)&v_lds[buf][(r0 + wave * RPI) * D], 16, 0, 0);
-            }
-        } else {  // last, partial tile: rows past the end of K/V read as zero
+    // Returns true when exactly NI direct loads per lane were issued (the count the
+    // partial wait in publish() relies on).
+    auto stage_rows = [&](const std::uint16_t* base, long stride, unsigned off, int first, std::uint16_t* tile) -> bool {
+        const std::uint16_t* src = base + static_cast<long>(first) * stride;   // only dereferenced for rows in range
+        if (first >= 0 && first + kBN <= p.Lk) {
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 const int r0 = i * RPI * NW;
-                std::uint16_t* kd = &k_lds[buf][(r0 + wave * RPI) * D];
-                std::uint16_t* vd = &v_lds[buf][(r0 + wave * RPI) * D];
-                if (t * kBN + r0 + srow < p.Lk) {
-                    __builtin_amdgcn_global_load_lds((gptr_t)(kt + static_cast<long>(r0) * p.ks_l + koff), (lptr_t)kd, 16, 0, 0);
-                    __builtin_amdgcn_global_load_lds((gptr_t)(vt + static_cast<long>(r0) * p.vs_l + voff), (lptr_t)vd, 16, 0, 0);
-                } else {
-                    *reinterpret_cast<u32x4*>(kd + lane * 8) = u32x4{0, 0, 0, 0};
-                    *reinterpret_cast<u32x4*>(vd + lane * 8) = u32x4{0, 0, 0, 0};
-                }
+                __builtin_amdgcn_global_load_lds((gptr_t)(src + static_cast<long>(r0) * stride + off),
+                                                 (lptr_t)(tile + (r0 + wave * RPI) * D), 16, 0, 0);
             }
+            return true;
+        } else {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int r0 = i * RPI * NW;
+                std::uint16_t* dst = tile + (r0 + wave * RPI) * D;
+                const int row = first + r0 + srow;
+                if (row >= 0 && row < p.Lk)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(src + static_cast<long>(r0) * stride + off), (lptr_t)dst, 16, 0, 0);
+                else
+                    *reinterpret_cast<u32x4*>(dst + lane * 8) = u32x4{0, 0, 0, 0};
+            }
+            return false;
         }
     };
-    // Direct loads land in LDS asynchronously: drain them before the barrier that publishes the tile.
-    auto publish = [&]() {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Requests K tile t+1 and V tile t (the pair tile t's successor blocks need).
+    auto stage_pair = [&](int t) -> bool {
+        const bool a = stage_rows(kbase, p.ks_l, koff, (t + 1) * kBN - 32, k_lds[(t + 1) % NST]);
+        const bool c = stage_rows(vbase, p.vs_l, voff, t * kBN, v_lds[t % NST]);
+        return a && c;
+    };
+    // Barrier that publishes every tile requested so far, except (newest_pending) the
+    // most recently requested pair, whose 2*NI loads per lane may stay in flight.
+    auto publish = [&](bool newest_pending) {
+        if (newest_pending) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI) : "memory");
+        else                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     };
+    // Start of tile t: request the pair LA tiles ahead; end of tile t: tiles up to t+1 must be in.
+    auto stage_ahead = [&](int t) -> bool { return t + LA < n_tiles ? stage_pair(t + LA) && LA == 2 : false; };
 
-    float16_t oacc[DBLK];
+    float16_t oacc[QB][DBLK];
+    float m_run[QB], l_run[QB];
 #pragma unroll
-    for (int i = 0; i < DBLK; ++i)
+    for (int qb = 0; qb < QB; ++qb) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-    float m_run = -INFINITY;  // running max of raw scores (before scaling)
-    float l_run = 0.f;        // this half-wave's share of the running sum
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[qb][i][r] = 0.f;
+    }
 
-    stage_tile(0, 0);
-    publish();
+    {
+        stage_rows(kbase, p.ks_l, koff, -32, k_lds[0]);   // K tile 0: keys 0..31 in its upper half
+        stage_pair(0);
+        bool pending = false;
+        if (LA == 2 && 1 < n_tiles) pending = stage_pair(1);
+        publish(pending);
+    }
 
-    // Per-lane LDS read offsets (elements).  K operand of k-step ks: row lq (+32 kb),
-    // chunk 2ks+lh; V^T operand of d-block db: row 4lh + m16/4 (+ 32kb + 16s2 [+8]),
-    // chunk 4db + 2(grp&1) + (m16&3)/2, 8-byte half (m16&1).  Row offsets that are
-    // multiples of 16 (K: 32) leave the swizzle unchanged, so they stay immediates.
     const int grp = lane >> 4, m16 = lane & 15;
     int k_rd[KSTEPS], v_rd[DBLK];
 #pragma unroll
@@ -268,144 +294,197 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void flash_fwd_kernel(const FlashP
         for (int db = 0; db < DBLK; ++db)
             v_rd[db] = vrow * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
     }
-
-    // Raise the running max only when a tile exceeds it by more than this much
-    // (raw score units): exp2((s - m) * scale_log2) then stays below 2^8.
     const float lazy_margin = 8.0f / p.scale_log2;
 
-    // Tiles this wave computes on: a causal tile that lies entirely above the
-    // wave's queries contributes nothing.  The wave still helps stage those tiles
-    // for the others (second loop below).
-    const int wave_tiles = kCausal ? min(n_tiles, (q0 + 31) / kBN + 1) : n_tiles;
-
-    for (int t = 0; t < wave_tiles; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < n_tiles) stage_tile(t + 1, buf ^ 1);
-        const int key0 = t * kBN;
-        {
-            // ---- S^T = K Q^T for the two 32-key blocks of the tile
-            float16_t sacc[2];
+    auto needs_mask = [&](int j, int qb) { return (kCausal && j * 32 + 31 > q0 + 32 * qb) || j * 32 + 32 > p.Lk; };
+    auto apply_mask = [&](int j, int qb, float16_t& sc) {
+        const int my_q = q0 + 32 * qb + lq;
+        const int last_visible = kCausal ? min(my_q, p.Lk - 1) : p.Lk - 1;
+        const int rel = last_visible - j * 32 - 4 * lh;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+        for (int r = 0; r < 16; ++r)
+            if ((r >> 2) * 8 + (r & 3) > rel) sc[r] = -INFINITY;
+    };
+    auto lane_max = [](const float16_t& sc) {
+        float mx = sc[0];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+        return mx;
+    };
+    // Raise the running max of query block qb if block max `mx` (this lane's half) needs it.
+    auto raise_max = [&](float (&mx)[QB]) {
+        bool grow = false;
+        float mloc[QB];
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const i16x8 a = *reinterpret_cast<const i16x8*>(&k_lds[buf][k_rd[ks] + kb * 32 * D]);
-                    sacc[kb] = Mma<T>::run(a, qreg[ks], sacc[kb]);
-                }
-            }
-
-            // ---- masking (only tiles that touch the diagonal or the end of K):
-            // element (kb, r) sits at key offset kb*32 + (r/4)*8 + r%4 from this lane's
-            // first key; it is dead when that offset exceeds `rel`.
-            const bool need_mask = (kCausal && key0 + kBN - 1 > q0) || (key0 + kBN > p.Lk);
-            if (need_mask) {
-                const int last_visible = kCausal ? min(my_q, p.Lk - 1) : p.Lk - 1;
-                const int rel = last_visible - key0 - 4 * lh;
+        for (int qb = 0; qb < QB; ++qb) {
+            mloc[qb] = half_swap_max(mx[qb]);
+            grow = grow || (mloc[qb] > m_run[qb] + lazy_margin);
+        }
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // wave-uniform, rare after block 0
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (kb * 32 + (r >> 2) * 8 + (r & 3) > rel) sacc[kb][r] = -INFINITY;
-            }
-
-            // ---- online softmax with a lazily raised running max
-            float mloc = sacc[0][0];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
-            mloc = half_swap_max(mloc);
-            if (__builtin_amdgcn_ballot_w64(mloc > m_run + lazy_margin) != 0) {  // wave-uniform
-                const float m_new = fmaxf(m_run, mloc);
-                const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2);
-                m_run = m_new;
-                l_run *= alpha;
+            for (int qb = 0; qb < QB; ++qb) {
+                const float m_new = fmaxf(m_run[qb], mloc[qb]);
+                const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.scale_log2);
+                m_run[qb] = m_new;
+                l_run[qb] *= alpha;
 #pragma unroll
                 for (int i = 0; i < DBLK; ++i)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) oacc[qb][i][r] *= alpha;
             }
-            const float mc = m_run * p.scale_log2;
+        }
+    };
+    // Mask where needed, then raise.  `mx` holds the unmasked in-lane maxima on entry.
+    auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB]) {
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb)
+            if (needs_mask(j, qb)) {
+                apply_mask(j, qb, sc[qb]);
+                mx[qb] = lane_max(sc[qb]);
+            }
+        raise_max(mx);
+    };
 
-            // ---- P^T as MFMA B operands (two k-steps of 16 keys per 32-key block)
-            i16x8 pb[2][2];
+    // One block: exponentials of `cur` = S(j) and, if kNext, the MFMAs of S(j+1) into `nxt`,
+    // then PV(j).  The MFMA part is a fixed schedule of KSTEPS + 2*DBLK slots (QB MFMAs per
+    // slot, sharing one LDS fragment), fenced so that the compiler keeps the order: fragment
+    // reads run two slots ahead (three rotating fragment registers) and the 8*QB exp pairs
+    // (2 fma + 2 exp + cvt + dot2 each) are spread between the MFMAs so the matrix pipe has
+    // an instruction in flight while the VALU works.  P(s2=0) is complete before the first
+    // PV MFMA, P(s2=1) before the first PV MFMA that uses it; the in-lane row maxima of
+    // S(j+1) are taken in the last slots.
+    auto block = [&](int j, float16_t (&cur)[QB], float16_t (&nxt)[QB], auto next_tag) {
+        constexpr bool kNext = decltype(next_tag)::value;
+        constexpr int S0 = kNext ? 0 : KSTEPS;           // first slot that exists
+        constexpr int NS = KSTEPS + 2 * DBLK;            // slot c >= KSTEPS: PV(s2 = (c-KSTEPS)/DBLK, db = (c-KSTEPS)%DBLK)
+        float mc[QB];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+        for (int qb = 0; qb < QB; ++qb) mc[qb] = m_run[qb] * p.scale_log2;
+        const std::uint16_t* kt = &k_lds[((j + 2) >> 1) % NST][((j + 2) & 1) * 32 * D];   // rows of block j+1
+        const std::uint16_t* vt = &v_lds[(j >> 1) % NST][(j & 1) * 32 * D];
+        i16x8 frag[3];
+        u32x4 pw[QB][2];
+        float mx[QB];
+        auto fetch = [&](int c) {                         // operand of slot c -> frag[c % 3]
+            if (c < KSTEPS) {
+                frag[c % 3] = *reinterpret_cast<const i16x8*>(kt + k_rd[c]);
+            } else {
+                const int s2 = (c - KSTEPS) / DBLK, db = (c - KSTEPS) % DBLK;
+                const std::uint16_t* vp = vt + v_rd[db] + 16 * s2 * D;
+                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
+                frag[c % 3] = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+        };
+        auto exp_pair = [&](int qb, int i) {              // elements 2i, 2i+1 of cur[qb]
+            const float e0 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i], p.scale_log2, -mc[qb]));
+            const float e1 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i + 1], p.scale_log2, -mc[qb]));
+            const std::uint32_t w = Mma<T>::pack2(e0, e1);
+            l_run[qb] = Mma<T>::add_pair(w, l_run[qb]);
+            pw[qb][i / 4][i % 4] = w;
+        };
+        // pair (qb, i) is issued just before the MFMAs of slot pair_slot(qb, i)
+        auto pair_slot = [](int qb, int i) {
+            if (i < 4) return kNext ? (qb * 4 + i) * KSTEPS / (4 * QB) : KSTEPS;
+            return KSTEPS + (qb * 4 + i - 4) * DBLK / (4 * QB);
+        };
+
+        fetch(S0);
+        fetch(S0 + 1);
 #pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
-                    u32x4 w;
+        for (int c = S0; c < NS; ++c) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float e0 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][8 * s2 + 2 * e], p.scale_log2, -mc));
-                        const float e1 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][8 * s2 + 2 * e + 1], p.scale_log2, -mc));
-                        w[e] = Mma<T>::pack2(e0, e1);
-                        l_run = Mma<T>::add_pair(w[e], l_run);
+            for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (pair_slot(qb, i) == c) exp_pair(qb, i);
+            if (c < KSTEPS) {
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                    if (c == 0) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) nxt[qb][r] = 0.f;
                     }
-                    pb[kb][s2] = __builtin_bit_cast(i16x8, w);
+                    nxt[qb] = Mma<T>::run(frag[c % 3], qreg[qb][c], nxt[qb]);
                 }
+            } else {
+                const int s2 = (c - KSTEPS) / DBLK, db = (c - KSTEPS) % DBLK;
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb)
+                    oacc[qb][db] = Mma<T>::run(frag[c % 3], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
+            }
+            if (c + 2 < NS) fetch(c + 2);
+            if (kNext && c >= NS - QB) mx[c - (NS - QB)] = lane_max(nxt[c - (NS - QB)]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (kNext) finish_scores(j + 1, nxt, mx);
+    };
+    using Yes = std::true_type;
+    using No  = std::false_type;
 
-            // ---- O^T += V^T P^T
+    float16_t s_a[QB], s_b[QB];
+    if (wave_tiles > 0) {
+        // S(0): keys 0..31 = rows 32..63 of K tile 0
+        float mx[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_a[qb][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks)
+                s_a[qb] = Mma<T>::run(*reinterpret_cast<const i16x8*>(&k_lds[0][32 * D + k_rd[ks]]), qreg[qb][ks], s_a[qb]);
+            mx[qb] = lane_max(s_a[qb]);
+        }
+        finish_scores(0, s_a, mx);
+    }
+    for (int t = 0; t + 1 < wave_tiles; ++t) {
+        const bool pending = stage_ahead(t);
+        block(2 * t, s_a, s_b, Yes{});
+        block(2 * t + 1, s_b, s_a, Yes{});
+        publish(pending);
+    }
+    if (wave_tiles > 0) {  // the wave's last tile: nothing to compute ahead in its second block
+        const int t = wave_tiles - 1;
+        const bool pending = stage_ahead(t);
+        block(2 * t, s_a, s_b, Yes{});
+        block(2 * t + 1, s_b, s_a, No{});
+        publish(pending);
+    }
+    for (int t = wave_tiles; t < n_tiles; ++t) publish(stage_ahead(t));
+
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int my_q = q0 + 32 * qb + lq;
+        const float l_tot = half_swap_sum(l_run[qb]);
+        const float inv_l = 1.0f / l_tot;
+        if (my_q < p.Lq) {
+            std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
 #pragma unroll
             for (int db = 0; db < DBLK; ++db)
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int s2 = 0; s2 < 2; ++s2) {
-                        const std::uint16_t* vp = &v_lds[buf][v_rd[db] + (kb * 32 + 16 * s2) * D];
-                        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
-                        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
-                        const i16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        oacc[db] = Mma<T>::run(a, pb[kb][s2], oacc[db]);
-                    }
+                for (int g = 0; g < 4; ++g) {
+                    const int d = db * 32 + g * 8 + 4 * lh;
+                    u32x2 w;
+                    w[0] = Mma<T>::pack2(oacc[qb][db][4 * g + 0] * inv_l, oacc[qb][db][4 * g + 1] * inv_l);
+                    w[1] = Mma<T>::pack2(oacc[qb][db][4 * g + 2] * inv_l, oacc[qb][db][4 * g + 3] * inv_l);
+                    *reinterpret_cast<u32x2*>(op + d) = w;
+                }
+            if (p.lse != nullptr && lh == 0)
+                p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run[qb] * p.scale + logf(l_tot);
         }
-
-        // ---- publish the next tile
-        publish();
     }
-    for (int t = wave_tiles; t < n_tiles; ++t) {
-        if (t + 1 < n_tiles) stage_tile(t + 1, (t & 1) ^ 1);
-        publish();
-    }
-
-    // ---- epilogue: normalise and store O[q][d]; lane holds 4 consecutive d per (db, r/4)
-    const float l_tot = half_swap_sum(l_run);
-    const float inv_l = 1.0f / l_tot;
-    if (my_q < p.Lq) {
-        std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
-#pragma unroll
-        for (int db = 0; db < DBLK; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int d = db * 32 + g * 8 + 4 * lh;
-                u32x2 w;
-                w[0] = Mma<T>::pack2(oacc[db][4 * g + 0] * inv_l, oacc[db][4 * g + 1] * inv_l);
-                w[1] = Mma<T>::pack2(oacc[db][4 * g + 2] * inv_l, oacc[db][4 * g + 3] * inv_l);
-                *reinterpret_cast<u32x2*>(op + d) = w;
-            }
-        if (p.lse != nullptr && lh == 0)
-            p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run * p.scale + logf(l_tot);
-    }
-}
-
-template <typename T, int D, int NW>
-int launch_nw(FlashParams p, bool causal, hipStream_t s) {
-    p.n_qblocks = (p.Lq + NW * 32 - 1) / (NW * 32);
-    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
-    if (causal)
-        hipLaunchKernelGGL((flash_fwd_kernel<T, D, true, NW>), dim3(static_cast<unsigned>(blocks)), dim3(NW * 64), 0, s, p);
-    else
-        hipLaunchKernelGGL((flash_fwd_kernel<T, D, false, NW>), dim3(static_cast<unsigned>(blocks)), dim3(NW * 64), 0, s, p);
-    PARAS_HIP_TRY(hipGetLastError());
-    return PARAS_OK;
 }
 
 template <typename T, int D>
-int launch_t(const FlashParams& p, bool causal, hipStream_t s) {
-    // 4 waves (128 queries) per workgroup: 8 waves sharing each tile halve the L2 -> LDS
-    // traffic but measured 9 % slower (more waves idle at each barrier and on the causal diagonal).
-    return launch_nw<T, D, 4>(p, causal, s);
+int launch_t(FlashParams p, bool causal, hipStream_t s) {
+    p.n_qblocks = (p.Lq + kBM - 1) / kBM;
+    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
+    if (causal)
+        hipLaunchKernelGGL((flash_fwd_kernel<T, D, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, p);
+    else
+        hipLaunchKernelGGL((flash_fwd_kernel<T, D, false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, p);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -421,7 +500,7 @@ bool flash_supported(const paras_sdpa_args& a) {
     if (!(a.scale > 0.0) || !std::isfinite(a.scale)) return false;  // the running max is taken on raw scores
     if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.out)) return false;
     if (!mult8(a.q_strides) || !mult8(a.k_strides) || !mult8(a.v_strides)) return false;
-    const int64_t nq = (a.Lq + 127) / 128;
+    const int64_t nq = (a.Lq + kBM - 1) / kBM;
     if (a.B * a.Hq * nq > 0x7fffffffLL || a.Lq > 0x3fffffff || a.Lk > 0x3fffffff) return false;
     return true;
 }
