@@ -89,7 +89,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe", "copy"],
+                    choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe", "linear", "copy"],
                     help="'copy' is the counter calibration: a plain 1 GiB device copy, not part of 'all'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     args = ap.parse_args()
@@ -244,6 +244,24 @@ def main() -> int:
         log(f"moe: route {ms_route * 1e3:.1f} us, ffn {ms_ffn * 1e3:.1f} us = {tf:.1f} TFLOP/s ({tf / MFMA_BF16_PEAK_TFLOPS:.1%}), "
             f"layer {ms_all * 1e3:.1f} us = {T / ms_all * 1e3:.0f} tokens/s")
         del x, wg, wu, wd, fws, out
+
+    # ------------------------------------------------------------------ dense projection (the callers either side of the path)
+    if want("linear"):
+        M, N, K = 16384, 4096, 4096               # 4 x 4096 tokens through a hidden x hidden nn.Linear
+        xa = torch.randn(M, K, device=dev).to(bf)
+        wb = (0.02 * torch.randn(N, K, device=dev)).to(bf)
+        yc = torch.empty(M, N, dtype=bf, device=dev)
+        ms, _ = timer.run(lambda i: must(L.paras_gemm_nt(xa.data_ptr(), wb.data_ptr(), None, yc.data_ptr(), M, N, K, K, K, N, 0,
+                                                         1, 0, 0, 0, 0, 1.0, 0.0, capi.BF16, st)), steps, warmup)
+        flops = 2 * M * N * K
+        tf = flops / ms / 1e9
+        results["linear"] = {
+            "workload": "bf16 dense NT GEMM x W^T: M=16384 N=4096 K=4096 (nn.Linear of configs[2]'s tokens)",
+            "value": round(tf, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "kernel": "dense_gemm_nt_kernel<bf16>",
+            "algorithmic_flops_per_launch": flops, "roofline": roofline("mfma", tf, "dense_gemm_nt_kernel"),
+        }
+        log(f"linear: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s ({tf / MFMA_BF16_PEAK_TFLOPS:.1%})")
+        del xa, wb, yc
 
     # ------------------------------------------------------------------ counter calibration
     if args.workload == "copy":

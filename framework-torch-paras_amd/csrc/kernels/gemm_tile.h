@@ -1,0 +1,124 @@
+// Tile mainloop shared by the MFMA GEMM kernels (grouped expert GEMMs and the
+// dense NT GEMM): C tile = A[128 x K] * B[256 x K]^T with bf16/fp16 operands and
+// fp32 accumulation on v_mfma_f32_32x32x16.
+//
+// Both operands are read along their contiguous contraction dim, which is the
+// 8-element-per-lane operand layout of the MFMA, so neither needs a transpose.
+// Workgroup = 4 waves arranged 2x2; the 256 B rows come as two groups of 128
+// (gate / up weights, or two adjacent column blocks) and each wave owns 64x64
+// of each group: 128 fp32 accumulators per lane.  k-tile 64, global ->
+// registers -> LDS with the next k-tile's loads in flight during the MFMAs.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "core/device_math.h"
+
+namespace paras {
+namespace gemm {
+
+constexpr int kThreads = 256;
+constexpr int kBM = 128;
+constexpr int kBN = 128;          // columns per group; a workgroup computes two groups
+constexpr int kBK = 64;
+constexpr int kLS = kBK + 8;      // LDS row stride (elements): 16 consecutive rows hit distinct banks
+
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+
+template <typename T> struct MmaT;
+template <> struct MmaT<bf16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct MmaT<f16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+
+struct TileLds {
+    std::uint16_t a[kBM * kLS];
+    std::uint16_t b[2][kBN * kLS];
+};
+
+// a_ptr[i] / b_ptr[g][i]: this thread's four 16-byte chunks per operand row set
+// (chunk c = tid + i*256 -> tile row c/8, column (c%8)*8), already offset to k = 0.
+// Accumulates into acc[g][mi][ni]; lane (column lr = lane%32, half lh = lane/32) of
+// block (mi, ni) ends up holding rows (r/4)*8 + 4*lh + r%4, r = 0..15.
+template <typename T>
+__device__ __forceinline__ void tile_mainloop(const std::uint16_t* const (&a_ptr)[4], const std::uint16_t* const (&b_ptr)[2][4],
+                                              long K, TileLds& lds, float16_t (&acc)[2][2][2]) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lh = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    std::uint16_t* a_lds = lds.a;
+    std::uint16_t (*b_lds)[kBN * kLS] = lds.b;
+    u32x4 a_st[4], b_st[2][4];
+    auto load_tile = [&](long k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_ptr[i] + k0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_ptr[g][i] + k0);
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * kThreads;
+            const int off = (c >> 3) * kLS + (c & 7) * 8;
+            *reinterpret_cast<u32x4*>(&a_lds[off]) = a_st[i];
+            *reinterpret_cast<u32x4*>(&b_lds[0][off]) = b_st[0][i];
+            *reinterpret_cast<u32x4*>(&b_lds[1][off]) = b_st[1][i];
+        }
+    };
+
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[g][mi][ni][r] = 0.f;
+
+    const int a_off = (wm * 64 + lr) * kLS + lh * 8;
+    const int b_off = (wn * 64 + lr) * kLS + lh * 8;
+    const long k_tiles = K / kBK;
+    load_tile(0);
+    store_tile();
+    __syncthreads();
+    for (long kt = 0; kt < k_tiles; ++kt) {
+        if (kt + 1 < k_tiles) load_tile((kt + 1) * kBK);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            i16x8 af[2], bf[2][2];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+                af[mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off + mi * 32 * kLS + ks * 16]);
+#pragma unroll
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    bf[g][ni] = *reinterpret_cast<const i16x8*>(&b_lds[g][b_off + ni * 32 * kLS + ks * 16]);
+#pragma unroll
+            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ++ni)
+                        acc[g][mi][ni] = MmaT<T>::run(af[mi], bf[g][ni], acc[g][mi][ni]);
+        }
+        __syncthreads();
+        if (kt + 1 < k_tiles) {
+            store_tile();
+            __syncthreads();
+        }
+    }
+
+}
+
+}  // namespace gemm
+}  // namespace paras

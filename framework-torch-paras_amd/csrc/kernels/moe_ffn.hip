@@ -28,18 +28,13 @@
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
+#include "kernels/gemm_tile.h"
 #include "kernels/swiglu_math.h"
 
 namespace paras {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kBM = 128;
-constexpr int kBN = 128;          // columns per group; a workgroup computes two groups
-constexpr int kBK = 64;
-constexpr int kLS = kBK + 8;      // LDS row stride (elements): 16 consecutive rows hit distinct banks
-
-typedef short i16x8 __attribute__((ext_vector_type(8)));
+using namespace gemm;
 
 struct FfnGemmParams {
     const std::uint16_t* a;     // x [T, K] (gathered) or h [R, K]
@@ -55,23 +50,10 @@ struct FfnGemmParams {
     int ngt;                    // column units an XCD sweeps together
 };
 
-template <typename T> struct MmaT;
-template <> struct MmaT<bf16_t> {
-    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-};
-template <> struct MmaT<f16_t> {
-    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-};
-
 template <typename T, bool kSwiglu>
 __global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemmParams p) {
     using El = Elem<T>;
-    __shared__ __attribute__((aligned(16))) std::uint16_t a_lds[kBM * kLS];
-    __shared__ __attribute__((aligned(16))) std::uint16_t b_lds[2][kBN * kLS];
+    __shared__ __attribute__((aligned(16))) TileLds lds;
 
     // ---- tile coordinates.  Linear id L: xcd = L % 8 (hardware round-robin);
     // within an XCD walk (column group, m-tile, column-in-group).
@@ -132,69 +114,8 @@ __global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemm
             const std::uint16_t* base = g == 0 ? p.b : p.b2;
             b_ptr[g][i] = base + (static_cast<long>(e) * p.Nw + wrow) * p.K + (c & 7) * 8;
         }
-    u32x4 a_st[4], b_st[2][4];
-    auto load_tile = [&](long k0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_ptr[i] + k0);
-#pragma unroll
-        for (int g = 0; g < 2; ++g)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_ptr[g][i] + k0);
-    };
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + i * kThreads;
-            const int off = (c >> 3) * kLS + (c & 7) * 8;
-            *reinterpret_cast<u32x4*>(&a_lds[off]) = a_st[i];
-            *reinterpret_cast<u32x4*>(&b_lds[0][off]) = b_st[0][i];
-            *reinterpret_cast<u32x4*>(&b_lds[1][off]) = b_st[1][i];
-        }
-    };
-
     float16_t acc[2][2][2];
-#pragma unroll
-    for (int g = 0; g < 2; ++g)
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[g][mi][ni][r] = 0.f;
-
-    const int a_off = (wm * 64 + lr) * kLS + lh * 8;
-    const int b_off = (wn * 64 + lr) * kLS + lh * 8;
-    const long k_tiles = p.K / kBK;
-    load_tile(0);
-    store_tile();
-    __syncthreads();
-    for (long kt = 0; kt < k_tiles; ++kt) {
-        if (kt + 1 < k_tiles) load_tile((kt + 1) * kBK);
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            i16x8 af[2], bf[2][2];
-#pragma unroll
-            for (int mi = 0; mi < 2; ++mi)
-                af[mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off + mi * 32 * kLS + ks * 16]);
-#pragma unroll
-            for (int g = 0; g < 2; ++g)
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    bf[g][ni] = *reinterpret_cast<const i16x8*>(&b_lds[g][b_off + ni * 32 * kLS + ks * 16]);
-#pragma unroll
-            for (int g = 0; g < 2; ++g)
-#pragma unroll
-                for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        acc[g][mi][ni] = MmaT<T>::run(af[mi], bf[g][ni], acc[g][mi][ni]);
-        }
-        __syncthreads();
-        if (kt + 1 < k_tiles) {
-            store_tile();
-            __syncthreads();
-        }
-    }
+    tile_mainloop<T>(a_ptr, b_ptr, p.K, lds, acc);
 
     // ---- epilogue.  Accumulator lane (column lr, half lh) holds rows (r/4)*8 + 4*lh + r%4.
 #pragma unroll

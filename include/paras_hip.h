@@ -270,6 +270,25 @@ PARAS_API int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up,
                             void* out, void* workspace, int64_t T, int64_t E, int64_t k,
                             int64_t H, int64_t I, int dtype, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* Dense NT GEMM (replaces the host bounce of mm / bmm / addmm / linear,       */
+/* csrc/ops/vision_ops.cpp:248-309 (LinearFunction), :388-423 (mm_out,         */
+/* bmm_out, addmm_out): copy to CPU, ATen GEMM with fp32 accumulation and one  */
+/* rounding, copy back).  Per batch b:                                         */
+/*   C[b] = T( alpha * A[b] B[b]^T + beta * addend[b] )                        */
+/* A [M, K] rows lda apart, B [N, K] rows ldb apart (both contiguous along K:  */
+/* x W^T of nn.Linear, q k^T), C [M, N] rows ldc apart; batch strides in       */
+/* elements (0 = shared).  addend may be NULL; ld_add = 0 broadcasts one row   */
+/* (a bias) over the M rows.  bf16 / f16 on MFMA; K must be a multiple of 64   */
+/* and operand rows 16-byte aligned (PARAS_ERR_UNSUPPORTED otherwise: the      */
+/* caller keeps its host path for those).                                      */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c,
+                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                            int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
+                            int64_t stride_b, int64_t stride_c, int64_t stride_add,
+                            double alpha, double beta, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -62,6 +62,7 @@ SIGNATURES = {
     "paras_moe_route": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp]),
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
+    "paras_gemm_nt": (i32, [vp, vp, vp, vp] + [i64] * 12 + [f64, f64, i32, vp]),
 }
 
 _lib = None
@@ -218,3 +219,25 @@ def moe_ffn(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, k, workspa
                               _ptr(inv_order), _ptr(offsets), _ptr(out), _ptr(workspace), T, E, k, H, I,
                               DT[x.dtype], _stream()))
     return out
+
+
+def gemm_nt(a, b, addend=None, alpha=1.0, beta=1.0):
+    """C = alpha * a @ b^T (+ beta * addend); a [.., M, K], b [.., N, K] (2-D or batched 3-D,
+    last dim contiguous); addend [N] (bias), [M, N] or [B, M, N]."""
+    batched = a.dim() == 3
+    B = a.shape[0] if batched else 1
+    M, K = a.shape[-2:]
+    N = b.shape[-2]
+    c = torch.empty((B, M, N) if batched else (M, N), dtype=a.dtype, device=a.device)
+    sa = a.stride(0) if batched else 0
+    sb = b.stride(0) if (batched and b.dim() == 3) else 0
+    ld_add = sadd = 0
+    if addend is not None:
+        if addend.dim() >= 2:
+            ld_add = addend.stride(-2)
+        if addend.dim() == 3:
+            sadd = addend.stride(0)
+    check(lib().paras_gemm_nt(_ptr(a), _ptr(b), _ptr(addend) if addend is not None else None, _ptr(c), M, N, K,
+                              a.stride(-2), b.stride(-2), N, ld_add, B, sa, sb, M * N, sadd, alpha, beta,
+                              DT[a.dtype], _stream()))
+    return c

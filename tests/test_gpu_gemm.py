@@ -1,0 +1,96 @@
+"""Dense NT GEMM (mm / bmm / addmm / linear on the device) through the C ABI.
+
+The reference runs these on ATen-CPU with fp32 accumulation and one rounding
+(csrc/ops/vision_ops.cpp:248-309,388-423); the oracle's matmul_nt accumulates
+in double and rounds once.  Bar: every element within one 16-bit ulp of the
+oracle (summation order is the only difference), and torch-CPU addmm / linear
+as the library check for the epilogue.
+"""
+import pytest
+import torch
+
+import capi
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def ulp16(ref, dtype):
+    mant = 7 if dtype == torch.bfloat16 else 10
+    a = ref.double().abs().clamp_min(2.0 ** -14)
+    return torch.exp2(torch.floor(torch.log2(a)) - mant)
+
+
+def assert_gemm_close(out, ref, dtype):
+    err = (out.double().cpu() - ref.double()).abs()
+    tol = ulp16(ref, dtype) * 1.001 + 1e-6
+    assert bool((err <= tol).all()), f"worst {err.max().item():.3e}, {(err > tol).sum().item()} beyond one ulp"
+
+
+SHAPES = [(128, 256, 64), (1, 8, 64), (130, 257, 128), (300, 100, 192), (512, 1024, 1024), (77, 4096, 320)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_gemm_nt_matches_oracle(shape, dtype):
+    M, N, K = shape
+    torch.manual_seed(M * 7 + N * 3 + K)
+    a, b = torch.randn(M, K).to(dtype), (0.1 * torch.randn(N, K)).to(dtype)
+    out = capi.gemm_nt(a.cuda(), b.cuda())
+    assert_gemm_close(out, O.matmul_nt(a, b), dtype)
+
+
+def test_gemm_nt_bias_and_addmm_epilogue():
+    torch.manual_seed(1)
+    M, N, K = 200, 384, 256
+    dt = torch.bfloat16
+    a, w, bias = torch.randn(M, K).to(dt), (0.05 * torch.randn(N, K)).to(dt), torch.randn(N).to(dt)
+    out = capi.gemm_nt(a.cuda(), w.cuda(), bias.cuda())
+    assert_gemm_close(out, torch.nn.functional.linear(a, w, bias), dt)        # library check: x W^T + b
+    self_ = torch.randn(M, N).to(dt)
+    out = capi.gemm_nt(a.cuda(), w.cuda(), self_.cuda(), alpha=0.5, beta=2.0)
+    exact = 0.5 * (a.double() @ w.double().t()) + 2.0 * self_.double()
+    assert_gemm_close(out, exact.to(dt), dt)
+    assert_gemm_close(out, torch.addmm(self_, a, w.t(), beta=2.0, alpha=0.5), dt)
+
+
+def test_gemm_nt_batched_strided_and_shared_operand():
+    torch.manual_seed(2)
+    B, M, N, K = 3, 96, 160, 128
+    dt = torch.float16
+    a = torch.randn(B, M, K + 8).to(dt)
+    b = (0.1 * torch.randn(B, N, K)).to(dt)
+    ad, bd = a.cuda()[:, :, :K], b.cuda()                           # rows 16-byte aligned, not dense
+    a = a[:, :, :K]
+    assert not ad.is_contiguous()
+    out = capi.gemm_nt(ad, bd)
+    for i in range(B):
+        assert_gemm_close(out[i], O.matmul_nt(a[i].contiguous(), b[i]), dt)
+    out = capi.gemm_nt(ad, bd[0])                                   # one weight matrix for the whole batch
+    for i in range(B):
+        assert_gemm_close(out[i], O.matmul_nt(a[i].contiguous(), b[0]), dt)
+
+
+def test_gemm_nt_errors_and_empty():
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(capi.ParasError, match="multiple of 64"):
+        capi.gemm_nt(z(8, 72), z(8, 72))
+    with pytest.raises(capi.ParasError, match="bf16 or f16"):
+        capi.gemm_nt(torch.zeros(8, 64, device="cuda"), torch.zeros(8, 64, device="cuda"))
+    assert capi.gemm_nt(z(0, 64), z(8, 64)).shape == (0, 8)
+
+
+def test_gemm_nt_linearity_at_projection_size():
+    """Size-independent property at a transformer projection shape: (2 a) W^T == 2 (a W^T) bit for
+    bit, since scaling by a power of two commutes with every rounding; plus sampled rows vs the oracle."""
+    torch.manual_seed(3)
+    M, N, K = 4096, 4096, 4096
+    dt = torch.bfloat16
+    a1 = torch.randn(M, K, device="cuda").to(dt)
+    a2 = a1 * 2                                                     # exact: a power of two
+    w = (0.02 * torch.randn(N, K, device="cuda")).to(dt)
+    y1, y2 = capi.gemm_nt(a1, w), capi.gemm_nt(a2, w)
+    assert torch.equal(y2, y1 * 2)                                  # scaling by 2 commutes with every rounding
+    rows = torch.randint(0, M, (8,))
+    ref = O.matmul_nt(a1[rows].cpu(), w.cpu())
+    assert_gemm_close(y1[rows], ref, dt)

@@ -301,3 +301,53 @@ def test_threads_dispatch_concurrently(device):
     [t.start() for t in ts]
     [t.join() for t in ts]
     assert not errs, errs
+
+
+# ---- GEMM on the device (reference: host bounce, csrc/ops/vision_ops.cpp:248-309,388-423;
+# its tests compare with torch-CPU, tests/test_matmul_sort_creation_ops.py:28-98) --------
+def _one_ulp(actual, expected, dtype):
+    mant = 7 if dtype == torch.bfloat16 else 10
+    e = expected.double()
+    tol = torch.exp2(torch.floor(torch.log2(e.abs().clamp_min(2.0 ** -14))) - mant) * 1.001 + 1e-6
+    err = (actual.cpu().double() - e).abs()
+    assert bool((err <= tol).all()), f"worst {err.max().item():.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_linear_mm_bmm_addmm_on_device(device, dtype):
+    torch.manual_seed(0)
+    x, w, b = torch.randn(6, 50, 256).to(dtype), (0.05 * torch.randn(384, 256)).to(dtype), torch.randn(384).to(dtype)
+    xd, wd, bd = x.to(device), w.to(device), b.to(device)
+    _one_ulp(F.linear(xd, wd, bd), F.linear(x, w, b), dtype)                  # nn.Linear: weight used in place as w.t()
+    _one_ulp(F.linear(xd, wd), F.linear(x, w), dtype)
+    m1, m2 = torch.randn(70, 128).to(dtype), (0.1 * torch.randn(128, 200)).to(dtype)
+    _one_ulp(torch.mm(m1.to(device), m2.to(device)), torch.mm(m1, m2), dtype)  # row-major mat2: one transposing copy
+    s = torch.randn(70, 200).to(dtype)
+    _one_ulp(torch.addmm(s.to(device), m1.to(device), m2.to(device), beta=0.5, alpha=2.0),
+             torch.addmm(s, m1, m2, beta=0.5, alpha=2.0), dtype)
+    a3, b3 = torch.randn(4, 33, 64).to(dtype), (0.1 * torch.randn(4, 64, 48)).to(dtype)
+    _one_ulp(torch.bmm(a3.to(device), b3.to(device)), torch.bmm(a3, b3), dtype)
+    q, k = torch.randn(2, 3, 40, 64).to(dtype), torch.randn(2, 3, 24, 64).to(dtype)
+    _one_ulp(torch.matmul(q.to(device), k.to(device).transpose(-1, -2)), torch.matmul(q, k.transpose(-1, -2)), dtype)
+
+
+def test_gemm_other_dtypes_and_shapes_take_the_host_route(device):
+    torch.manual_seed(1)
+    a, b = torch.randn(17, 30), torch.randn(30, 9)
+    assert_close(torch.mm(a.to(device), b.to(device)), torch.mm(a, b), "fp32 mm")          # reference tolerance
+    a16, b16 = torch.randn(8, 24).bfloat16(), torch.randn(24, 8).bfloat16()                 # K not a multiple of 64
+    assert_bit_exact(torch.mm(a16.to(device), b16.to(device)), torch.mm(a16, b16), "bf16 mm, host route")
+    with pytest.raises(RuntimeError):
+        torch.mm(a.to(device), torch.randn(31, 9).to(device))
+
+
+def test_linear_backward_through_device_gemm(device):
+    torch.manual_seed(2)
+    x, w = torch.randn(32, 128).bfloat16(), (0.1 * torch.randn(64, 128)).bfloat16()
+    xd, wd = x.to(device).requires_grad_(), w.to(device).requires_grad_()
+    xc, wc = x.clone().requires_grad_(), w.clone().requires_grad_()
+    F.linear(xd, wd).float().pow(2).sum().backward()
+    F.linear(xc, wc).float().pow(2).sum().backward()
+    for got, want in ((xd.grad, xc.grad), (wd.grad, wc.grad)):
+        err = (got.cpu().float() - want.float()).abs().max().item()
+        assert err <= 0.02 * want.float().abs().max().item() + 1e-3, err
