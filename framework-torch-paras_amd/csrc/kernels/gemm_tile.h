@@ -92,24 +92,35 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* const (&a_ptr
     __syncthreads();
     for (long kt = 0; kt < k_tiles; ++kt) {
         if (kt + 1 < k_tiles) load_tile((kt + 1) * kBK);
-#pragma unroll
-        for (int ks = 0; ks < kBK / 16; ++ks) {
-            i16x8 af[2], bf[2][2];
+        // Fixed issue order, fenced slot by slot: one MFMA per slot, the fragments of the next
+        // k-step requested while the current one computes (A into a second register pair right
+        // away, each B fragment back into its own registers as soon as its two MFMAs have
+        // issued), so an operand is asked for about six MFMAs before it is used.
+        i16x8 af[2][2], bf[4];
+        auto read_a = [&](int buf, int ks) {
 #pragma unroll
             for (int mi = 0; mi < 2; ++mi)
-                af[mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off + mi * 32 * kLS + ks * 16]);
+                af[buf][mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off + mi * 32 * kLS + ks * 16]);
+        };
+        auto read_b = [&](int q, int ks) {   // q = 2*g + ni
+            bf[q] = *reinterpret_cast<const i16x8*>(&b_lds[q >> 1][b_off + (q & 1) * 32 * kLS + ks * 16]);
+        };
+        read_a(0, 0);
 #pragma unroll
-            for (int g = 0; g < 2; ++g)
+        for (int q = 0; q < 4; ++q) read_b(q, 0);
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    bf[g][ni] = *reinterpret_cast<const i16x8*>(&b_lds[g][b_off + ni * 32 * kLS + ks * 16]);
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            const int cur = ks & 1;
+            const bool more = ks + 1 < kBK / 16;
 #pragma unroll
-            for (int g = 0; g < 2; ++g)
+            for (int q = 0; q < 4; ++q)
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        acc[g][mi][ni] = MmaT<T>::run(af[mi], bf[g][ni], acc[g][mi][ni]);
+                for (int mi = 0; mi < 2; ++mi) {
+                    acc[q >> 1][mi][q & 1] = MmaT<T>::run(af[cur][mi], bf[q], acc[q >> 1][mi][q & 1]);
+                    if (more && q == 0 && mi == 0) read_a(cur ^ 1, ks + 1);
+                    if (more && mi == 1) read_b(q, ks + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
         }
         __syncthreads();
         if (kt + 1 < k_tiles) {

@@ -191,11 +191,12 @@ int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_d
     g1.K = H; g1.N = I; g1.Nw = I; g1.R = R; g1.E = E; g1.k = k;
     g1.mt_total = mt_total;
     g1.n_units = static_cast<int>((I + kBN - 1) / kBN);
-    // Column units an XCD sweeps together: up to 4, fewer when there are not
-    // enough units to keep all 8 XCDs busy.
+    // Column units an XCD sweeps together: up to 2 (one expert's weight panel for them is
+    // 4 MB at K = 4096, the size of an XCD's L2; 4 units measured 8 % slower), fewer when
+    // there are not enough units to keep all 8 XCDs busy.
     auto plan = [](FfnGemmParams& g) {
         int ngt = g.n_units / 8;
-        g.ngt = ngt < 1 ? 1 : (ngt > 4 ? 4 : ngt);
+        g.ngt = ngt < 1 ? 1 : (ngt > 2 ? 2 : ngt);
     };
     auto grid_of = [&](const FfnGemmParams& g) {
         const long groups = (g.n_units + 8 * g.ngt - 1) / (8 * g.ngt);
