@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
             key = key < p.Lk ? key : p.Lk - 1;  // masked later; keep the load in bounds
             const std::uint16_t* kp = kbase + static_cast<long>(key) * p.ks_l + 8 * lg;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) dst[kb][ks] = *reinterpret_cast<const i16x8*>(kp + 32 * ks);
+            for (int ks = 0; ks < 4; ++ks) dst[kb][ks] = __builtin_bit_cast(i16x8, load16_nt(kp + 32 * ks));  // read once: keep it out of the caches
         }
     };
     auto load_v = [&](int t) {
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
             const int c = lane + i * 64;  // 16-byte chunk of the 32 x 128 tile
             const int row = c >> 4, col = (c & 15) * 8;
             const int key = k_begin + t * kTile + row;
-            vst[i] = key < k_end ? load16(vbase + static_cast<long>(key) * p.vs_l + col) : u32x4{0, 0, 0, 0};
+            vst[i] = key < k_end ? load16_nt(vbase + static_cast<long>(key) * p.vs_l + col) : u32x4{0, 0, 0, 0};
         }
     };
     auto store_v = [&](int buf) {
