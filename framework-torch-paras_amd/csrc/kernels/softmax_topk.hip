@@ -1,0 +1,204 @@
+// Row softmax and row top-k on the device, with the reference host engine's
+// arithmetic (csrc/ops/pointwise_ops.cpp:926-981 and :1292-1381):
+//
+//   softmax  per row, in fp64: m = max_j v_j; s = sum_j exp(v_j - m);
+//            out_j = T_out( exp(v_j - m) / s ).  T_out is the input dtype, or
+//            fp32 for 16-bit inputs when the caller asks (half_to_float).
+//   top-k    the k largest (or smallest) of a row in sorted order, ties to the
+//            lower index, found as the reference does: slot s takes the best
+//            element that comes after slot s-1 in (value, index) order.
+//            Comparisons are on the values widened to double, so they are
+//            exact for every float dtype; indices are int64.
+//
+// One workgroup per row; rows are re-read from L2 between passes (these ops sit
+// on router logits and attention rows: thousands of elements, not millions).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+#include "paras_hip.h"
+
+namespace paras {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+
+__device__ __forceinline__ double wave_max_f64(double v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmax(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const typename Elem<TI>::store_t* __restrict__ x,
+                                                              typename Elem<TO>::store_t* __restrict__ out, long n) {
+    using EI = Elem<TI>;
+    using EO = Elem<TO>;
+    __shared__ double slots[kWaves];
+    const auto* xr = x + static_cast<long>(blockIdx.x) * n;
+    auto* outr = out + static_cast<long>(blockIdx.x) * n;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+
+    double m = -INFINITY;
+    for (long j = threadIdx.x; j < n; j += kBlock) {
+        const double v = EI::to_f64(xr[j]);
+        if (v > m) m = v;                       // as the host: a NaN never replaces the max
+    }
+    m = wave_max_f64(m);
+    if (lane == 0) slots[wave] = m;
+    __syncthreads();
+    m = slots[0];
+#pragma unroll
+    for (int i = 1; i < kWaves; ++i) m = fmax(m, slots[i]);
+    __syncthreads();
+
+    double s = 0.0;
+    for (long j = threadIdx.x; j < n; j += kBlock) s += exp(EI::to_f64(xr[j]) - m);
+    s = wave_sum(s);
+    if (lane == 0) slots[wave] = s;
+    __syncthreads();
+    s = 0.0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) s += slots[i];
+
+    for (long j = threadIdx.x; j < n; j += kBlock) outr[j] = EO::from_f64(exp(EI::to_f64(xr[j]) - m) / s);
+}
+
+// (value, index) order of the reference: larger value first (smaller when !largest), then lower index.
+__device__ __forceinline__ bool comes_before(double va, long ia, double vb, long ib, bool largest) {
+    return largest ? (va > vb || (va == vb && ia < ib)) : (va < vb || (va == vb && ia < ib));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void topk_rows_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                           typename Elem<T>::store_t* __restrict__ values,
+                                                           long* __restrict__ indices, long n, long k, int largest_i) {
+    using E = Elem<T>;
+    __shared__ double v_slots[kWaves];
+    __shared__ long   i_slots[kWaves];
+    const bool largest = largest_i != 0;
+    const auto* xr = x + static_cast<long>(blockIdx.x) * n;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+
+    double prev_v = 0.0;
+    long prev_i = -1;
+    for (long s = 0; s < k; ++s) {
+        double best_v = 0.0;
+        long best_i = -1;
+        for (long j = threadIdx.x; j < n; j += kBlock) {
+            const double v = E::to_f64(xr[j]);
+            // strictly after the previous slot in (value, index) order
+            if (s > 0 && !comes_before(prev_v, prev_i, v, j, largest)) continue;
+            if (best_i < 0 || comes_before(v, j, best_v, best_i, largest)) {
+                best_v = v;
+                best_i = j;
+            }
+        }
+        // wave, then workgroup argbest; index -1 marks "none"
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const double ov = __shfl_xor(best_v, off, kWave);
+            const long oi = __shfl_xor(best_i, off, kWave);
+            if (oi >= 0 && (best_i < 0 || comes_before(ov, oi, best_v, best_i, largest))) {
+                best_v = ov;
+                best_i = oi;
+            }
+        }
+        if (lane == 0) {
+            v_slots[wave] = best_v;
+            i_slots[wave] = best_i;
+        }
+        __syncthreads();
+        best_v = v_slots[0];
+        best_i = i_slots[0];
+#pragma unroll
+        for (int i = 1; i < kWaves; ++i) {
+            if (i_slots[i] >= 0 && (best_i < 0 || comes_before(v_slots[i], i_slots[i], best_v, best_i, largest))) {
+                best_v = v_slots[i];
+                best_i = i_slots[i];
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            // a row of NaNs has no element that "comes before" another: the host engine then
+            // reports index -1 for later slots; keep that
+            values[static_cast<long>(blockIdx.x) * k + s] = best_i >= 0 ? xr[best_i] : E::from_f64(0.0);
+            indices[static_cast<long>(blockIdx.x) * k + s] = best_i;
+        }
+        prev_v = best_v;
+        prev_i = best_i;
+    }
+}
+
+template <typename TI>
+int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, hipStream_t s) {
+    using SI = typename Elem<TI>::store_t;
+    const dim3 g(static_cast<unsigned>(rows)), b(kBlock);
+    if (dtype_out == PARAS_F32 && sizeof(SI) == 2)
+        hipLaunchKernelGGL((softmax_rows_kernel<TI, float>), g, b, 0, s, static_cast<const SI*>(x), static_cast<float*>(out), n);
+    else
+        hipLaunchKernelGGL((softmax_rows_kernel<TI, TI>), g, b, 0, s, static_cast<const SI*>(x), static_cast<SI*>(out), n);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+template <typename T>
+int launch_topk(const void* x, void* values, long* indices, long rows, long n, long k, int largest, hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    hipLaunchKernelGGL((topk_rows_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(kBlock), 0, s, static_cast<const S*>(x),
+                       static_cast<S*>(values), indices, n, k, largest);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // namespace
+}  // namespace paras
+
+extern "C" {
+
+int paras_softmax_rows(const void* x, void* out, int64_t rows, int64_t n, int dtype_in, int dtype_out, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(rows >= 0 && n >= 0, "paras_softmax_rows: negative shape");
+    if (rows == 0 || n == 0) return PARAS_OK;
+    PARAS_REQUIRE(x && out, "paras_softmax_rows: null pointer");
+    PARAS_REQUIRE(rows <= 0x7fffffffLL, "paras_softmax_rows: too many rows");
+    PARAS_REQUIRE(dtype_out == dtype_in || (dtype_out == PARAS_F32 && (dtype_in == PARAS_BF16 || dtype_in == PARAS_F16)),
+                  "paras_softmax_rows: the output dtype is the input dtype, or fp32 for a 16-bit input");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    switch (dtype_in) {
+        case PARAS_F32:  return launch_softmax<float>(x, out, rows, n, dtype_out, s);
+        case PARAS_F64:  return launch_softmax<double>(x, out, rows, n, dtype_out, s);
+        case PARAS_BF16: return launch_softmax<bf16_t>(x, out, rows, n, dtype_out, s);
+        case PARAS_F16:  return launch_softmax<f16_t>(x, out, rows, n, dtype_out, s);
+        default: return fail(PARAS_ERR_INVALID, "paras_softmax_rows: unknown dtype %d", dtype_in);
+    }
+}
+
+int paras_topk_rows(const void* x, void* values, int64_t* indices, int64_t rows, int64_t n, int64_t k, int largest,
+                    int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(rows >= 0 && n >= 0, "paras_topk_rows: negative shape");
+    PARAS_REQUIRE(k >= 0 && k <= n, "paras_topk_rows: k out of range");
+    if (rows == 0 || k == 0) return PARAS_OK;
+    PARAS_REQUIRE(x && values && indices, "paras_topk_rows: null pointer");
+    PARAS_REQUIRE(rows <= 0x7fffffffLL, "paras_topk_rows: too many rows");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    long* idx = reinterpret_cast<long*>(indices);
+    switch (dtype) {
+        case PARAS_F32:  return launch_topk<float>(x, values, idx, rows, n, k, largest, s);
+        case PARAS_F64:  return launch_topk<double>(x, values, idx, rows, n, k, largest, s);
+        case PARAS_BF16: return launch_topk<bf16_t>(x, values, idx, rows, n, k, largest, s);
+        case PARAS_F16:  return launch_topk<f16_t>(x, values, idx, rows, n, k, largest, s);
+        default: return fail(PARAS_ERR_INVALID, "paras_topk_rows: unknown dtype %d", dtype);
+    }
+}
+
+}  // extern "C"

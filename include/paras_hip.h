@@ -289,6 +289,21 @@ PARAS_API int paras_gemm_nt(const void* a, const void* b, const void* addend, vo
                             int64_t stride_b, int64_t stride_c, int64_t stride_add,
                             double alpha, double beta, int dtype, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* Row softmax and row top-k (replace softmax_out / topk_out,                  */
+/* csrc/ops/pointwise_ops.cpp:926-981 and :1292-1381), over the last dim of a  */
+/* contiguous [rows, n] tensor.                                                */
+/*   softmax: fp64 per row, out_j = T_out(exp(v_j - max) / sum); dtype_out is  */
+/*            dtype_in, or PARAS_F32 for a 16-bit input (half_to_float).       */
+/*   top-k:   values [rows, k] (dtype of x) and int64 indices [rows, k], sorted,*/
+/*            largest != 0 -> descending; ties go to the lower index.  Rows    */
+/*            containing NaN have no defined order.                            */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_softmax_rows(const void* x, void* out, int64_t rows, int64_t n,
+                                 int dtype_in, int dtype_out, void* stream);
+PARAS_API int paras_topk_rows(const void* x, void* values, int64_t* indices, int64_t rows,
+                              int64_t n, int64_t k, int largest, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

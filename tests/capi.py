@@ -63,6 +63,8 @@ SIGNATURES = {
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
     "paras_gemm_nt": (i32, [vp, vp, vp, vp] + [i64] * 12 + [f64, f64, i32, vp]),
+    "paras_softmax_rows": (i32, [vp, vp, i64, i64, i32, i32, vp]),
+    "paras_topk_rows": (i32, [vp, vp, vp, i64, i64, i64, i32, i32, vp]),
 }
 
 _lib = None
@@ -241,3 +243,21 @@ def gemm_nt(a, b, addend=None, alpha=1.0, beta=1.0):
                               a.stride(-2), b.stride(-2), N, ld_add, B, sa, sb, M * N, sadd, alpha, beta,
                               DT[a.dtype], _stream()))
     return c
+
+
+def softmax_rows(x, out_dtype=None):
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    n = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // n if n else 0
+    check(lib().paras_softmax_rows(_ptr(x), _ptr(out), rows, n, DT[x.dtype], DT[out_dtype], _stream()))
+    return out
+
+
+def topk_rows(x, k, largest=True):
+    n = x.shape[-1]
+    rows = x.numel() // n if n else 0
+    values = torch.empty(*x.shape[:-1], k, dtype=x.dtype, device=x.device)
+    indices = torch.empty(*x.shape[:-1], k, dtype=torch.int64, device=x.device)
+    check(lib().paras_topk_rows(_ptr(x), _ptr(values), _ptr(indices), rows, n, k, 1 if largest else 0, DT[x.dtype], _stream()))
+    return values, indices

@@ -1,0 +1,67 @@
+"""Row softmax and row top-k on the device through the C ABI, against the oracle
+(reference arithmetic: csrc/ops/pointwise_ops.cpp:926-981, 1292-1381) and the
+reference tests' own checks (torch-CPU parity, tests/test_pointwise_ops.py:224-267,
+369-413, including its tie literal)."""
+import pytest
+import torch
+
+import capi
+import oracle as O
+from conftest import assert_bit_exact
+
+pytestmark = pytest.mark.gpu
+FLOATS = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("shape", [(1, 1), (7, 8), (33, 300), (4, 5000), (2, 3, 129)])
+def test_softmax_matches_oracle(dtype, shape):
+    torch.manual_seed(sum(shape))
+    x = (3 * torch.randn(*shape)).to(dtype)
+    got = capi.softmax_rows(x.cuda()).cpu()
+    want = O.softmax_last(x)
+    # device exp() and the host's libm may differ in the last bit of a double, and the row sum is
+    # taken in a different order: after narrowing that shows, rarely, as one unit in the last place
+    if dtype in (torch.bfloat16, torch.float16):
+        diff = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) <= 1e-3
+    else:
+        assert torch.allclose(got, want, rtol=1e-6 if dtype == torch.float32 else 1e-13, atol=0)
+    assert torch.allclose(got.double().sum(-1), torch.ones(shape[:-1], dtype=torch.float64), atol=2e-2 if dtype in (torch.bfloat16, torch.float16) else 1e-5)
+
+
+def test_softmax_half_to_float_and_extremes():
+    x = torch.tensor([[0.0, -1e4, 1e4, 5.0], [float("-inf"), 0.0, 0.0, float("-inf")]], dtype=torch.float16)
+    got = capi.softmax_rows(x.cuda(), torch.float32).cpu()
+    assert got.dtype == torch.float32
+    assert torch.allclose(got, O.softmax_last(x, torch.float32), rtol=1e-6, atol=0)
+    assert torch.allclose(got, torch.softmax(x.float(), -1), rtol=1e-6, atol=1e-30)
+    with pytest.raises(capi.ParasError):
+        capi.softmax_rows(torch.zeros(2, 4, device="cuda"), torch.float16)
+    assert capi.softmax_rows(torch.zeros(0, 4, device="cuda")).shape == (0, 4)
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("largest", [True, False])
+def test_topk_matches_oracle_bitwise(dtype, largest):
+    torch.manual_seed(11)
+    for shape, k in (((5, 8), 2), ((9, 64), 8), ((3, 1000), 17), ((2, 2, 300), 300), ((4, 7), 0)):
+        x = torch.randn(*shape).to(dtype)
+        x = (x * 4).round() / 4 if dtype != torch.float64 else x          # quantised: plenty of ties
+        gv, gi = capi.topk_rows(x.cuda(), k, largest)
+        wv, wi = O.topk_last(x, k, largest)
+        assert_bit_exact(gi, wi, f"topk indices {shape} k={k}")
+        assert_bit_exact(gv, wv, f"topk values {shape} k={k}")
+
+
+def test_topk_reference_tie_literal_and_torch_parity():
+    x = torch.tensor([[5.0, 3.0, 5.0, 5.0, 1.0, 3.0]])                  # tests/test_pointwise_ops.py:405-413
+    v, i = capi.topk_rows(x.cuda(), 4)
+    assert i.cpu().tolist() == [[0, 2, 3, 1]] and v.cpu().tolist() == [[5.0, 5.0, 5.0, 3.0]]
+    torch.manual_seed(5)
+    y = torch.randn(16, 257)                                              # distinct values: order is unique
+    v, i = capi.topk_rows(y.cuda(), 9)
+    tv, ti = torch.topk(y, 9, dim=-1)
+    assert torch.equal(i.cpu(), ti) and torch.equal(v.cpu(), tv)
+    with pytest.raises(capi.ParasError, match="k out of range"):
+        capi.topk_rows(y.cuda(), 300)

@@ -351,3 +351,21 @@ def test_linear_backward_through_device_gemm(device):
     for got, want in ((xd.grad, xc.grad), (wd.grad, wc.grad)):
         err = (got.cpu().float() - want.float()).abs().max().item()
         assert err <= 0.02 * want.float().abs().max().item() + 1e-3, err
+
+
+def test_softmax_and_topk_ops_on_device(device):
+    torch.manual_seed(3)
+    x = torch.randn(4, 6, 50)
+    xd = x.to(device)
+    for dim in (-1, 1, 0):
+        assert_close(torch.softmax(xd, dim), torch.softmax(x, dim), f"softmax dim {dim}")
+    h = x.half()
+    out = torch.softmax(h.to(device), -1, dtype=torch.float32)           # half_to_float
+    assert out.dtype == torch.float32
+    assert_close(out, torch.softmax(h, -1, dtype=torch.float32), "softmax half_to_float")
+    for dim, k in ((-1, 5), (1, 3)):
+        v, i = torch.topk(xd, k, dim=dim)
+        tv, ti = torch.topk(x, k, dim=dim)
+        assert torch.equal(i.cpu(), ti) and torch.equal(v.cpu(), tv)
+    v, i = torch.topk(torch.tensor([[5, 3, 5, 5, 1, 3]]).to(device), 4)  # integer dtype: host route
+    assert v.cpu().tolist() == [[5, 5, 5, 3]]
