@@ -53,23 +53,23 @@ __global__ __launch_bounds__(kThreads, 2) void dense_gemm_nt_kernel(const DenseP
     const int lr = lane & 31, lh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    const std::uint16_t* a_ptr[4];
-    const std::uint16_t* b_ptr[2][4];
+    unsigned a_off[4], b_off[2][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int c = tid + i * kThreads;
         long arow = row0 + (c >> 3);
         if (arow >= p.M) arow = p.M - 1;     // clamped rows are computed but never stored
-        a_ptr[i] = A + arow * p.lda + (c & 7) * 8;
+        a_off[i] = static_cast<unsigned>(arow * p.lda + (c & 7) * 8);
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             long brow = n0 + g * kBN + (c >> 3);
             if (brow >= p.N) brow = p.N - 1;
-            b_ptr[g][i] = B + brow * p.ldb + (c & 7) * 8;
+            b_off[g][i] = static_cast<unsigned>(brow * p.ldb + (c & 7) * 8);
         }
     }
+    const std::uint16_t* const b_base[2] = {B, B};
     float16_t acc[2][2][2];
-    tile_mainloop<T>(a_ptr, b_ptr, p.K, lds, acc);
+    tile_mainloop<T>(A, a_off, b_base, b_off, p.K, lds, acc);
 
     std::uint16_t* C = p.c + bidx * p.sc;
     const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
@@ -116,6 +116,8 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
     const int64_t m_tiles = (M + gemm::kBM - 1) / gemm::kBM, n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
+    if (M * lda >= (1LL << 32) || N * ldb >= (1LL << 32))
+        return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: an operand matrix spans 2^32 elements or more");
     hipStream_t s = nullptr;
     int rc = resolve_stream(stream, &s);
     if (rc != PARAS_OK) return rc;

@@ -21,7 +21,8 @@ constexpr int kThreads = 256;
 constexpr int kBM = 128;
 constexpr int kBN = 128;          // columns per group; a workgroup computes two groups
 constexpr int kBK = 64;
-constexpr int kLS = kBK + 8;      // LDS row stride (elements): 16 consecutive rows hit distinct banks
+constexpr int kLS = kBK + 8;      // LDS row stride (elements): 16 consecutive rows hit distinct banks.  (Unpadded rows
+                                  // with an XOR swizzle of the chunks measured no faster.)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 
@@ -43,12 +44,15 @@ struct TileLds {
     std::uint16_t b[2][kBN * kLS];
 };
 
-// a_ptr[i] / b_ptr[g][i]: this thread's four 16-byte chunks per operand row set
-// (chunk c = tid + i*256 -> tile row c/8, column (c%8)*8), already offset to k = 0.
+// a_off[i] / b_off[g][i]: element offsets (from the uniform bases a_base / b_base[g]) of this
+// thread's four 16-byte chunks per operand row set at k = 0 (chunk c = tid + i*256 -> tile row
+// c/8, column (c%8)*8).  32-bit offsets against a scalar base keep the addressing out of the
+// vector registers; callers check that every operand spans fewer than 2^32 elements.
 // Accumulates into acc[g][mi][ni]; lane (column lr = lane%32, half lh = lane/32) of
 // block (mi, ni) ends up holding rows (r/4)*8 + 4*lh + r%4, r = 0..15.
 template <typename T>
-__device__ __forceinline__ void tile_mainloop(const std::uint16_t* const (&a_ptr)[4], const std::uint16_t* const (&b_ptr)[2][4],
+__device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
+                                              const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][4],
                                               long K, TileLds& lds, float16_t (&acc)[2][2][2]) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lh = lane >> 5;
@@ -58,11 +62,11 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* const (&a_ptr
     u32x4 a_st[4], b_st[2][4];
     auto load_tile = [&](long k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_ptr[i] + k0);
+        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_base + k0 + a_off[i]);
 #pragma unroll
         for (int g = 0; g < 2; ++g)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_ptr[g][i] + k0);
+            for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_base[g] + k0 + b_off[g][i]);
     };
     auto store_tile = [&]() {
 #pragma unroll
@@ -84,8 +88,8 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* const (&a_ptr
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[g][mi][ni][r] = 0.f;
 
-    const int a_off = (wm * 64 + lr) * kLS + lh * 8;
-    const int b_off = (wn * 64 + lr) * kLS + lh * 8;
+    const int a_off0 = (wm * 64 + lr) * kLS + lh * 8;
+    const int b_off0 = (wn * 64 + lr) * kLS + lh * 8;
     const long k_tiles = K / kBK;
     load_tile(0);
     store_tile();
@@ -100,10 +104,10 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* const (&a_ptr
         auto read_a = [&](int buf, int ks) {
 #pragma unroll
             for (int mi = 0; mi < 2; ++mi)
-                af[buf][mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off + mi * 32 * kLS + ks * 16]);
+                af[buf][mi] = *reinterpret_cast<const i16x8*>(&a_lds[a_off0 + mi * 32 * kLS + ks * 16]);
         };
         auto read_b = [&](int q, int ks) {   // q = 2*g + ni
-            bf[q] = *reinterpret_cast<const i16x8*>(&b_lds[q >> 1][b_off + (q & 1) * 32 * kLS + ks * 16]);
+            bf[q] = *reinterpret_cast<const i16x8*>(&b_lds[q >> 1][b_off0 + (q & 1) * 32 * kLS + ks * 16]);
         };
         read_a(0, 0);
 #pragma unroll

@@ -94,16 +94,17 @@ __global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemm
     const int wm = wave >> 1, wn = wave & 1;
 
     // ---- global -> register staging: 16-byte chunks, 8 per row of a k-tile
-    const std::uint16_t* a_ptr[4];
+    unsigned a_off[4], b_off[2][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int c = tid + i * kThreads;
         long prow = row0 + (c >> 3);
         if (prow >= row_end) prow = row_end - 1;  // clamp: result rows beyond the expert are not stored
         const long src = p.order ? p.order[prow] / p.k : prow;
-        a_ptr[i] = p.a + src * p.K + (c & 7) * 8;
+        a_off[i] = static_cast<unsigned>(src * p.K + (c & 7) * 8);
     }
-    const std::uint16_t* b_ptr[2][4];
+    // weights of this expert: a uniform base per column group, rows as 32-bit offsets
+    const std::uint16_t* const b_base[2] = {p.b + static_cast<long>(e) * p.Nw * p.K, p.b2 + static_cast<long>(e) * p.Nw * p.K};
 #pragma unroll
     for (int g = 0; g < 2; ++g)
 #pragma unroll
@@ -111,11 +112,10 @@ __global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemm
             const int c = tid + i * kThreads;
             long wrow = (kSwiglu ? n0 : n0 + g * kBN) + (c >> 3);
             if (wrow >= p.Nw) wrow = p.Nw - 1;
-            const std::uint16_t* base = g == 0 ? p.b : p.b2;
-            b_ptr[g][i] = base + (static_cast<long>(e) * p.Nw + wrow) * p.K + (c & 7) * 8;
+            b_off[g][i] = static_cast<unsigned>(wrow * p.K + (c & 7) * 8);
         }
     float16_t acc[2][2][2];
-    tile_mainloop<T>(a_ptr, b_ptr, p.K, lds, acc);
+    tile_mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, acc);
 
     // ---- epilogue.  Accumulator lane (column lr, half lh) holds rows (r/4)*8 + 4*lh + r%4.
 #pragma unroll
@@ -257,6 +257,8 @@ int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up, const voi
                     reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0,
                   "paras_moe_ffn: tensors must be 16-byte aligned");
     PARAS_REQUIRE(T * k <= 0x3fffffffLL, "paras_moe_ffn: too many routed rows");
+    if (T * H >= (1LL << 32) || T * k * I >= (1LL << 32) || I * H >= (1LL << 32))
+        return fail(PARAS_ERR_UNSUPPORTED, "paras_moe_ffn: an operand (x, the routed intermediate, or one expert's weight matrix) spans 2^32 elements or more");
     hipStream_t s = nullptr;
     int rc = resolve_stream(stream, &s);
     if (rc != PARAS_OK) return rc;
