@@ -446,8 +446,15 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     if (wave_tiles > 0) {  // the wave's last tile: nothing to compute ahead in its second block
         const int t = wave_tiles - 1;
         const bool pending = stage_ahead(t);
-        block(2 * t, s_a, s_b, Yes{});
-        block(2 * t + 1, s_b, s_a, No{});
+        // The tile's second block contributes nothing when it starts past the end of K or, for a
+        // causal wave, past the wave's last query (every other wave's diagonal tile).
+        const int second0 = (2 * t + 1) * 32;
+        if (second0 >= p.Lk || (kCausal && second0 > q0 + WQ - 1)) {
+            block(2 * t, s_a, s_b, No{});
+        } else {
+            block(2 * t, s_a, s_b, Yes{});
+            block(2 * t + 1, s_b, s_a, No{});
+        }
         publish(pending);
     }
     for (int t = wave_tiles; t < n_tiles; ++t) publish(stage_ahead(t));
