@@ -94,3 +94,24 @@ def test_gemm_nt_linearity_at_projection_size():
     rows = torch.randint(0, M, (8,))
     ref = O.matmul_nt(a1[rows].cpu(), w.cpu())
     assert_gemm_close(y1[rows], ref, dt)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_nt_many_tiles_with_ragged_edges(dtype):
+    """Thousands of tiles, with M and N that are not multiples of the tile; sampled rows (first,
+    last, tile boundaries) against the oracle."""
+    torch.manual_seed(9)
+    M, N, K = 8269, 4129, 192
+    a = torch.randn(M, K, device="cuda").to(dtype)
+    b = (0.1 * torch.randn(N, K, device="cuda")).to(dtype)
+    bias = torch.randn(N, device="cuda").to(dtype)
+    out = capi.gemm_nt(a, b)
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 257, 4095, 4096, 8191, 8192, M - 2, M - 1])
+    ref = O.matmul_nt(a[rows].cpu(), b.cpu())
+    assert_gemm_close(out[rows], ref, dtype)
+    out2 = capi.gemm_nt(a, b, bias, alpha=1.0, beta=1.0)
+    assert_gemm_close(out2[rows], torch.nn.functional.linear(a[rows].cpu(), b.cpu(), bias.cpu()), dtype)
+    # whole-matrix property: doubling A doubles every output bit for bit (away from f16's subnormals,
+    # where 2 * round(v) and round(2 v) keep different numbers of bits)
+    big = out.float().abs() > 1e-3
+    assert torch.equal(capi.gemm_nt(a * 2, b)[big], (out * 2)[big])
