@@ -100,8 +100,32 @@ __device__ __forceinline__ T wave_allreduce(T v, Op op) {
     for (int off = kWave / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWave));
     return v;
 }
+// Sum of a double over the 64 lanes, every lane gets the result.  The generic butterfly
+// above goes through the LDS crossbar (ds_bpermute) twelve times in a dependent chain; this one
+// stays in the VALU: four DPP exchanges inside each row of 16 lanes (quad swaps, then the
+// half-row and row mirrors, which pair up equal partial sums), then the four row sums are read
+// with v_readlane and added.
+template <int kCtrl>
+__device__ __forceinline__ double dpp_move_f64(double v) {
+    const std::uint64_t b = __builtin_bit_cast(std::uint64_t, v);
+    const int lo = static_cast<int>(b), hi = static_cast<int>(b >> 32);
+    const int lo2 = __builtin_amdgcn_update_dpp(lo, lo, kCtrl, 0xf, 0xf, false);
+    const int hi2 = __builtin_amdgcn_update_dpp(hi, hi, kCtrl, 0xf, 0xf, false);
+    return __builtin_bit_cast(double, (static_cast<std::uint64_t>(static_cast<std::uint32_t>(hi2)) << 32) |
+                                          static_cast<std::uint32_t>(lo2));
+}
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+    const std::uint64_t b = __builtin_bit_cast(std::uint64_t, v);
+    const std::uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(b), lane);
+    const std::uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(b >> 32), lane);
+    return __builtin_bit_cast(double, (static_cast<std::uint64_t>(hi) << 32) | lo);
+}
 __device__ __forceinline__ double wave_sum(double v) {
-    return wave_allreduce(v, [](double a, double b) { return a + b; });
+    v += dpp_move_f64<0xB1>(v);    // quad_perm [1,0,3,2]: lane ^ 1
+    v += dpp_move_f64<0x4E>(v);    // quad_perm [2,3,0,1]: lane ^ 2
+    v += dpp_move_f64<0x141>(v);   // row_half_mirror: the other quad of the half row
+    v += dpp_move_f64<0x140>(v);   // row_mirror: the other half of the row
+    return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
 __device__ __forceinline__ float wave_sum(float v) {
     return wave_allreduce(v, [](float a, float b) { return a + b; });

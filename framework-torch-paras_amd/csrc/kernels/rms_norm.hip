@@ -26,17 +26,18 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 
-// Sum over the workgroup; result valid in every thread.  `slots` is LDS of
-// kWavesPerBlock doubles.  Safe to call repeatedly with the same slots.
-__device__ __forceinline__ double block_sum(double v, double* slots) {
+// Sum over the workgroup; result valid in every thread.  `slots` is LDS of 2 * kWavesPerBlock
+// doubles used as two alternating sets: a call uses set `parity & 1`, so the readers of one call
+// never race with the writers of the next and a single barrier per call is enough (the set is
+// reused only two calls later, with this call's barrier in between).
+__device__ __forceinline__ double block_sum(double v, double* slots, int parity) {
     v = wave_sum(v);
-    const int wave = threadIdx.x / kWave;
-    __syncthreads();  // previous readers of slots are done
-    if ((threadIdx.x & (kWave - 1)) == 0) slots[wave] = v;
+    double* set = slots + (parity & 1) * kWavesPerBlock;
+    if ((threadIdx.x & (kWave - 1)) == 0) set[threadIdx.x / kWave] = v;
     __syncthreads();
     double t = 0.0;
 #pragma unroll
-    for (int i = 0; i < kWavesPerBlock; ++i) t += slots[i];
+    for (int i = 0; i < kWavesPerBlock; ++i) t += set[i];
     return t;
 }
 
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(kBlock, 8) void rms_norm_fwd_vec(
     using E = Elem<T>;
     using S = typename E::store_t;
     constexpr int V = E::kVec;
-    __shared__ double slots[kWavesPerBlock];
+    __shared__ double slots[2 * kWavesPerBlock];
 
     const int nvec = H / V;  // 16-byte vectors per row
     u32x4 wv[NV];
@@ -73,6 +74,7 @@ __global__ __launch_bounds__(kBlock, 8) void rms_norm_fwd_vec(
         const int c = threadIdx.x + i * kBlock;
         if (c < nvec) wv[i] = load16(w + static_cast<long>(c) * V);  // shared by every row: an L2 hit
     }
+    int sum_calls = 0;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         const S* xr = x + r * H;
         S* outr = out + r * H;
@@ -95,7 +97,7 @@ __global__ __launch_bounds__(kBlock, 8) void rms_norm_fwd_vec(
                 }
             }
         }
-        ss = block_sum(ss, slots);
+        ss = block_sum(ss, slots, sum_calls++);
         // 16-bit tensors: mean by the reciprocal and the refined rsqrt (outputs
         // cannot see the difference); fp32 / fp64 tensors: the host's own form.
         const double rs = sizeof(S) == 2 ? rsqrt_f64(fma(ss, inv_h, eps)) : 1.0 / sqrt(ss / static_cast<double>(H) + eps);
@@ -137,7 +139,8 @@ __global__ __launch_bounds__(kBlock) void rms_norm_fwd_any(
     typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, long H,
     double eps) {
     using E = Elem<T>;
-    __shared__ double slots[kWavesPerBlock];
+    __shared__ double slots[2 * kWavesPerBlock];
+    int sum_calls = 0;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         const auto* xr = x + r * H;
         auto* outr = out + r * H;
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_fwd_any(
             const double v = E::to_f64(xr[j]);
             ss = fma(v, v, ss);
         }
-        ss = block_sum(ss, slots);
+        ss = block_sum(ss, slots, sum_calls++);
         const double rs = 1.0 / sqrt(ss / static_cast<double>(H) + eps);
         if (threadIdx.x == 0) rstd[r] = static_cast<float>(rs);
         for (long j = threadIdx.x; j < H; j += kBlock)
@@ -165,7 +168,8 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dx(
     const typename Elem<T>::store_t* __restrict__ w, const float* __restrict__ rstd,
     typename Elem<T>::store_t* __restrict__ gx, long rows, long H) {
     using E = Elem<T>;
-    __shared__ double slots[kWavesPerBlock];
+    __shared__ double slots[2 * kWavesPerBlock];
+    int sum_calls = 0;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         const auto* gr = go + r * H;
         const auto* xr = x + r * H;
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dx(
         double dot = 0.0;
         for (long j = threadIdx.x; j < H; j += kBlock)
             dot += E::to_f64(gr[j]) * E::to_f64(w[j]) * E::to_f64(xr[j]);
-        dot = block_sum(dot, slots);
+        dot = block_sum(dot, slots, sum_calls++);
         const double coef = rr * rr * rr / static_cast<double>(H);
         for (long j = threadIdx.x; j < H; j += kBlock) {
             const double gj = E::to_f64(gr[j]), wj = E::to_f64(w[j]), xj = E::to_f64(xr[j]);
