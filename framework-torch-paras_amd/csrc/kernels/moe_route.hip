@@ -26,6 +26,7 @@
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
+#include "paras_hip.h"
 
 namespace paras {
 namespace {
@@ -180,9 +181,11 @@ int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dty
     int rc = resolve_stream(stream, &s);
     if (rc != PARAS_OK) return rc;
     if (T == 0) {
-        PARAS_HIP_TRY(hipMemsetAsync(counts, 0, sizeof(int64_t) * E, s));
-        PARAS_HIP_TRY(hipMemsetAsync(offsets, 0, sizeof(int64_t) * (E + 1), s));
-        return PARAS_OK;
+        // fill kernels rather than hipMemsetAsync: the caller may be capturing this stream into a graph
+        const int64_t one = 1, ne = E, ne1 = E + 1;
+        rc = paras_fill_strided(counts, 1, &ne, &one, 8, 0, stream);
+        if (rc != PARAS_OK) return rc;
+        return paras_fill_strided(offsets, 1, &ne1, &one, 8, 0, stream);
     }
     PARAS_REQUIRE(logits && topi && topw && order && workspace, "paras_moe_route: null pointer");
     static_assert(sizeof(long) == sizeof(int64_t), "LP64 expected");

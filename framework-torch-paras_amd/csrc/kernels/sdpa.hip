@@ -7,6 +7,7 @@
 #include "core/device_context.h"
 #include "core/status.h"
 #include "kernels/sdpa_internal.h"
+#include "paras_hip.h"
 
 namespace paras {
 namespace {
@@ -73,9 +74,10 @@ int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream) {
     if (rc != PARAS_OK) return rc;
     if (a.Lk == 0) {
         // softmax over nothing, then a product with an empty inner dim: zeros.
-        const size_t esz = a.dtype == PARAS_F64 ? 8 : a.dtype == PARAS_F32 ? 4 : 2;
-        PARAS_HIP_TRY(hipMemsetAsync(a.out, 0, static_cast<size_t>(a.B * a.Hq * a.Lq * a.Dv) * esz, s));
-        return PARAS_OK;
+        // (a fill kernel rather than hipMemsetAsync: callers may be capturing this stream into a graph)
+        const int esz = a.dtype == PARAS_F64 ? 8 : a.dtype == PARAS_F32 ? 4 : 2;
+        const int64_t n = a.B * a.Hq * a.Lq * a.Dv, one = 1;
+        return paras_fill_strided(a.out, 1, &n, &one, esz, 0, stream);
     }
     switch (choose(a)) {
         case SdpaKernel::Flash: return launch_flash(a, s);
