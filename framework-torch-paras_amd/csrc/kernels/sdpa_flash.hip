@@ -161,11 +161,28 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     auto ksw = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
     auto vsw = [](int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
 
-    // LDS ring: NST tiles each of K and V (2 x 32 KiB per workgroup, two workgroups per CU).
-    constexpr int NST = 2;
-    constexpr int LA  = NST - 1;             // tiles of lookahead
-    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds[NST][kBN * D];
-    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds[NST][kBN * D];
+    // LDS: two tiles each of K and V (4 x 16 KiB per workgroup at D = 128, two workgroups per
+    // CU).  They are four separate arrays on purpose: the compiler makes an LDS read wait for
+    // every direct-to-LDS load in flight unless it can prove from the variables involved that the
+    // two do not overlap, and the point of the double buffer is to read one tile while the next
+    // one streams in.  The main loop therefore names its buffers at compile time (`Par`), the
+    // rarely taken paths pick them at run time (`AnyPar`) and accept the wait.
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds0[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds1[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds0[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds1[kBN * D];
+    using Par0 = std::integral_constant<int, 0>;
+    using Par1 = std::integral_constant<int, 1>;
+    struct AnyPar { int value; };
+    // buffer of tile index parity `par`; `flip` selects the other one
+    auto kbuf = [&](auto par, bool flip) -> std::uint16_t* {
+        if constexpr (std::is_same<decltype(par), AnyPar>::value) return ((par.value ^ (flip ? 1 : 0)) & 1) ? k_lds1 : k_lds0;
+        else return (decltype(par)::value != 0) != flip ? k_lds1 : k_lds0;
+    };
+    auto vbuf = [&](auto par, bool flip) -> std::uint16_t* {
+        if constexpr (std::is_same<decltype(par), AnyPar>::value) return ((par.value ^ (flip ? 1 : 0)) & 1) ? v_lds1 : v_lds0;
+        else return (decltype(par)::value != 0) != flip ? v_lds1 : v_lds0;
+    };
 
     const int nq = p.n_qblocks;
     const int BH = p.B * p.Hq;
@@ -215,54 +232,43 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     }
     const int wave_tiles = kCausal ? min(n_tiles, (q0 + WQ - 1) / kBN + 1) : n_tiles;
 
-    // ---- staging: 64 LDS rows <- global rows first .. first+63 (rows outside [0, Lk) read as zero)
+    // ---- staging: 64 LDS rows <- global rows first .. first+63, straight from memory into LDS
+    // with buffer loads.  The buffer descriptor spans rows [0, Lk) of this (batch, kv head), so
+    // rows outside it (before the first key in K tile 0, past the end of K in the last tiles)
+    // arrive as zeros without a branch: the hardware range-checks every dword of every lane.
     const int srow = wave * RPI + lane / CHUNKS;
     const int slot = lane % CHUNKS;
-    const unsigned koff = static_cast<unsigned>(srow * p.ks_l + ((slot ^ ksw(srow)) * 8));
-    const unsigned voff = static_cast<unsigned>(srow * p.vs_l + ((slot ^ vsw(srow)) * 8));
-    typedef __attribute__((address_space(1))) const void* gptr_t;
+    const int k_row_bytes = static_cast<int>(p.ks_l) * 2, v_row_bytes = static_cast<int>(p.vs_l) * 2;
+    const int k_lane = srow * k_row_bytes + ((slot ^ ksw(srow)) * 16);
+    const int v_lane = srow * v_row_bytes + ((slot ^ vsw(srow)) * 16);
     typedef __attribute__((address_space(3))) void* lptr_t;
-    // Returns true when exactly NI direct loads per lane were issued (the count the
-    // partial wait in publish() relies on).
-    auto stage_rows = [&](const std::uint16_t* base, long stride, unsigned off, int first, std::uint16_t* tile) -> bool {
-        const std::uint16_t* src = base + static_cast<long>(first) * stride;   // only dereferenced for rows in range
-        if (first >= 0 && first + kBN <= p.Lk) {
+    auto make_rsrc = [&](const std::uint16_t* base, int row_bytes) {
+        const int bytes = (p.Lk - 1) * row_bytes + D * 2;           // < 2^31: checked by flash_supported
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<std::uint16_t*>(base), 0, bytes, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(kbase, k_row_bytes);
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(vbase, v_row_bytes);
+    auto stage_rows = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile) {
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int r0 = i * RPI * NW;
-                __builtin_amdgcn_global_load_lds((gptr_t)(src + static_cast<long>(r0) * stride + off),
-                                                 (lptr_t)(tile + (r0 + wave * RPI) * D), 16, 0, 0);
-            }
-            return true;
-        } else {
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int r0 = i * RPI * NW;
-                std::uint16_t* dst = tile + (r0 + wave * RPI) * D;
-                const int row = first + r0 + srow;
-                if (row >= 0 && row < p.Lk)
-                    __builtin_amdgcn_global_load_lds((gptr_t)(src + static_cast<long>(r0) * stride + off), (lptr_t)dst, 16, 0, 0);
-                else
-                    *reinterpret_cast<u32x4*>(dst + lane * 8) = u32x4{0, 0, 0, 0};
-            }
-            return false;
+        for (int i = 0; i < NI; ++i) {
+            const int r0 = i * RPI * NW;
+            // a negative offset is a huge unsigned one: out of range like the rows past the end
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)(tile + (r0 + wave * RPI) * D), 16,
+                                                     lane_off + (first + r0) * row_bytes, 0, 0, 0);
         }
     };
-    // Requests K tile t+1 and V tile t (the pair tile t's successor blocks need).
-    auto stage_pair = [&](int t) -> bool {
-        const bool a = stage_rows(kbase, p.ks_l, koff, (t + 1) * kBN - 32, k_lds[(t + 1) % NST]);
-        const bool c = stage_rows(vbase, p.vs_l, voff, t * kBN, v_lds[t % NST]);
-        return a && c;
+    // Requests the pair tile t's blocks need beyond K tile t: K tile t+1 and V tile t (`par` = parity of t).
+    auto stage_pair = [&](int t, auto par) {
+        stage_rows(k_rsrc, k_lane, k_row_bytes, (t + 1) * kBN - 32, kbuf(par, true));
+        stage_rows(v_rsrc, v_lane, v_row_bytes, t * kBN, vbuf(par, false));
     };
-    // Barrier that publishes every tile requested so far, except (newest_pending) the
-    // most recently requested pair, whose 2*NI loads per lane may stay in flight.
-    auto publish = [&](bool newest_pending) {
-        if (newest_pending) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI) : "memory");
-        else                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Barrier that publishes every tile requested so far.
+    auto publish = [&]() {
+        // s_waitcnt simm16 on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8.  The
+        // builtin (not inline asm) so that the compiler's own wait bookkeeping sees the loads retire.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
     };
-    // Start of tile t: request the pair LA tiles ahead; end of tile t: tiles up to t+1 must be in.
-    auto stage_ahead = [&](int t) -> bool { return t + LA < n_tiles ? stage_pair(t + LA) && LA == 2 : false; };
 
     float16_t oacc[QB][DBLK];
     float m_run[QB], l_run[QB];
@@ -276,13 +282,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             for (int r = 0; r < 16; ++r) oacc[qb][i][r] = 0.f;
     }
 
-    {
-        stage_rows(kbase, p.ks_l, koff, -32, k_lds[0]);   // K tile 0: keys 0..31 in its upper half
-        stage_pair(0);
-        bool pending = false;
-        if (LA == 2 && 1 < n_tiles) pending = stage_pair(1);
-        publish(pending);
-    }
+    stage_rows(k_rsrc, k_lane, k_row_bytes, -32, k_lds0);   // K tile 0: keys 0..31 in its upper half
+    stage_pair(0, Par0{});
+    publish();
 
     const int grp = lane >> 4, m16 = lane & 15;
     int k_rd[KSTEPS], v_rd[DBLK];
@@ -347,40 +349,56 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 
     // One block: exponentials of `cur` = S(j) and, if kNext, the MFMAs of S(j+1) into `nxt`,
     // then PV(j).  The MFMA part is a fixed schedule of KSTEPS + 2*DBLK slots (QB MFMAs per
-    // slot, sharing one LDS fragment), fenced so that the compiler keeps the order: fragment
-    // reads run two slots ahead (three rotating fragment registers) and the 8*QB exp pairs
-    // (2 fma + 2 exp + cvt + dot2 each) are spread between the MFMAs so the matrix pipe has
-    // an instruction in flight while the VALU works.  P(s2=0) is complete before the first
-    // PV MFMA, P(s2=1) before the first PV MFMA that uses it; the in-lane row maxima of
-    // S(j+1) are taken in the last slots.
-    auto block = [&](int j, float16_t (&cur)[QB], float16_t (&nxt)[QB], auto next_tag) {
+    // slot, sharing one LDS fragment), fenced so that the compiler keeps the order.  Fragment
+    // reads run two slots ahead through a ring of four registers that lives across blocks: a
+    // block expects the operands of its first two slots in flight and, in its last two slots,
+    // requests those of its successor (`tail`: KFirst = a block that starts with score MFMAs,
+    // VFirst = one that only has PV left, NoTail = the successor's rows are not resident yet).
+    // The 8*QB exp pairs (2 fma + 2 exp + cvt + dot2 each) are spread between the MFMAs so the
+    // matrix pipe has an instruction in flight while the VALU works.  P(s2=0) is complete
+    // before the first PV MFMA, P(s2=1) before the first PV MFMA that uses it; the row maxima
+    // of S(j+1) are reduced as a tree in the slots after the last exp pair, so the rescale
+    // decision is ready when the last MFMA issues.
+    i16x8 frag[4];
+    constexpr int NS = KSTEPS + 2 * DBLK;                 // slot c >= KSTEPS: PV(s2 = (c-KSTEPS)/DBLK, db = (c-KSTEPS)%DBLK)
+    static_assert(NS % 4 == 0 && KSTEPS % 4 == 0, "the fragment ring is indexed by slot % 4 across blocks");
+    // `par` is the parity of block j's tile (j >> 1): V(j) lives in the V buffer of that parity,
+    // the K rows of block j+1 in the K buffer of the other one.
+    auto fetch = [&](int j, int c, auto par) {            // operand of slot c of block j -> frag[c % 4]
+        if (c < KSTEPS) {
+            const std::uint16_t* kt = kbuf(par, true) + ((j + 2) & 1) * 32 * D;   // rows of block j+1
+            frag[c % 4] = *reinterpret_cast<const i16x8*>(kt + k_rd[c]);
+        } else {
+            const std::uint16_t* vt = vbuf(par, false) + (j & 1) * 32 * D;
+            const int s2 = (c - KSTEPS) / DBLK, db = (c - KSTEPS) % DBLK;
+            const std::uint16_t* vp = vt + v_rd[db] + 16 * s2 * D;
+            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
+            frag[c % 4] = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+    };
+    struct KFirst {}; struct VFirst {}; struct NoTail {};
+    auto first_fetches = [&](int j, auto kind, auto par) {   // what block j's first two slots consume
+        constexpr int s0 = std::is_same<decltype(kind), KFirst>::value ? 0 : KSTEPS;
+        fetch(j, s0, par);
+        fetch(j, s0 + 1, par);
+    };
+    auto block = [&](int j, float16_t (&cur)[QB], float16_t (&nxt)[QB], auto next_tag, auto tail, auto par) {
         constexpr bool kNext = decltype(next_tag)::value;
+        constexpr bool kTail = !std::is_same<decltype(tail), NoTail>::value;
         constexpr int S0 = kNext ? 0 : KSTEPS;           // first slot that exists
-        constexpr int NS = KSTEPS + 2 * DBLK;            // slot c >= KSTEPS: PV(s2 = (c-KSTEPS)/DBLK, db = (c-KSTEPS)%DBLK)
+        static_assert(QB == 1, "the max tree below is written for one query block per wave");
         float mc[QB];
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) mc[qb] = m_run[qb] * p.scale_log2;
-        const std::uint16_t* kt = &k_lds[((j + 2) >> 1) % NST][((j + 2) & 1) * 32 * D];   // rows of block j+1
-        const std::uint16_t* vt = &v_lds[(j >> 1) % NST][(j & 1) * 32 * D];
-        i16x8 frag[3];
         u32x4 pw[QB][2];
-        float mx[QB];
-        auto fetch = [&](int c) {                         // operand of slot c -> frag[c % 3]
-            if (c < KSTEPS) {
-                frag[c % 3] = *reinterpret_cast<const i16x8*>(kt + k_rd[c]);
-            } else {
-                const int s2 = (c - KSTEPS) / DBLK, db = (c - KSTEPS) % DBLK;
-                const std::uint16_t* vp = vt + v_rd[db] + 16 * s2 * D;
-                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
-                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
-                frag[c % 3] = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            }
-        };
+        float mx[QB], t3[5], t2[2];
         auto exp_pair = [&](int qb, int i) {              // elements 2i, 2i+1 of cur[qb]
             const float e0 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i], p.scale_log2, -mc[qb]));
             const float e1 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i + 1], p.scale_log2, -mc[qb]));
             const std::uint32_t w = Mma<T>::pack2(e0, e1);
             l_run[qb] = Mma<T>::add_pair(w, l_run[qb]);
+            asm volatile("" : "+v"(l_run[qb]));           // keeps the row-sum update in this slot
             pw[qb][i / 4][i % 4] = w;
         };
         // pair (qb, i) is issued just before the MFMAs of slot pair_slot(qb, i)
@@ -388,9 +406,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             if (i < 4) return kNext ? (qb * 4 + i) * KSTEPS / (4 * QB) : KSTEPS;
             return KSTEPS + (qb * 4 + i - 4) * DBLK / (4 * QB);
         };
+        constexpr int MAX0 = KSTEPS + DBLK + (DBLK >= 4 ? 1 : 0);   // after the last exp pair; S(j+1) finished KSTEPS slots ago
 
-        fetch(S0);
-        fetch(S0 + 1);
 #pragma unroll
         for (int c = S0; c < NS; ++c) {
 #pragma unroll
@@ -405,16 +422,33 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 #pragma unroll
                         for (int r = 0; r < 16; ++r) nxt[qb][r] = 0.f;
                     }
-                    nxt[qb] = Mma<T>::run(frag[c % 3], qreg[qb][c], nxt[qb]);
+                    nxt[qb] = Mma<T>::run(frag[c % 4], qreg[qb][c], nxt[qb]);
                 }
             } else {
                 const int s2 = (c - KSTEPS) / DBLK, db = (c - KSTEPS) % DBLK;
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb)
-                    oacc[qb][db] = Mma<T>::run(frag[c % 3], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
+                    oacc[qb][db] = Mma<T>::run(frag[c % 4], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
             }
-            if (c + 2 < NS) fetch(c + 2);
-            if (kNext && c >= NS - QB) mx[c - (NS - QB)] = lane_max(nxt[c - (NS - QB)]);
+            if (c + 2 < NS) fetch(j, c + 2, par);
+            else if constexpr (kTail)    // only ever the second block of the same tile: same parity
+                fetch(j + 1, (std::is_same<decltype(tail), KFirst>::value ? 0 : KSTEPS) + (c + 2 - NS), par);
+            if constexpr (kNext) {
+                const float16_t& sv = nxt[0];
+                if (c == MAX0) {
+#pragma unroll
+                    for (int g = 0; g < 5; ++g) {
+                        t3[g] = fmaxf(fmaxf(sv[3 * g], sv[3 * g + 1]), sv[3 * g + 2]);
+                        asm volatile("" : "+v"(t3[g]));   // keeps the reduction in this slot
+                    }
+                }
+                if (c == MAX0 + 1) {
+                    t2[0] = fmaxf(fmaxf(t3[0], t3[1]), t3[2]);
+                    t2[1] = fmaxf(fmaxf(t3[3], t3[4]), sv[15]);
+                    mx[0] = fmaxf(t2[0], t2[1]);
+                    asm volatile("" : "+v"(mx[0]));
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (kNext) finish_scores(j + 1, nxt, mx);
@@ -432,32 +466,52 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             for (int r = 0; r < 16; ++r) s_a[qb][r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks)
-                s_a[qb] = Mma<T>::run(*reinterpret_cast<const i16x8*>(&k_lds[0][32 * D + k_rd[ks]]), qreg[qb][ks], s_a[qb]);
+                s_a[qb] = Mma<T>::run(*reinterpret_cast<const i16x8*>(&k_lds0[32 * D + k_rd[ks]]), qreg[qb][ks], s_a[qb]);
             mx[qb] = lane_max(s_a[qb]);
         }
         finish_scores(0, s_a, mx);
     }
-    for (int t = 0; t + 1 < wave_tiles; ++t) {
-        const bool pending = stage_ahead(t);
-        block(2 * t, s_a, s_b, Yes{});
-        block(2 * t + 1, s_b, s_a, Yes{});
-        publish(pending);
+    // One tile of the main loop (`par` = parity of t, a compile-time name for the buffers; two
+    // tiles per trip).  The first fragment reads are in flight while the next pair is requested.
+    auto tile = [&](int t, auto par) {
+        first_fetches(2 * t, KFirst{}, par);
+        __builtin_amdgcn_sched_barrier(0);                // keep the reads ahead of the requests
+        stage_rows(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN - 32, kbuf(par, false));   // = stage_pair(t + 1)
+        stage_rows(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true));
+        block(2 * t, s_a, s_b, Yes{}, KFirst{}, par);
+        block(2 * t + 1, s_b, s_a, Yes{}, NoTail{}, par); // its successor's K rows arrive with the barrier below
+        publish();
+    };
+    int t_main = 0;
+    for (; t_main + 2 < wave_tiles; t_main += 2) {
+        tile(t_main, Par0{});
+        tile(t_main + 1, Par1{});
+    }
+    if (t_main + 1 < wave_tiles) {
+        tile(t_main, Par0{});
+        ++t_main;
     }
     if (wave_tiles > 0) {  // the wave's last tile: nothing to compute ahead in its second block
         const int t = wave_tiles - 1;
-        const bool pending = stage_ahead(t);
+        const AnyPar par{t};
+        if (t + 1 < n_tiles) stage_pair(t + 1, AnyPar{t + 1});
         // The tile's second block contributes nothing when it starts past the end of K or, for a
         // causal wave, past the wave's last query (every other wave's diagonal tile).
         const int second0 = (2 * t + 1) * 32;
         if (second0 >= p.Lk || (kCausal && second0 > q0 + WQ - 1)) {
-            block(2 * t, s_a, s_b, No{});
+            first_fetches(2 * t, VFirst{}, par);
+            block(2 * t, s_a, s_b, No{}, NoTail{}, par);
         } else {
-            block(2 * t, s_a, s_b, Yes{});
-            block(2 * t + 1, s_b, s_a, No{});
+            first_fetches(2 * t, KFirst{}, par);
+            block(2 * t, s_a, s_b, Yes{}, VFirst{}, par);
+            block(2 * t + 1, s_b, s_a, No{}, NoTail{}, par);
         }
-        publish(pending);
+        publish();
     }
-    for (int t = wave_tiles; t < n_tiles; ++t) publish(stage_ahead(t));
+    for (int t = wave_tiles; t < n_tiles; ++t) {           // done early (causal): keep staging for the other waves
+        if (t + 1 < n_tiles) stage_pair(t + 1, AnyPar{t + 1});
+        publish();
+    }
 
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -509,6 +563,12 @@ bool flash_supported(const paras_sdpa_args& a) {
     if (!mult8(a.q_strides) || !mult8(a.k_strides) || !mult8(a.v_strides)) return false;
     const int64_t nq = (a.Lq + kBM - 1) / kBM;
     if (a.B * a.Hq * nq > 0x7fffffffLL || a.Lq > 0x3fffffff || a.Lk > 0x3fffffff) return false;
+    // K / V tiles are fetched with 32-bit byte offsets against a buffer descriptor per (batch, head)
+    // that spans rows [0, Lk); offsets of rows up to one tile outside it must not wrap into it.
+    for (const int64_t* st : {a.k_strides, a.v_strides}) {
+        if (st[2] < 0) return false;
+        if ((a.Lk + 2 * kBN) * st[2] * 2 + a.D * 2 >= 0x7fffffffLL) return false;
+    }
     return true;
 }
 
