@@ -8,9 +8,10 @@
 //   workgroup = 4 wavefronts = 128 queries of one (batch, head); each wave owns
 //   32 queries.  K/V are streamed in tiles of 64 keys through LDS (two buffers
 //   each, one barrier per tile), shared by the 4 waves.  Tiles go from global
-//   memory straight into LDS (global_load_lds_dwordx4: no staging registers, no
-//   LDS store instructions); rows are unpadded and the 16-byte chunks of a row
-//   are XOR-swizzled so that operand reads stay conflict free.
+//   memory straight into LDS (buffer_load_dwordx4 ... lds: no staging registers,
+//   no LDS store instructions; the buffer descriptor's range check supplies the
+//   zeros for rows outside [0, Lk)); rows are unpadded and the 16-byte chunks of a
+//   row are XOR-swizzled so that operand reads stay conflict free.
 //
 // The products are formed transposed so that a lane always owns ONE query:
 //   S^T = K Q^T    A = K tile from LDS (lane: key l%32, 8 consecutive d),
@@ -45,7 +46,17 @@
 // work of the same wave.  K is staged half a tile ahead of V: K tile u holds
 // keys [64u-32, 64u+32), so the two blocks whose scores are computed during V
 // tile t (blocks 2t+1, 2t+2) both live in K tile t+1, and K and V need only two
-// LDS buffers each with a single barrier per tile.
+// LDS buffers each with a single barrier per tile.  The operand fragments run
+// through a register ring that carries across the two blocks of a tile, and a
+// tile's first fragments are requested before the next tile pair is.
+//
+// Three things in the structure exist to keep the compiler's wait insertion
+// exact (it is conservative in ways that serialise this loop otherwise): the
+// tiles come through buffer loads (an LDS-direct global load makes every later
+// LDS wait a full one), each buffer is its own __shared__ array named at
+// compile time in the main loop (an LDS read waits for all direct loads in
+// flight unless the variables prove them disjoint), and nothing with a branch
+// sits between a fragment's request and the MFMA that consumes it.
 //
 // v_mfma_f32_32x32x16_{bf16,f16}: 32 MFMAs per wave per 64-key tile at D=128.
 #include <hip/hip_runtime.h>

@@ -134,6 +134,33 @@ def test_flash_strided_inputs_and_explicit_scale():
     assert kern == "flash_mfma" and max_abs(out, want) <= ABS_16BIT
 
 
+@pytest.mark.parametrize("Lk", [77, 191, 300])
+def test_flash_never_reads_past_the_last_key(Lk):
+    """K / V as views of larger buffers whose rows past Lk hold NaN: the tiles that hang over the
+    end of K must be completed with zeros, not with what lies behind the last key."""
+    B, H, Lq, D = 2, 3, 200, 128
+    q = torch.randn(B, H, Lq, D).bfloat16()
+    k, v = torch.randn(B, H, Lk, D).bfloat16(), torch.randn(B, H, Lk, D).bfloat16()
+    kbuf = torch.full((B, H, Lk + 130, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    vbuf = torch.full((B, H, Lk + 130, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kbuf[:, :, :Lk], vbuf[:, :, :Lk] = k.cuda(), v.cuda()
+    for causal in (False, True):
+        out, _, _, kern = capi.sdpa(q.cuda(), kbuf[:, :, :Lk], vbuf[:, :, :Lk], is_causal=causal)
+        want, _ = O.sdpa_math(q, k, v, is_causal=causal, gemm="aten")
+        assert kern == "flash_mfma"
+        assert bool(torch.isfinite(out).all()) and max_abs(out, want) <= ABS_16BIT
+
+
+def test_flash_broadcast_key_rows():
+    """Row stride 0 (one key / value row expanded over Lk): every key is the same row."""
+    B, H, Lq, Lk, D = 1, 2, 96, 150, 64
+    q = torch.randn(B, H, Lq, D).half()
+    k1, v1 = torch.randn(B, H, 1, D).half(), torch.randn(B, H, 1, D).half()
+    out, _, _, kern = capi.sdpa(q.cuda(), k1.cuda().expand(B, H, Lk, D), v1.cuda().expand(B, H, Lk, D), is_causal=False)
+    want, _ = O.sdpa_math(q, k1.expand(B, H, Lk, D).contiguous(), v1.expand(B, H, Lk, D).contiguous(), gemm="aten")
+    assert kern == "flash_mfma" and max_abs(out, want) <= ABS_16BIT
+
+
 DECODE_SHAPES = [(2, 8, 2, 1, 1000), (1, 4, 4, 1, 77), (3, 32, 8, 1, 2048), (1, 8, 2, 2, 300), (2, 16, 1, 1, 129), (1, 2, 2, 8, 5000)]
 
 
