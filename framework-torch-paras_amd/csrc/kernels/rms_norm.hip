@@ -57,8 +57,9 @@ __device__ __forceinline__ double rsqrt_f64(double v) {
 }
 
 // Register-resident row: H == vectors per row * kVec, vectors per row <= kBlock*NV.
+// (Four vectors per thread need more than the 64 registers that eight waves per SIMD leave.)
 template <typename T, int NV>
-__global__ __launch_bounds__(kBlock, 8) void rms_norm_fwd_vec(
+__global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
     const typename Elem<T>::store_t* __restrict__ x, const typename Elem<T>::store_t* __restrict__ w,
     typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, int H,
     double eps, double inv_h) {
