@@ -38,3 +38,13 @@ def test_no_device_means_error_not_fallback():
         torch.randn(4).to("paras")
     with pytest.raises(RuntimeError):
         torch.empty(4, device="paras:0")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU per box: asking bench.py for more must end with a message, not a rendezvous."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parents[1]
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
