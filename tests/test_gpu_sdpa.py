@@ -161,6 +161,44 @@ def test_flash_broadcast_key_rows():
     assert kern == "flash_mfma" and max_abs(out, want) <= ABS_16BIT
 
 
+def test_flash_random_shapes_layouts_and_padding():
+    """Forty seeded random cases (ragged lengths around the 32 / 64 / 128 tile edges, GQA ratios,
+    [B,L,H,D] views, rows embedded in NaN-filled buffers, explicit scales) against an fp32 torch
+    evaluation of softmax(q k^T s + causal) v on the same device: the tolerance is the 16-bit bar."""
+    import random
+    rng = random.Random(1)
+    g = torch.Generator(device="cuda").manual_seed(1)
+
+    def rnd(*shape, dt):
+        return torch.randn(*shape, device="cuda", generator=g).to(dt)
+
+    for _ in range(40):
+        D, dt = rng.choice([64, 128]), rng.choice([torch.bfloat16, torch.float16])
+        Hkv, rep, B = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 4]), rng.choice([1, 2, 3])
+        Hq = Hkv * rep
+        Lq = rng.choice([2, 5, 31, 32, 33, 64, 100, 127, 128, 129, 200, 255, 256, 257, 384, 500, 513])
+        Lk = rng.choice([2, 31, 32, 33, 63, 64, 65, 96, 100, 127, 128, 129, 160, 191, 192, 193, 255, 256, 300, 511, 512, 640])
+        causal, layout, scale = rng.random() < 0.6, rng.choice(["bhld", "blhd", "padded"]), rng.choice([None, 0.05, 0.2])
+        if layout == "bhld":
+            q, k, v = rnd(B, Hq, Lq, D, dt=dt), rnd(B, Hkv, Lk, D, dt=dt), rnd(B, Hkv, Lk, D, dt=dt)
+        elif layout == "blhd":
+            q, k, v = (rnd(B, L, H, D, dt=dt).permute(0, 2, 1, 3) for L, H in ((Lq, Hq), (Lk, Hkv), (Lk, Hkv)))
+        else:
+            q = rnd(B, Hq, Lq, D + 8, dt=dt)[..., :D]
+            kb = torch.full((B, Hkv, Lk + 70, D + 16), float("nan"), device="cuda", dtype=dt)
+            vb = torch.full((B, Hkv, Lk + 70, D + 16), float("nan"), device="cuda", dtype=dt)
+            kb[:, :, :Lk, :D], vb[:, :, :Lk, :D] = rnd(B, Hkv, Lk, D, dt=dt), rnd(B, Hkv, Lk, D, dt=dt)
+            k, v = kb[:, :, :Lk, :D], vb[:, :, :Lk, :D]
+        out, _, _, kern = capi.sdpa(q, k, v, is_causal=causal, scale=scale)
+        s = (q.float() @ k.float().repeat_interleave(rep, 1).transpose(-1, -2)) * (scale if scale is not None else 1 / math.sqrt(D))
+        if causal:
+            s = s.masked_fill(~torch.ones(Lq, Lk, device="cuda").tril().bool(), -math.inf)
+        want = torch.softmax(s, -1) @ v.float().repeat_interleave(rep, 1)
+        case_id = f"B={B} Hq={Hq} Hkv={Hkv} Lq={Lq} Lk={Lk} D={D} {dt} causal={causal} {layout} scale={scale}"
+        assert kern in ("flash_mfma", "decode_split"), case_id     # a handful of queries goes to the decode kernel
+        assert bool(torch.isfinite(out).all()) and float((out.float() - want).abs().max()) <= ABS_16BIT, case_id
+
+
 DECODE_SHAPES = [(2, 8, 2, 1, 1000), (1, 4, 4, 1, 77), (3, 32, 8, 1, 2048), (1, 8, 2, 2, 300), (2, 16, 1, 1, 129), (1, 2, 2, 8, 5000)]
 
 
