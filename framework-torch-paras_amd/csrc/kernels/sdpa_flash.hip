@@ -58,6 +58,13 @@
 // flight unless the variables prove them disjoint), and nothing with a branch
 // sits between a fragment's request and the MFMA that consumes it.
 //
+// An optional mask (bytes, nonzero = attend; or additive values of the tensor type;
+// broadcast over any of batch / head / query, contiguous along the keys) is applied
+// to the finished scores of a block; the mask bytes of block j+1 are requested when
+// block j starts.  Queries with no visible key so far carry a running maximum of
+// -inf and contribute zeros; a query with no visible key at all ends as 0/0 = NaN,
+// like the reference's softmax.
+//
 // v_mfma_f32_32x32x16_{bf16,f16}: 32 MFMAs per wave per 64-key tile at D=128.
 #include <hip/hip_runtime.h>
 
@@ -91,6 +98,11 @@ struct FlashParams {
     int  n_qblocks;
     float scale_log2;  // scale * log2(e)
     float scale;
+    // optional mask over [B, Hq, Lq, Lk] (element strides; 0 = broadcast): bytes (nonzero = attend)
+    // or additive values of the tensor dtype
+    const unsigned char* mask;
+    long ms_b, ms_h, ms_q, ms_k;
+    float inv_scale;   // the scores are kept unscaled: an additive mask value m enters as m / scale
 };
 
 template <typename T> struct Mma;
@@ -155,8 +167,10 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return lo + hi;
 }
 
-template <typename T, int D, bool kCausal>
+// kMask: 0 none, 1 bytes (nonzero = attend), 2 additive values of type T.
+template <typename T, int D, bool kCausal, int kMask>
 __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) {
+    static_assert(!(kCausal && kMask != 0), "a mask and the causal rule are mutually exclusive");
     // 32-query blocks per wave.  The code is written for any QB; 2 halves the LDS operand
     // traffic per query but needs one wave per SIMD and measured 30 % slower (nothing hides
     // LDS / barrier latency then), so 1 it is: two waves per SIMD, 256 registers each.
@@ -318,6 +332,53 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         for (int r = 0; r < 16; ++r)
             if ((r >> 2) * 8 + (r & 3) > rel) sc[r] = -INFINITY;
     };
+    // ---- optional user mask.  Lane (query, half lh) needs, for block j, keys j*32 + 8g + 4 lh + i
+    // (g, i = 0..3; accumulator register 4g + i): four runs of four consecutive keys.  The runs of
+    // block j+1 are requested at the start of block j and applied when its scores are finished.
+    constexpr int MREGS = kMask == 0 ? 1 : (kMask == 1 ? 4 : 8);
+    const unsigned char* mrow = nullptr;
+    if constexpr (kMask != 0) {
+        const int my_q = q0 + lq;
+        const long qrow = my_q < p.Lq ? my_q : p.Lq - 1;
+        mrow = p.mask + (static_cast<long>(b) * p.ms_b + static_cast<long>(hq) * p.ms_h + qrow * p.ms_q) * (kMask == 1 ? 1 : 2);
+    }
+    // The mask is contiguous along the keys and Lk >= 4 (flash_supported): a run that hangs over the
+    // end of the row is read from the row's last four elements and shifted down, so no load leaves
+    // the row and no branch is needed; keys >= Lk get zero bits and are masked by the end-of-K rule.
+    auto mask_load = [&](int j, std::uint32_t (&mr)[MREGS]) {
+        if constexpr (kMask != 0) {
+            typedef std::uint32_t u32_any __attribute__((aligned(1)));
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int key = j * 32 + 8 * g + 4 * lh;
+                const int at = min(key, p.Lk - 4);
+                const unsigned sh = static_cast<unsigned>(key - at);          // 0 unless the run hangs over
+                if constexpr (kMask == 1) {
+                    const std::uint32_t w = *reinterpret_cast<const u32_any*>(mrow + at);
+                    mr[g] = sh < 4 ? w >> (8 * sh) : 0u;
+                } else {
+                    const std::uint64_t w = static_cast<std::uint64_t>(*reinterpret_cast<const u32_any*>(mrow + 2 * at)) |
+                                            (static_cast<std::uint64_t>(*reinterpret_cast<const u32_any*>(mrow + 2 * at + 4)) << 32);
+                    const std::uint64_t v = sh < 4 ? w >> (16 * sh) : 0ull;
+                    mr[2 * g] = static_cast<std::uint32_t>(v);
+                    mr[2 * g + 1] = static_cast<std::uint32_t>(v >> 32);
+                }
+            }
+        }
+    };
+    auto mask_apply = [&](const std::uint32_t (&mr)[MREGS], float16_t& sc) {
+        if constexpr (kMask == 1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (((mr[r >> 2] >> (8 * (r & 3))) & 0xffu) == 0) sc[r] = -INFINITY;
+        } else if constexpr (kMask == 2) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const std::uint16_t bits = static_cast<std::uint16_t>(mr[r >> 1] >> (16 * (r & 1)));
+                sc[r] = fmaf(Elem<T>::to_f32(bits), p.inv_scale, sc[r]);
+            }
+        }
+    };
     auto lane_max = [](const float16_t& sc) {
         float mx = sc[0];
 #pragma unroll
@@ -337,7 +398,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
                 const float m_new = fmaxf(m_run[qb], mloc[qb]);
-                const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.scale_log2);
+                // (equal covers -inf on both sides: a query that has seen no key yet keeps its zeros)
+                const float alpha = m_run[qb] == m_new ? 1.f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.scale_log2);
                 m_run[qb] = m_new;
                 l_run[qb] *= alpha;
 #pragma unroll
@@ -348,13 +410,13 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         }
     };
     // Mask where needed, then raise.  `mx` holds the unmasked in-lane maxima on entry.
-    auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB]) {
+    auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB], const std::uint32_t (&mr)[MREGS]) {
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-            if (needs_mask(j, qb)) {
-                apply_mask(j, qb, sc[qb]);
-                mx[qb] = lane_max(sc[qb]);
-            }
+        for (int qb = 0; qb < QB; ++qb) {
+            if constexpr (kMask != 0) mask_apply(mr, sc[qb]);
+            if (needs_mask(j, qb)) apply_mask(j, qb, sc[qb]);
+            if (kMask != 0 || needs_mask(j, qb)) mx[qb] = lane_max(sc[qb]);
+        }
         raise_max(mx);
     };
 
@@ -401,7 +463,13 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         static_assert(QB == 1, "the max tree below is written for one query block per wave");
         float mc[QB];
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) mc[qb] = m_run[qb] * p.scale_log2;
+        for (int qb = 0; qb < QB; ++qb) {
+            mc[qb] = m_run[qb] * p.scale_log2;
+            // every key so far masked out: the reference point is arbitrary, and it must not be -inf
+            if constexpr (kMask != 0) mc[qb] = m_run[qb] == -INFINITY ? 0.f : mc[qb];
+        }
+        std::uint32_t mnext[MREGS];
+        if constexpr (kNext) mask_load(j + 1, mnext);
         u32x4 pw[QB][2];
         float mx[QB], t3[5], t2[2];
         auto exp_pair = [&](int qb, int i) {              // elements 2i, 2i+1 of cur[qb]
@@ -444,7 +512,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             if (c + 2 < NS) fetch(j, c + 2, par);
             else if constexpr (kTail)    // only ever the second block of the same tile: same parity
                 fetch(j + 1, (std::is_same<decltype(tail), KFirst>::value ? 0 : KSTEPS) + (c + 2 - NS), par);
-            if constexpr (kNext) {
+            if constexpr (kNext && kMask == 0) {      // (with a user mask the maxima are taken after masking)
                 const float16_t& sv = nxt[0];
                 if (c == MAX0) {
 #pragma unroll
@@ -462,7 +530,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (kNext) finish_scores(j + 1, nxt, mx);
+        if constexpr (kNext) finish_scores(j + 1, nxt, mx, mnext);
     };
     using Yes = std::true_type;
     using No  = std::false_type;
@@ -480,7 +548,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
                 s_a[qb] = Mma<T>::run(*reinterpret_cast<const i16x8*>(&k_lds0[32 * D + k_rd[ks]]), qreg[qb][ks], s_a[qb]);
             mx[qb] = lane_max(s_a[qb]);
         }
-        finish_scores(0, s_a, mx);
+        std::uint32_t m0[MREGS];
+        mask_load(0, m0);
+        finish_scores(0, s_a, mx, m0);
     }
     // One tile of the main loop (`par` = parity of t, a compile-time name for the buffers; two
     // tiles per trip).  The first fragment reads are in flight while the next pair is requested.
@@ -548,13 +618,14 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 }
 
 template <typename T, int D>
-int launch_t(FlashParams p, bool causal, hipStream_t s) {
+int launch_t(FlashParams p, bool causal, int mask_kind, hipStream_t s) {
     p.n_qblocks = (p.Lq + kBM - 1) / kBM;
     const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
-    if (causal)
-        hipLaunchKernelGGL((flash_fwd_kernel<T, D, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, p);
-    else
-        hipLaunchKernelGGL((flash_fwd_kernel<T, D, false>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, p);
+    const dim3 grid(static_cast<unsigned>(blocks)), wg(256);
+    if (causal)              hipLaunchKernelGGL((flash_fwd_kernel<T, D, true, 0>), grid, wg, 0, s, p);
+    else if (mask_kind == 1) hipLaunchKernelGGL((flash_fwd_kernel<T, D, false, 1>), grid, wg, 0, s, p);
+    else if (mask_kind == 2) hipLaunchKernelGGL((flash_fwd_kernel<T, D, false, 2>), grid, wg, 0, s, p);
+    else                     hipLaunchKernelGGL((flash_fwd_kernel<T, D, false, 0>), grid, wg, 0, s, p);
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
 }
@@ -567,7 +638,10 @@ bool mult8(const int64_t* strides) { return strides[0] % 8 == 0 && strides[1] % 
 bool flash_supported(const paras_sdpa_args& a) {
     if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
     if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
-    if (a.mask_kind != 0 || a.attn != nullptr) return false;
+    if (a.attn != nullptr) return false;                            // the weights are never formed here
+    if (a.mask_kind != 0 && (a.mask == nullptr || a.is_causal)) return false;
+    if (a.mask_kind < 0 || a.mask_kind > 2) return false;
+    if (a.mask_kind != 0 && (a.mask_strides[3] != 1 || a.Lk < 4)) return false;   // mask runs are read four keys at a time
     if (a.Lq < 1 || a.Lk < 1) return false;
     if (!(a.scale > 0.0) || !std::isfinite(a.scale)) return false;  // the running max is taken on raw scores
     if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.out)) return false;
@@ -598,10 +672,14 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     p.n_qblocks = 0;  // set by the launcher for the workgroup size it picks
     p.scale = static_cast<float>(a.scale);
     p.scale_log2 = static_cast<float>(a.scale * 1.4426950408889634);
+    p.mask = static_cast<const unsigned char*>(a.mask);
+    p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2]; p.ms_k = a.mask_strides[3];
+    p.inv_scale = static_cast<float>(1.0 / a.scale);
     const bool causal = a.is_causal != 0;
+    const int mk = a.mask_kind;
     if (a.dtype == PARAS_BF16)
-        return a.D == 128 ? launch_t<bf16_t, 128>(p, causal, s) : launch_t<bf16_t, 64>(p, causal, s);
-    return a.D == 128 ? launch_t<f16_t, 128>(p, causal, s) : launch_t<f16_t, 64>(p, causal, s);
+        return a.D == 128 ? launch_t<bf16_t, 128>(p, causal, mk, s) : launch_t<bf16_t, 64>(p, causal, mk, s);
+    return a.D == 128 ? launch_t<f16_t, 128>(p, causal, mk, s) : launch_t<f16_t, 64>(p, causal, mk, s);
 }
 
 }  // namespace paras

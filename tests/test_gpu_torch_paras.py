@@ -92,6 +92,24 @@ def test_sdpa_bool_mask(device):
                  F.scaled_dot_product_attention(q, k, v, attn_mask=m2), "broadcast bool mask")
 
 
+def test_sdpa_bf16_key_padding_mask_and_bias(device):
+    """The shapes a padded batch produces: bf16, a [B, 1, 1, Lk] bool mask, then an fp32 additive
+    bias (converted to the tensors' dtype, attention_ops.cpp:122-125).  Checked against torch's
+    own CPU result on the same bf16 inputs evaluated in fp32."""
+    B, H, L, D = 2, 4, 160, 64
+    q, k, v = (torch.randn(B, H, L, D).bfloat16() for _ in range(3))
+    lengths = torch.tensor([160, 97])
+    pad = torch.arange(L)[None, :] < lengths[:, None]                 # [B, L]
+    mask = pad[:, None, None, :]
+    got = F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), attn_mask=mask.to(device)).cpu()
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask)
+    assert got.dtype == torch.bfloat16 and float((got.float() - want).abs().max()) <= 2e-2
+    bias = torch.randn(1, H, L, L) * 0.5
+    got = F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), attn_mask=bias.to(device)).cpu()
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=bias.bfloat16().float())
+    assert float((got.float() - want).abs().max()) <= 2e-2
+
+
 def test_sdpa_additive_mask(device):
     q, k, v, dq, dk, dv = _qkv(device)
     bias = torch.randn(2, 4, 8, 8) * 0.1
