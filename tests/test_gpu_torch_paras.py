@@ -110,6 +110,23 @@ def test_sdpa_bf16_key_padding_mask_and_bias(device):
     assert float((got.float() - want).abs().max()) <= 2e-2
 
 
+@pytest.mark.parametrize("D", [96, 80, 40])
+def test_sdpa_16bit_other_head_sizes_run_zero_padded(device, D):
+    """Head sizes other than 64 / 128 go through the MFMA kernels with zero columns appended
+    (the default scale stays 1/sqrt(D) of the real size); results as for any other 16-bit call."""
+    B, H, L = 2, 3, 150
+    q, k, v = (torch.randn(B, H, L, D).half() for _ in range(3))
+    got = F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), is_causal=True).cpu()
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True)
+    assert got.shape == (B, H, L, D) and got.dtype == torch.float16 and got.is_contiguous()
+    assert float((got.float() - want).abs().max()) <= 2e-2
+    mask = torch.rand(B, 1, L, L) > 0.4
+    mask[..., 0] = True
+    got = F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), attn_mask=mask.to(device), scale=0.2).cpu()
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask, scale=0.2)
+    assert float((got.float() - want).abs().max()) <= 2e-2
+
+
 def test_sdpa_additive_mask(device):
     q, k, v, dq, dk, dv = _qkv(device)
     bias = torch.randn(2, 4, 8, 8) * 0.1
