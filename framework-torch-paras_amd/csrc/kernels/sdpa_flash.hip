@@ -32,8 +32,8 @@
 //                  exponent domain, so after the first block the rescale is
 //                  skipped almost always; the same (possibly stale) max is used
 //                  for P and for the row sum, so out = O / l is unchanged.
-//   row sums       v_dot2_f32_{bf16,f16} on the packed 16-bit P (two elements
-//                  per instruction, and exactly the values the PV product uses)
+//   row sums       fp32 adds of the exponentials before they are rounded to the
+//                  16-bit operand of the PV product
 //
 // Software pipeline inside a wave: the unit of work is a 32-key block and the
 // score MFMAs run one block ahead,
@@ -117,12 +117,6 @@ template <> struct Mma<bf16_t> {
         const f32x2 v = {lo, hi};
         return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, bf16x2));
     }
-    // acc + both halves of a packed pair
-    __device__ static __forceinline__ float add_pair(std::uint32_t pk, float acc) {
-        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        const bf16x2 ones = {static_cast<__bf16>(1.0f), static_cast<__bf16>(1.0f)};
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), ones, acc, false);
-    }
 };
 template <> struct Mma<f16_t> {
     __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
@@ -134,11 +128,6 @@ template <> struct Mma<f16_t> {
         typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
         const f32x2 v = {lo, hi};
         return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, f16x2));
-    }
-    __device__ static __forceinline__ float add_pair(std::uint32_t pk, float acc) {
-        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-        const f16x2 ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), ones, acc, false);
     }
 };
 
@@ -427,7 +416,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     // block expects the operands of its first two slots in flight and, in its last two slots,
     // requests those of its successor (`tail`: KFirst = a block that starts with score MFMAs,
     // VFirst = one that only has PV left, NoTail = the successor's rows are not resident yet).
-    // The 8*QB exp pairs (2 fma + 2 exp + cvt + dot2 each) are spread between the MFMAs so the
+    // The 8*QB exp pairs (2 fma + 2 exp + cvt + 2 add each) are spread between the MFMAs so the
     // matrix pipe has an instruction in flight while the VALU works.  P(s2=0) is complete
     // before the first PV MFMA, P(s2=1) before the first PV MFMA that uses it; the row maxima
     // of S(j+1) are reduced as a tree in the slots after the last exp pair, so the rescale
@@ -476,7 +465,10 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             const float e0 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i], p.scale_log2, -mc[qb]));
             const float e1 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i + 1], p.scale_log2, -mc[qb]));
             const std::uint32_t w = Mma<T>::pack2(e0, e1);
-            l_run[qb] = Mma<T>::add_pair(w, l_run[qb]);
+            // Plain adds of the unrounded exponentials: v_dot2_f32_bf16 on the packed pair is one
+            // instruction instead of two, but it runs on the matrix pipe's side and stalls the
+            // MFMA next to it (measured: 4 % of the kernel).
+            l_run[qb] += e0 + e1;
             asm volatile("" : "+v"(l_run[qb]));           // keeps the row-sum update in this slot
             pw[qb][i / 4][i % 4] = w;
         };
