@@ -396,18 +396,17 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     // (rare after the first block): O and l are rescaled, and `sc` itself, which was formed
     // against the old reference, is shifted to the new one.
     auto raise_max = [&](float (&mx)[QB], float16_t (&sc)[QB]) {
+        // The test runs on each lane's own half of the keys; the two halves of a query are only
+        // brought together (and `seen` updated) inside the rare branch.
         bool grow = false;
-        float mloc[QB];
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-            mloc[qb] = half_swap_max(mx[qb]);
-            grow = grow || (seen ? mloc[qb] > lazy_margin : mloc[qb] > -INFINITY);
-        }
+        for (int qb = 0; qb < QB; ++qb) grow = grow || (seen ? mx[qb] > lazy_margin : mx[qb] > -INFINITY);
         if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // wave-uniform
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
+                const float mloc = half_swap_max(mx[qb]);
                 // lanes that need no move still take any upward one; an all-masked block moves nothing
-                const float delta = seen ? fmaxf(mloc[qb], 0.f) : (mloc[qb] > -INFINITY ? mloc[qb] : 0.f);
+                const float delta = seen ? fmaxf(mloc, 0.f) : (mloc > -INFINITY ? mloc : 0.f);
                 const float alpha = __builtin_amdgcn_exp2f(-delta);
                 m_run[qb] += delta;
                 l_run[qb] *= alpha;
@@ -420,9 +419,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
                     sc[qb][r] -= delta;
                     sinit[qb][r] = -m_run[qb];
                 }
+                if (qb == 0) seen = seen || mloc > -INFINITY;
             }
         }
-        seen = seen || mloc[0] > -INFINITY;
     };
     // Mask where needed, then raise.  `mx` holds the unmasked in-lane maxima on entry.
     auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB], const std::uint32_t (&mr)[MREGS]) {
