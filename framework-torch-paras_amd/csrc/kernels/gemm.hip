@@ -31,21 +31,23 @@ struct DenseParams {
     long M, N, K;
     long lda, ldb, ldc, ld_add;
     long sa, sb, sc, sadd;      // batch strides (elements)
-    int  m_tiles, n_units;      // 128-row tiles, 256-column units
+    int  m_tiles, n_units;      // row tiles (128 or 256 rows), 256-column units
     float alpha, beta;
 };
 
-template <typename T>
-__global__ __launch_bounds__(kThreads, 2) void dense_gemm_nt_kernel(const DenseParams p) {
+// S = Tile128 (4 waves, 128 rows) or Tile256 (8 waves, 256 rows; for problems with enough
+// 256 x 256 tiles to fill the chip).
+template <typename T, typename S>
+__global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const DenseParams p) {
     using El = Elem<T>;
-    __shared__ __attribute__((aligned(16))) TileLds lds;
+    __shared__ __attribute__((aligned(16))) typename S::Lds lds;
 
     // Column units innermost: the workgroups running together share the A row panel
     // (and, across m-tiles, stream the same B panels through L2).
     const long per_batch = static_cast<long>(p.m_tiles) * p.n_units;
     const long bidx = blockIdx.x / per_batch, rem = blockIdx.x % per_batch;
     const int mt = static_cast<int>(rem / p.n_units), nu = static_cast<int>(rem % p.n_units);
-    const long row0 = static_cast<long>(mt) * kBM, n0 = static_cast<long>(nu) * 2 * kBN;
+    const long row0 = static_cast<long>(mt) * S::kBM, n0 = static_cast<long>(nu) * 2 * kBN;
     const std::uint16_t* A = p.a + bidx * p.sa;
     const std::uint16_t* B = p.b + bidx * p.sb;
 
@@ -53,23 +55,26 @@ __global__ __launch_bounds__(kThreads, 2) void dense_gemm_nt_kernel(const DenseP
     const int lr = lane & 31, lh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    unsigned a_off[4], b_off[2][4];
+    unsigned a_off[4], b_off[2][S::kBChunks];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int c = tid + i * kThreads;
+        const int c = tid + i * S::kThreads;
         long arow = row0 + (c >> 3);
         if (arow >= p.M) arow = p.M - 1;     // clamped rows are computed but never stored
         a_off[i] = static_cast<unsigned>(arow * p.lda + (c & 7) * 8);
+    }
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int i = 0; i < S::kBChunks; ++i) {
+            const int c = tid + i * S::kThreads;
             long brow = n0 + g * kBN + (c >> 3);
             if (brow >= p.N) brow = p.N - 1;
             b_off[g][i] = static_cast<unsigned>(brow * p.ldb + (c & 7) * 8);
         }
-    }
     const std::uint16_t* const b_base[2] = {B, B};
     float16_t acc[2][2][2];
-    tile_mainloop<T>(A, a_off, b_base, b_off, p.K, lds, acc);
+    S::template mainloop<T>(A, a_off, b_base, b_off, p.K, lds, acc);
 
     std::uint16_t* C = p.c + bidx * p.sc;
     const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
@@ -90,6 +95,11 @@ __global__ __launch_bounds__(kThreads, 2) void dense_gemm_nt_kernel(const DenseP
                     C[row * p.ldc + col] = El::from_f32(v);
                 }
             }
+}
+
+template <typename T, typename S>
+void launch_dense(const DenseParams& p, unsigned grid, hipStream_t s) {
+    hipLaunchKernelGGL((dense_gemm_nt_kernel<T, S>), dim3(grid), dim3(S::kThreads), 0, s, p);
 }
 
 }  // namespace
@@ -114,7 +124,11 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) != 0 || lda % 8 != 0 || ldb % 8 != 0 ||
         stride_a % 8 != 0 || stride_b % 8 != 0)
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
-    const int64_t m_tiles = (M + gemm::kBM - 1) / gemm::kBM, n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
+    const int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
+    const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
+    const bool use_wide = wide_tiles >= 2 * 256;   // at least two rounds of one workgroup per CU
+    const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
+    const int64_t m_tiles = (M + bm - 1) / bm;
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
     if (M * lda >= (1LL << 32) || N * ldb >= (1LL << 32))
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: an operand matrix spans 2^32 elements or more");
@@ -131,9 +145,14 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     p.sa = stride_a; p.sb = stride_b; p.sc = stride_c; p.sadd = stride_add;
     p.m_tiles = static_cast<int>(m_tiles); p.n_units = static_cast<int>(n_units);
     p.alpha = static_cast<float>(alpha); p.beta = static_cast<float>(beta);
-    const dim3 grid(static_cast<unsigned>(m_tiles * n_units * batch));
-    if (dtype == PARAS_BF16) hipLaunchKernelGGL((dense_gemm_nt_kernel<bf16_t>), grid, dim3(gemm::kThreads), 0, s, p);
-    else                     hipLaunchKernelGGL((dense_gemm_nt_kernel<f16_t>), grid, dim3(gemm::kThreads), 0, s, p);
+    const unsigned blocks = static_cast<unsigned>(m_tiles * n_units * batch);
+    if (use_wide) {
+        if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile256>(p, blocks, s);
+        else                     launch_dense<f16_t, gemm::Tile256>(p, blocks, s);
+    } else {
+        if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile128>(p, blocks, s);
+        else                     launch_dense<f16_t, gemm::Tile128>(p, blocks, s);
+    }
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
 }

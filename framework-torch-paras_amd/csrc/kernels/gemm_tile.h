@@ -1,16 +1,20 @@
-// Tile mainloop shared by the MFMA GEMM kernels (grouped expert GEMMs and the
-// dense NT GEMM): C tile = A[128 x K] * B[256 x K]^T with bf16/fp16 operands and
+// Tile mainloops shared by the MFMA GEMM kernels (grouped expert GEMMs and the
+// dense NT GEMM): C tile = A[rows x K] * B[256 x K]^T with bf16/fp16 operands and
 // fp32 accumulation on v_mfma_f32_32x32x16.
 //
 // Both operands are read along their contiguous contraction dim, which is the
 // 8-element-per-lane operand layout of the MFMA, so neither needs a transpose.
-// Workgroup = 4 waves arranged 2x2; the 256 B rows come as two groups of 128
-// (gate / up weights, or two adjacent column blocks) and each wave owns 64x64
-// of each group: 128 fp32 accumulators per lane.  k-tile 64, global ->
-// registers -> LDS with the next k-tile's loads in flight during the MFMAs.
+// The 256 B rows come as two groups of 128 (gate / up weights, or two adjacent
+// column blocks) and each wave owns 64x64 of each group: 128 fp32 accumulators
+// per lane.  k-tile 64, global -> registers -> LDS with the next k-tile's loads
+// in flight during the MFMAs.  Two shapes: 128 rows with 4 waves arranged 2x2
+// (two workgroups per CU, each with a single LDS stage), and 256 rows with 8
+// waves arranged 4x2 (one workgroup per CU, two LDS stages, namespace wide).
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "core/device_math.h"
 
@@ -134,6 +138,143 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
     }
 
 }
+
+// The same per-wave work (64 x 64 of each column group) with eight waves arranged 4 x 2 over a
+// 256 x (2 x 128) tile: a third fewer global loads and LDS stores per flop than the 128-row tile.
+// The eight waves move in step (one barrier per k-tile), so LDS is double buffered and a k-tile is
+// in registers for a whole tile time before it is stored.
+namespace wide {
+
+constexpr int kThreads = 512;
+constexpr int kBM = 256;
+
+struct StageLds {
+    std::uint16_t a[kBM * kLS];
+    std::uint16_t b[2][kBN * kLS];
+};
+struct TileLds {
+    StageLds st[2];
+};
+
+// a_off[i]: chunk c = tid + i*512 -> tile row c/8, column (c%8)*8 (i < 4); b_off[g][i]: the same
+// for the 128 rows of column group g (i < 2).
+template <typename T>
+__device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
+                                              const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][2],
+                                              long K, TileLds& lds, float16_t (&acc)[2][2][2]) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lh = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    u32x4 a_st[4], b_st[2][2];
+    auto load_tile = [&](long k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_base + k0 + a_off[i]);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) b_st[g][i] = load16(b_base[g] + k0 + b_off[g][i]);
+    };
+    auto store_one = [&](StageLds& st, int idx) {        // idx 0..3: A chunks, 4..7: B chunks (g, i)
+        const int i = idx < 4 ? idx : (idx - 4) & 1;
+        const int c = tid + i * kThreads;
+        const int off = (c >> 3) * kLS + (c & 7) * 8;
+        if (idx < 4) *reinterpret_cast<u32x4*>(&st.a[off]) = a_st[idx];
+        else         *reinterpret_cast<u32x4*>(&st.b[(idx - 4) >> 1][off]) = b_st[(idx - 4) >> 1][i];
+    };
+
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[g][mi][ni][r] = 0.f;
+
+    const int a_off0 = (wm * 64 + lr) * kLS + lh * 8;
+    const int b_off0 = (wn * 64 + lr) * kLS + lh * 8;
+    const long k_tiles = K / kBK;
+    // The k-steps form one continuous pipeline across k-tiles: the operand fragments of a k-step are
+    // requested while the previous one computes, also across the tile boundary.  For that the
+    // barrier of a tile sits before its LAST k-step: by then the next k-tile has been stored into
+    // the other stage (one 16-byte store per MFMA pair of k-steps 1 and 2; nobody reads that stage
+    // between the previous barrier and this one), after it the last k-step's MFMAs run from
+    // registers while the first fragments of the next tile and the global loads of the tile after
+    // it are requested.
+    i16x8 af[2][2], bf[4];
+    auto read_a = [&](const StageLds& st, int buf, int ks) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+            af[buf][mi] = *reinterpret_cast<const i16x8*>(&st.a[a_off0 + mi * 32 * kLS + ks * 16]);
+    };
+    auto read_b = [&](const StageLds& st, int q, int ks) {   // q = 2*g + ni
+        bf[q] = *reinterpret_cast<const i16x8*>(&st.b[q >> 1][b_off0 + (q & 1) * 32 * kLS + ks * 16]);
+    };
+    auto compute = [&](const StageLds& cur_st, StageLds& nxt_st, long k_after, auto next_tag) {
+        constexpr bool kNext = decltype(next_tag)::value;
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            const int cur = ks & 1;
+            const bool last = ks + 1 == kBK / 16;
+            if (kNext && last) {
+                __syncthreads();
+                load_tile(k_after);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi) {
+                    acc[q >> 1][mi][q & 1] = MmaT<T>::run(af[cur][mi], bf[q], acc[q >> 1][mi][q & 1]);
+                    if (!last) {
+                        if (q == 0 && mi == 0) read_a(cur_st, cur ^ 1, ks + 1);
+                        if (mi == 1) read_b(cur_st, q, ks + 1);
+                    } else if (kNext) {
+                        if (q == 0 && mi == 0) read_a(nxt_st, cur ^ 1, 0);
+                        if (mi == 1) read_b(nxt_st, q, 0);
+                    }
+                    if (kNext && (ks == 1 || ks == 2) && mi == 0) store_one(nxt_st, (ks - 1) * 4 + q);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        }
+    };
+    load_tile(0);
+#pragma unroll
+    for (int idx = 0; idx < 8; ++idx) store_one(lds.st[0], idx);
+    __syncthreads();
+    if (k_tiles > 1) load_tile(kBK);
+    read_a(lds.st[0], 0, 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) read_b(lds.st[0], q, 0);
+    for (long kt = 0; kt + 1 < k_tiles; ++kt) {
+        const long after = kt + 2 < k_tiles ? kt + 2 : k_tiles - 1;   // the last tiles reload a tile nobody stores
+        compute(lds.st[kt & 1], lds.st[(kt + 1) & 1], after * kBK, std::true_type{});
+    }
+    compute(lds.st[(k_tiles - 1) & 1], lds.st[k_tiles & 1], 0, std::false_type{});
+}
+
+}  // namespace wide
+
+// The two tile shapes as a kernel sees them.
+struct Tile128 {
+    static constexpr int kBM = gemm::kBM, kThreads = gemm::kThreads, kBChunks = 4;
+    using Lds = TileLds;
+    template <typename T>
+    __device__ static __forceinline__ void mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
+                                                    const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][4],
+                                                    long K, Lds& lds, float16_t (&acc)[2][2][2]) {
+        tile_mainloop<T>(a_base, a_off, b_base, b_off, K, lds, acc);
+    }
+};
+struct Tile256 {
+    static constexpr int kBM = wide::kBM, kThreads = wide::kThreads, kBChunks = 2;
+    using Lds = wide::TileLds;
+    template <typename T>
+    __device__ static __forceinline__ void mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
+                                                    const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][2],
+                                                    long K, Lds& lds, float16_t (&acc)[2][2][2]) {
+        wide::tile_mainloop<T>(a_base, a_off, b_base, b_off, K, lds, acc);
+    }
+};
 
 }  // namespace gemm
 }  // namespace paras

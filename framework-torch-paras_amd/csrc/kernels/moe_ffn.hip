@@ -14,12 +14,13 @@
 // contraction dim, which is exactly the 8-element-per-lane operand layout of
 // v_mfma_f32_32x32x16, so neither operand needs a transpose.
 //
-// Tiling: workgroup = 4 waves = 128 routed rows x two 128-column groups (gate
-// and up columns n0..n0+127 for GEMM 1; columns n0..n0+255 for GEMM 2), k-tile
-// 64, waves arranged 2x2 with 64x64 per column group each (128 fp32
-// accumulators per lane).  Global -> registers -> LDS with the next k-tile's
-// loads in flight during the MFMAs.  Rows of one expert are contiguous in the
-// routed order; m-tiles never straddle experts (the grid is sized for the
+// Tiling (gemm_tile.h): a workgroup computes 128 or 256 routed rows x two
+// 128-column groups (gate and up columns n0..n0+127 for GEMM 1; columns
+// n0..n0+255 for GEMM 2), k-tile 64, waves arranged 2x2 or 4x2 with 64x64 per
+// column group each (128 fp32 accumulators per lane); 256 rows when the
+// experts hold enough rows for them.  Global -> registers -> LDS with the next
+// k-tile's loads in flight during the MFMAs.  Rows of one expert are contiguous
+// in the routed order; m-tiles never straddle experts (the grid is sized for the
 // worst case and surplus workgroups exit).  The block index is unscrambled so
 // that the workgroups resident on one XCD cover all m-tiles of a few column
 // tiles: weight tiles are then shared through that XCD's L2.
@@ -50,10 +51,11 @@ struct FfnGemmParams {
     int ngt;                    // column units an XCD sweeps together
 };
 
-template <typename T, bool kSwiglu>
-__global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemmParams p) {
+template <typename T, bool kSwiglu, typename S>
+__global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnGemmParams p) {
     using El = Elem<T>;
-    __shared__ __attribute__((aligned(16))) TileLds lds;
+    constexpr int kBM = S::kBM;
+    __shared__ __attribute__((aligned(16))) typename S::Lds lds;
 
     // ---- tile coordinates.  Linear id L: xcd = L % 8 (hardware round-robin);
     // within an XCD walk (column group, m-tile, column-in-group).
@@ -94,10 +96,10 @@ __global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemm
     const int wm = wave >> 1, wn = wave & 1;
 
     // ---- global -> register staging: 16-byte chunks, 8 per row of a k-tile
-    unsigned a_off[4], b_off[2][4];
+    unsigned a_off[4], b_off[2][S::kBChunks];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int c = tid + i * kThreads;
+        const int c = tid + i * S::kThreads;
         long prow = row0 + (c >> 3);
         if (prow >= row_end) prow = row_end - 1;  // clamp: result rows beyond the expert are not stored
         const long src = p.order ? p.order[prow] / p.k : prow;
@@ -108,14 +110,14 @@ __global__ __launch_bounds__(kThreads, 2) void grouped_gemm_kernel(const FfnGemm
 #pragma unroll
     for (int g = 0; g < 2; ++g)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + i * kThreads;
+        for (int i = 0; i < S::kBChunks; ++i) {
+            const int c = tid + i * S::kThreads;
             long wrow = (kSwiglu ? n0 : n0 + g * kBN) + (c >> 3);
             if (wrow >= p.Nw) wrow = p.Nw - 1;
             b_off[g][i] = static_cast<unsigned>(wrow * p.K + (c & 7) * 8);
         }
     float16_t acc[2][2][2];
-    tile_mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, acc);
+    S::template mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, acc);
 
     // ---- epilogue.  Accumulator lane (column lr, half lh) holds rows (r/4)*8 + 4*lh + r%4.
 #pragma unroll
@@ -172,14 +174,14 @@ __global__ __launch_bounds__(kThreads) void moe_combine_kernel(const std::uint16
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-template <typename T>
-int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
+template <typename T, typename S>
+int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
             const long* order, const long* inv_order, const long* offsets, void* out, void* workspace, long T_,
             int E, int k, long H, long I, hipStream_t s) {
     const long R = T_ * k;
     auto* h = static_cast<std::uint16_t*>(workspace);
     auto* y = reinterpret_cast<std::uint16_t*>(static_cast<char*>(workspace) + align_up(static_cast<size_t>(R) * I * 2, 256));
-    const int mt_total = static_cast<int>((R + kBM - 1) / kBM) + E;
+    const int mt_total = static_cast<int>((R + S::kBM - 1) / S::kBM) + E;
 
     FfnGemmParams g1{};
     g1.a = static_cast<const std::uint16_t*>(x);
@@ -203,7 +205,7 @@ int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_d
         return static_cast<unsigned>(groups * 8 * g.ngt * g.mt_total);
     };
     plan(g1);
-    hipLaunchKernelGGL((grouped_gemm_kernel<T, true>), dim3(grid_of(g1)), dim3(kThreads), 0, s, g1);
+    hipLaunchKernelGGL((grouped_gemm_kernel<T, true, S>), dim3(grid_of(g1)), dim3(S::kThreads), 0, s, g1);
     PARAS_HIP_TRY(hipGetLastError());
 
     FfnGemmParams g2{};
@@ -217,7 +219,7 @@ int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_d
     g2.mt_total = mt_total;
     g2.n_units = static_cast<int>((H + 2 * kBN - 1) / (2 * kBN));
     plan(g2);
-    hipLaunchKernelGGL((grouped_gemm_kernel<T, false>), dim3(grid_of(g2)), dim3(kThreads), 0, s, g2);
+    hipLaunchKernelGGL((grouped_gemm_kernel<T, false, S>), dim3(grid_of(g2)), dim3(S::kThreads), 0, s, g2);
     PARAS_HIP_TRY(hipGetLastError());
 
     const long total = T_ * (H / 8);
@@ -227,6 +229,20 @@ int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_d
                        inv_order, static_cast<std::uint16_t*>(out), T_, k, H);
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
+}
+
+// 256-row tiles when the experts are big enough for them: an expert's last tile is half empty on
+// average, so the rows per expert should be many times the tile, and there must be enough tiles
+// to fill the chip.
+template <typename T>
+int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
+            const long* order, const long* inv_order, const long* offsets, void* out, void* workspace, long T_,
+            int E, int k, long H, long I, hipStream_t s) {
+    const long R = T_ * k;
+    const long wide_tiles = (R / Tile256::kBM) * ((H + 2 * kBN - 1) / (2 * kBN));
+    if (R / E >= 4 * Tile256::kBM && wide_tiles >= 2 * 256)
+        return run_ffn_shape<T, Tile256>(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, out, workspace, T_, E, k, H, I, s);
+    return run_ffn_shape<T, Tile128>(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, out, workspace, T_, E, k, H, I, s);
 }
 
 }  // namespace

@@ -115,3 +115,19 @@ def test_gemm_nt_many_tiles_with_ragged_edges(dtype):
     # where 2 * round(v) and round(2 v) keep different numbers of bits)
     big = out.float().abs() > 1e-3
     assert torch.equal(capi.gemm_nt(a * 2, b)[big], (out * 2)[big])
+
+
+def test_gemm_nt_256_row_tiles_agree_with_128_row_tiles():
+    """A batch of four problems is big enough for the 256-row tiles, each problem alone is not:
+    both forms add the same products in the same order, so they agree bit for bit (ragged M and
+    N, strided batch)."""
+    torch.manual_seed(21)
+    Bt, M, N, K = 4, 4100, 2100, 128
+    a = torch.randn(Bt, M, K, device="cuda").bfloat16()
+    b = (0.1 * torch.randn(Bt, N, K, device="cuda")).bfloat16()
+    whole = capi.gemm_nt(a, b)
+    assert whole.shape == (Bt, M, N)
+    for i in range(Bt):
+        assert torch.equal(whole[i], capi.gemm_nt(a[i], b[i])), f"batch {i}"
+    ref = O.matmul_nt(a[3, -3:].cpu(), b[3].cpu())
+    assert_gemm_close(whole[3, -3:], ref, torch.bfloat16)

@@ -130,3 +130,27 @@ def test_config5_routing_exact_and_sampled_tokens():
     ref = O.moe_ffn(x[sel], wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
     err = assert_ffn_close(out.cpu()[sel], ref, dt)
     assert err.mean().item() < 5e-4
+
+
+def test_ffn_256_row_tiles_with_ragged_tiny_and_empty_experts():
+    """Big enough for the 256-row tiles (8192 tokens, top-2, 5 experts of which one gets three
+    tokens and one none): sampled tokens, all of the tiny expert's among them, against the oracle."""
+    torch.manual_seed(5)
+    T, H, E, k, I = 8192, 2048, 5, 2, 512
+    dt = torch.bfloat16
+    logits = torch.randn(T, E)
+    logits[:, 3] -= 30.0                      # expert 3: only the three tokens below
+    logits[:, 4] -= 60.0                      # expert 4: nobody
+    tiny = torch.tensor([5, 4000, T - 1])
+    logits[tiny, 3] += 60.0
+    logits = logits.to(dt)
+    x = torch.randn(T, H).to(dt)
+    wg, wu = (0.03 * torch.randn(E, I, H)).to(dt), (0.03 * torch.randn(E, I, H)).to(dt)
+    wd = (0.03 * torch.randn(E, H, I)).to(dt)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    assert counts.cpu().tolist()[3:] == [3, 0]
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    sel = torch.cat([tiny, torch.randperm(T)[:40]])
+    r = O.moe_route(logits[sel], k)
+    ref = O.moe_ffn(x[sel], wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
+    assert_ffn_close(out.cpu()[sel], ref, dt)
