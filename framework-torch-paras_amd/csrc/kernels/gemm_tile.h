@@ -166,15 +166,15 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
     const int lr = lane & 31, lh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
     u32x4 a_st[4], b_st[2][2];
+    auto load_one = [&](int idx, long k0) {              // idx 0..3: A chunks, 4..7: B chunks (g, i)
+        if (idx < 4) a_st[idx] = load16(a_base + k0 + a_off[idx]);
+        else         b_st[(idx - 4) >> 1][(idx - 4) & 1] = load16(b_base[(idx - 4) >> 1] + k0 + b_off[(idx - 4) >> 1][(idx - 4) & 1]);
+    };
     auto load_tile = [&](long k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a_st[i] = load16(a_base + k0 + a_off[i]);
-#pragma unroll
-        for (int g = 0; g < 2; ++g)
-#pragma unroll
-            for (int i = 0; i < 2; ++i) b_st[g][i] = load16(b_base[g] + k0 + b_off[g][i]);
+        for (int idx = 0; idx < 8; ++idx) load_one(idx, k0);
     };
-    auto store_one = [&](StageLds& st, int idx) {        // idx 0..3: A chunks, 4..7: B chunks (g, i)
+    auto store_one = [&](StageLds& st, int idx) {
         const int i = idx < 4 ? idx : (idx - 4) & 1;
         const int c = tid + i * kThreads;
         const int off = (c >> 3) * kLS + (c & 7) * 8;
@@ -197,10 +197,10 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
     // The k-steps form one continuous pipeline across k-tiles: the operand fragments of a k-step are
     // requested while the previous one computes, also across the tile boundary.  For that the
     // barrier of a tile sits before its LAST k-step: by then the next k-tile has been stored into
-    // the other stage (one 16-byte store per MFMA pair of k-steps 1 and 2; nobody reads that stage
-    // between the previous barrier and this one), after it the last k-step's MFMAs run from
-    // registers while the first fragments of the next tile and the global loads of the tile after
-    // it are requested.
+    // the other stage (one 16-byte store per MFMA pair of k-steps 1 and 2, each followed by the
+    // global load of the same chunk of the tile after that; nobody reads that stage between the
+    // previous barrier and this one), after it the last k-step's MFMAs run from registers while
+    // the first fragments of the next tile are requested.
     i16x8 af[2][2], bf[4];
     auto read_a = [&](const StageLds& st, int buf, int ks) {
 #pragma unroll
@@ -216,10 +216,7 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
         for (int ks = 0; ks < kBK / 16; ++ks) {
             const int cur = ks & 1;
             const bool last = ks + 1 == kBK / 16;
-            if (kNext && last) {
-                __syncthreads();
-                load_tile(k_after);
-            }
+            if (kNext && last) __syncthreads();
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -232,7 +229,10 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
                         if (q == 0 && mi == 0) read_a(nxt_st, cur ^ 1, 0);
                         if (mi == 1) read_b(nxt_st, q, 0);
                     }
-                    if (kNext && (ks == 1 || ks == 2) && mi == 0) store_one(nxt_st, (ks - 1) * 4 + q);
+                    if (kNext && (ks == 1 || ks == 2) && mi == 0) {
+                        store_one(nxt_st, (ks - 1) * 4 + q);
+                        load_one((ks - 1) * 4 + q, k_after);   // the register is free again: a whole tile of time to arrive
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
         }
