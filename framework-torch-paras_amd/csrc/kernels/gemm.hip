@@ -35,8 +35,8 @@ struct DenseParams {
     float alpha, beta;
 };
 
-// S = Tile128 (4 waves, 128 rows) or Tile256 (8 waves, 256 rows; for problems with enough
-// 256 x 256 tiles to fill the chip).
+// S = Tile128 (4 waves, 128 rows) or Tile256 (8 waves, 256 rows; for problems with at least
+// 128 tiles of 256 x 256).
 template <typename T, typename S>
 __global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const DenseParams p) {
     using El = Elem<T>;
@@ -126,7 +126,7 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
     const int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
     const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
-    const bool use_wide = wide_tiles >= 2 * 256;   // at least two rounds of one workgroup per CU
+    const bool use_wide = wide_tiles >= 128;       // measured: faster from half a round of one workgroup per CU upwards
     const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
     const int64_t m_tiles = (M + bm - 1) / bm;
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");

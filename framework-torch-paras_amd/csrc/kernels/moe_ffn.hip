@@ -232,15 +232,15 @@ int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const voi
 }
 
 // 256-row tiles when the experts are big enough for them: an expert's last tile is half empty on
-// average, so the rows per expert should be many times the tile, and there must be enough tiles
-// to fill the chip.
+// average, so the rows per expert should be many times the tile, and there must be tiles for at
+// least half the CUs.
 template <typename T>
 int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
             const long* order, const long* inv_order, const long* offsets, void* out, void* workspace, long T_,
             int E, int k, long H, long I, hipStream_t s) {
     const long R = T_ * k;
     const long wide_tiles = (R / Tile256::kBM) * ((H + 2 * kBN - 1) / (2 * kBN));
-    if (R / E >= 4 * Tile256::kBM && wide_tiles >= 2 * 256)
+    if (R / E >= 4 * Tile256::kBM && wide_tiles >= 128)
         return run_ffn_shape<T, Tile256>(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, out, workspace, T_, E, k, H, I, s);
     return run_ffn_shape<T, Tile128>(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, out, workspace, T_, E, k, H, I, s);
 }
