@@ -8,7 +8,8 @@ bf16 causal flash-attention forward at B=4, H=32, S=4096, D=128 (configs[2]) in
 TFLOP/s, counted with the causal-halved figure 4*B*H*S^2*D/2.  The same line
 carries, under "workloads", the other configurations the metric names
 (RMSNorm and SwiGLU of configs[1] in GB/s, the GQA decode of configs[3], the
-MoE layer of configs[4]), each with its own roofline object.
+MoE layer of configs[4]), the dense projection GEMM and the backward / RoPE
+helper ops that sit either side of the path, each with its own roofline object.
 
 A step is one pass of the workload's kernels over one batch of synthetic
 inputs (seeded N(0,1) / N(1,0.02) / N(0,0.02) as BASELINE.json states) that
@@ -89,7 +90,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe", "linear", "copy"],
+                    choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe", "linear", "backward_ops", "copy"],
                     help="'copy' is the counter calibration: a plain 1 GiB device copy, not part of 'all'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     args = ap.parse_args()
@@ -263,6 +264,53 @@ def main() -> int:
         log(f"linear: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s ({tf / MFMA_BF16_PEAK_TFLOPS:.1%})")
         del xa, wb, yc
 
+    # ------------------------------------------------------------------ the ops either side of the path
+    if want("backward_ops"):
+        rows, Hd, I = 16384, 4096, 14336
+        x = torch.randn(rows, Hd, device=dev).to(bf)
+        go = torch.randn(rows, Hd, device=dev).to(bf)
+        w = (1 + 0.02 * torch.randn(Hd, device=dev)).to(bf)
+        y, gx, gw = torch.empty_like(x), torch.empty_like(x), torch.empty_like(w)
+        rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+        must(L.paras_rms_norm_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, Hd, 1e-6, capi.BF16, st))
+        ws = torch.empty(L.paras_rms_norm_bwd_workspace(rows, Hd), dtype=torch.uint8, device=dev)
+        ms_b, _ = timer.run(lambda i: must(L.paras_rms_norm_bwd(go.data_ptr(), x.data_ptr(), w.data_ptr(), rstd.data_ptr(),
+                                                                 gx.data_ptr(), gw.data_ptr(), ws.data_ptr(), rows, Hd, capi.BF16, st)),
+                            steps, warmup)
+        bytes_b = 3 * rows * Hd * 2 + rows * 4 + 2 * Hd * 2
+        del y, gx, ws
+        gate = torch.randn(rows, I, device=dev).to(bf)
+        up = torch.randn(rows, I, device=dev).to(bf)
+        g2 = torch.randn(rows, I, device=dev).to(bf)
+        dg, du = torch.empty_like(gate), torch.empty_like(gate)
+        n = rows * I
+        ms_s, _ = timer.run(lambda i: must(L.paras_swiglu_bwd(g2.data_ptr(), gate.data_ptr(), up.data_ptr(), dg.data_ptr(),
+                                                               du.data_ptr(), n, capi.BF16, st)), max(steps // 5, 5), max(warmup // 5, 2))
+        bytes_s = 5 * n * 2
+        del gate, up, g2, dg, du
+        qh = torch.randn(4 * 32 * 4096, 128, device=dev).to(bf)
+        qo = torch.empty_like(qh)
+        ms_r, _ = timer.run(lambda i: must(L.paras_rotate_half(qh.data_ptr(), qo.data_ptr(), qh.shape[0], 128, 0, capi.BF16, st)),
+                            steps, warmup)
+        bytes_r = 2 * qh.numel() * 2
+        gb = lambda b, ms: b / ms / 1e6
+        results["backward_ops"] = {
+            "workload": "bf16 RMSNorm backward 16384x4096, SwiGLU backward 16384x14336, rotate_half 4x32x4096x128",
+            "value": round((bytes_b + bytes_s + bytes_r) / (ms_b + ms_s + ms_r) / 1e6, 1), "unit": "GB/s",
+            "ms_per_step": round(ms_b + ms_s + ms_r, 4),
+            "rms_norm_bwd": {"ms": round(ms_b, 4), "algorithmic_bytes_per_launch": bytes_b,
+                             "kernel": "rms_norm_bwd_fused<bf16,2> + rms_norm_bwd_dw_final_wide",
+                             "roofline": roofline("hbm", gb(bytes_b, ms_b), "rms_norm_bwd_fused")},
+            "swiglu_bwd": {"ms": round(ms_s, 4), "algorithmic_bytes_per_launch": bytes_s, "kernel": "swiglu_bwd_any<bf16> (all fp64)",
+                           "roofline": roofline("hbm", gb(bytes_s, ms_s), "swiglu_bwd_any")},
+            "rotate_half": {"ms": round(ms_r, 4), "algorithmic_bytes_per_launch": bytes_r, "kernel": "rotate_half_vec16",
+                            "roofline": roofline("hbm", gb(bytes_r, ms_r), "rotate_half_vec16")},
+        }
+        log(f"backward_ops: rms_norm_bwd {ms_b * 1e3:.1f} us {gb(bytes_b, ms_b):.0f} GB/s ({gb(bytes_b, ms_b) / HBM_PEAK_GBS:.1%})   "
+            f"swiglu_bwd {ms_s * 1e3:.1f} us {gb(bytes_s, ms_s):.0f} GB/s ({gb(bytes_s, ms_s) / HBM_PEAK_GBS:.1%})   "
+            f"rotate_half {ms_r * 1e3:.1f} us {gb(bytes_r, ms_r):.0f} GB/s ({gb(bytes_r, ms_r) / HBM_PEAK_GBS:.1%})")
+        del x, go, qh, qo
+
     # ------------------------------------------------------------------ counter calibration
     if args.workload == "copy":
         n = 1 << 29                                # 2^29 bf16 elements: 1 GiB read + 1 GiB written
@@ -299,7 +347,7 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": head["workload"], "device": torch.cuda.get_device_name(0),
                    "timing": "HIP events on the launch stream, inputs resident in HBM"},
-        "roofline": head.get("roofline") or head["rms_norm"]["roofline"],
+        "roofline": head.get("roofline") or next(v["roofline"] for v in head.values() if isinstance(v, dict) and "roofline" in v),
         "cpu_baseline": cpu,
         "workloads": results,
     }

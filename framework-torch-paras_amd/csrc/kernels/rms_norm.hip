@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dx(
     }
 }
 
-constexpr int kDwSlabRows = 256;  // rows per partial column sum
+constexpr int kDwSlabRows = 16;   // rows per partial column sum
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_partial(
@@ -216,6 +216,112 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final(
     double acc = 0.0;
     for (long s = 0; s < slabs; ++s) acc += partial[s * H + j];
     gw[j] = E::from_f64(acc);
+}
+
+// 16-bit tensors with 16-byte aligned rows of at most kBlock*NV vectors: dx and the partial
+// column sums in ONE pass over grad_out and x.  A workgroup owns a slab of kDwSlabRows rows; each
+// thread keeps the same NV vectors of every row (and of w), so its 8*NV column sums live in
+// registers across the slab, and the next row's vectors are requested before the current row's
+// reduction.  Arithmetic in fp64 in the host's order of operations.  (NV = 2 needs 136 registers:
+// three workgroups per CU.  Re-reading w per row to fit four measured 20 % slower.)
+template <typename T, int NV>
+__global__ __launch_bounds__(kBlock, (NV == 1 ? 4 : 3)) void rms_norm_bwd_fused(
+    const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
+    const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
+    using E = Elem<T>;
+    constexpr int V = 8;
+    __shared__ double slots[2 * kWavesPerBlock];
+    const int nvec = H / V;
+    const long slab = blockIdx.x;
+    const long r0 = slab * kDwSlabRows;
+    const long r1 = r0 + kDwSlabRows < rows ? r0 + kDwSlabRows : rows;
+    bool have[NV];
+    u32x4 wv[NV], gv[NV], xv[NV], gn[NV], xn[NV];
+    double dw[NV][V];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * kBlock;
+        have[i] = c < nvec;
+        if (have[i]) {
+            wv[i] = load16(w + static_cast<long>(c) * V);
+            gn[i] = load16_nt(go + r0 * H + static_cast<long>(c) * V);
+            xn[i] = load16_nt(x + r0 * H + static_cast<long>(c) * V);
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) dw[i][j] = 0.0;
+    }
+    int sum_calls = 0;
+    for (long r = r0; r < r1; ++r) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            gv[i] = gn[i];
+            xv[i] = xn[i];
+            if (have[i] && r + 1 < r1) {
+                const int c = threadIdx.x + i * kBlock;
+                gn[i] = load16_nt(go + (r + 1) * H + static_cast<long>(c) * V);
+                xn[i] = load16_nt(x + (r + 1) * H + static_cast<long>(c) * V);
+            }
+        }
+        const double rr = static_cast<double>(rstd[r]);
+        double dot = 0.0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (have[i]) {
+                const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv[i]);
+                const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv[i]);
+                const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const double g = E::to_f64(ge[j]), xj = E::to_f64(xe[j]);
+                    dot += g * E::to_f64(we[j]) * xj;
+                    dw[i][j] += g * xj * rr;
+                }
+            }
+        dot = block_sum(dot, slots, sum_calls++);
+        const double coef = rr * rr * rr / static_cast<double>(H);
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (have[i]) {
+                const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv[i]);
+                const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv[i]);
+                const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
+                u32x4 o;
+                std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    oe[j] = E::from_f64(E::to_f64(ge[j]) * E::to_f64(we[j]) * rr - coef * E::to_f64(xe[j]) * dot);
+                store16_nt(gx + r * H + static_cast<long>(threadIdx.x + i * kBlock) * V, o);
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+        if (have[i]) {
+            double* dst = partial + slab * H + static_cast<long>(threadIdx.x + i * kBlock) * V;
+#pragma unroll
+            for (int j = 0; j < V; ++j) dst[j] = dw[i][j];
+        }
+}
+
+// Column sums of the slabs in a fixed order: thread (column c of 8, lane l of 32) adds slabs
+// l, l+32, ... and the 32 lane sums meet in LDS in lane order.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final_wide(
+    const double* __restrict__ partial, typename Elem<T>::store_t* __restrict__ gw, long slabs, long H) {
+    using E = Elem<T>;
+    __shared__ double part[32][8];
+    const int c = threadIdx.x & 7, l = threadIdx.x >> 3;
+    const long j = static_cast<long>(blockIdx.x) * 8 + c;
+    double acc = 0.0;
+    if (j < H)
+        for (long sl = l; sl < slabs; sl += 32) acc += partial[sl * H + j];
+    part[l][c] = acc;
+    __syncthreads();
+    if (l == 0 && j < H) {
+        double t = 0.0;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) t += part[k][c];
+        gw[j] = E::from_f64(t);
+    }
 }
 
 int grid_for_rows(long rows) {
@@ -255,17 +361,40 @@ template <typename T>
 int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, void* gx,
                void* gw, void* workspace, long rows, long H, hipStream_t s) {
     using S = typename Elem<T>::store_t;
+    const long slabs = (rows + kDwSlabRows - 1) / kDwSlabRows;
+    PARAS_REQUIRE(slabs <= 0x7fffffffL, "paras_rms_norm_bwd: too many rows");
+    if constexpr (sizeof(S) == 2) {
+        const bool aligned = (H % 8 == 0) && ((reinterpret_cast<uintptr_t>(go) | reinterpret_cast<uintptr_t>(x) |
+                                               reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gx)) % 16 == 0);
+        const long nvec = H / 8;
+        if (aligned && nvec <= kBlock * 2) {
+            const auto* g16 = static_cast<const std::uint16_t*>(go);
+            const auto* x16 = static_cast<const std::uint16_t*>(x);
+            const auto* w16 = static_cast<const std::uint16_t*>(w);
+            auto* gx16 = static_cast<std::uint16_t*>(gx);
+            auto* part = static_cast<double*>(workspace);
+            if (nvec <= kBlock)
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1>), dim3(static_cast<unsigned>(slabs)), dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            else
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 2>), dim3(static_cast<unsigned>(slabs)), dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            PARAS_HIP_TRY(hipGetLastError());
+            hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + 7) / 8)), dim3(kBlock), 0, s,
+                               part, static_cast<S*>(gw), slabs, H);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
+    }
     hipLaunchKernelGGL((rms_norm_bwd_dx<T>), dim3(grid_for_rows(rows)), dim3(kBlock), 0, s,
                        static_cast<const S*>(go), static_cast<const S*>(x), static_cast<const S*>(w),
                        rstd, static_cast<S*>(gx), rows, H);
     PARAS_HIP_TRY(hipGetLastError());
-    const long slabs = (rows + kDwSlabRows - 1) / kDwSlabRows;
     const unsigned gx_blocks = static_cast<unsigned>((H + kBlock - 1) / kBlock);
+    PARAS_REQUIRE(slabs <= 65535, "paras_rms_norm_bwd: too many rows for this dtype / row size");
     hipLaunchKernelGGL((rms_norm_bwd_dw_partial<T>), dim3(gx_blocks, static_cast<unsigned>(slabs)),
                        dim3(kBlock), 0, s, static_cast<const S*>(go), static_cast<const S*>(x), rstd,
                        static_cast<double*>(workspace), rows, H);
     PARAS_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL((rms_norm_bwd_dw_final<T>), dim3(gx_blocks), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + 7) / 8)), dim3(kBlock), 0, s,
                        static_cast<const double*>(workspace), static_cast<S*>(gw), slabs, H);
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;

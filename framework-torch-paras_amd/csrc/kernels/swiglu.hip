@@ -103,6 +103,24 @@ __global__ __launch_bounds__(kBlock) void rotate_half_any(const S* __restrict__ 
     }
 }
 
+// 16-bit elements, D a multiple of 16, 16-byte aligned: one 16-byte vector per lane, the
+// partner vector sits half a row away, the sign flips are one XOR per register.
+__global__ __launch_bounds__(kBlock) void rotate_half_vec16(const std::uint16_t* __restrict__ x,
+                                                            std::uint16_t* __restrict__ out, long nvec,
+                                                            int vec_per_row, int backward) {
+    const int half = vec_per_row / 2;
+    const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= nvec) return;
+    const int col = static_cast<int>(i % vec_per_row);
+    const bool first = col < half;
+    u32x4 v = load16_nt(x + (first ? i + half : i - half) * 8);
+    if (backward ? !first : first) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] ^= 0x80008000u;
+    }
+    store16_nt(out + i * 8, v);
+}
+
 int stream_grid(long work_items_per_block_iter, long total) {
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -214,8 +232,16 @@ int paras_rotate_half(const void* x, void* out, int64_t rows, int64_t D, int bac
             break;
         case PARAS_BF16:
         case PARAS_F16:
-            hipLaunchKernelGGL((rotate_half_any<uint16_t>), grid, block, 0, s, static_cast<const uint16_t*>(x),
-                               static_cast<uint16_t*>(out), n, (long)D, backward);
+            if (D % 16 == 0 && D / 8 <= 0x7fffffff && n / 8 <= 0x7fffffffL * kBlock &&
+                ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+                const long nvec = n / 8;
+                hipLaunchKernelGGL(rotate_half_vec16, dim3(static_cast<unsigned>((nvec + kBlock - 1) / kBlock)), block, 0, s,
+                                   static_cast<const uint16_t*>(x), static_cast<uint16_t*>(out), nvec,
+                                   static_cast<int>(D / 8), backward);
+            } else {
+                hipLaunchKernelGGL((rotate_half_any<uint16_t>), grid, block, 0, s, static_cast<const uint16_t*>(x),
+                                   static_cast<uint16_t*>(out), n, (long)D, backward);
+            }
             break;
         default: return fail(PARAS_ERR_INVALID, "paras_rotate_half: unknown dtype %d", dtype);
     }

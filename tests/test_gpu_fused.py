@@ -139,3 +139,31 @@ def test_full_size_rms_norm_and_swiglu_bf16():
     neg = capi.swiglu(gd, -ud)
     assert torch.equal(neg.view(torch.int16) ^ res.view(torch.int16),
                        torch.full_like(res.view(torch.int16), -32768))    # odd in `up`, bit for bit
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(70, 4096), (33, 2048), (16, 520), (300, 1024), (5, 8)])
+def test_rms_norm_backward_one_pass_kernel(shape, dtype):
+    """Row sizes the one-pass backward kernel takes (16-byte aligned rows of up to 4096 elements),
+    with slabs of rows that are full, ragged and single."""
+    rows, H = shape
+    torch.manual_seed(rows + H)
+    x, w, go = torch.randn(rows, H).to(dtype), (1 + 0.1 * torch.randn(H)).to(dtype), torch.randn(rows, H).to(dtype)
+    _, rstd = O.rms_norm(x, w, 1e-6)
+    gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(rstd))
+    wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
+    assert_bit_exact(gx, wgx, "rms_norm grad_input")
+    assert_bit_exact(gw, wgw, "rms_norm grad_weight")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rotate_half_vector_path_and_fallbacks(dtype):
+    for shape in [(3, 5, 128), (7, 64), (2, 16), (4, 48), (3, 24), (5, 130)]:
+        xr = torch.randn(*shape).to(dtype)
+        assert_bit_exact(capi.rotate_half(dev(xr)), O.rotate_half(xr), f"rotate_half {shape}")
+        assert_bit_exact(capi.rotate_half(dev(xr), True), O.rotate_half(xr, True), f"rotate_half backward {shape}")
+    # a view that starts 2 bytes into an allocation: not 16-byte aligned
+    buf = torch.randn(4 * 128 + 1).to(dtype)
+    xr = buf[1:].view(4, 128)
+    got = capi.rotate_half(dev(buf)[1:].view(4, 128))
+    assert_bit_exact(got, O.rotate_half(xr.contiguous()), "rotate_half unaligned")
