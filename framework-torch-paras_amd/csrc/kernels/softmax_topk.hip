@@ -10,8 +10,9 @@
 //            Comparisons are on the values widened to double, so they are
 //            exact for every float dtype; indices are int64.
 //
-// One workgroup per row; rows are re-read from L2 between passes (these ops sit
-// on router logits and attention rows: thousands of elements, not millions).
+// Rows of up to 256 elements: one wave per row, the row in registers.  Longer rows: one
+// workgroup per row, re-read from L2 between passes (these ops sit on router logits and
+// attention rows: thousands of elements, not millions).
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -134,10 +135,111 @@ __global__ __launch_bounds__(kBlock) void topk_rows_kernel(const typename Elem<T
     }
 }
 
+// ---- short rows (n <= 64 * EPL): one wave per row, four rows per workgroup, the row in
+// registers (lane l holds elements l, l + 64, ...), no LDS and no barrier.  Router logits and
+// other rows of a few dozen elements would otherwise leave most of a 256-thread workgroup idle.
+template <typename TI, typename TO, int EPL>
+__global__ __launch_bounds__(kBlock) void softmax_rows_wave_kernel(const typename Elem<TI>::store_t* __restrict__ x,
+                                                                   typename Elem<TO>::store_t* __restrict__ out, long rows, int n) {
+    using EI = Elem<TI>;
+    using EO = Elem<TO>;
+    const int lane = threadIdx.x % kWave;
+    const long row = static_cast<long>(blockIdx.x) * kWaves + threadIdx.x / kWave;
+    if (row >= rows) return;                    // whole waves leave: nothing below synchronises the workgroup
+    const auto* xr = x + row * n;
+    auto* outr = out + row * n;
+    double v[EPL];
+    double m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int j = lane + i * kWave;
+        v[i] = j < n ? EI::to_f64(xr[j]) : -INFINITY;
+        if (j < n && v[i] > m) m = v[i];        // as the host: a NaN never replaces the max
+    }
+    m = wave_max_f64(m);
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int j = lane + i * kWave;
+        v[i] = j < n ? exp(v[i] - m) : 0.0;
+        sum += v[i];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int j = lane + i * kWave;
+        if (j < n) outr[j] = EO::from_f64(v[i] / sum);
+    }
+}
+
+template <typename T, int EPL>
+__global__ __launch_bounds__(kBlock) void topk_rows_wave_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                                typename Elem<T>::store_t* __restrict__ values,
+                                                                long* __restrict__ indices, long rows, int n, int k, int largest_i) {
+    using E = Elem<T>;
+    const bool largest = largest_i != 0;
+    const int lane = threadIdx.x % kWave;
+    const long row = static_cast<long>(blockIdx.x) * kWaves + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const auto* xr = x + row * n;
+    double v[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int j = lane + i * kWave;
+        v[i] = j < n ? E::to_f64(xr[j]) : 0.0;
+    }
+    double prev_v = 0.0;
+    long prev_i = -1;
+    for (int s = 0; s < k; ++s) {
+        double best_v = 0.0;
+        long best_i = -1;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const long j = lane + i * kWave;
+            if (j >= n) continue;
+            if (s > 0 && !comes_before(prev_v, prev_i, v[i], j, largest)) continue;   // strictly after the previous slot
+            if (best_i < 0 || comes_before(v[i], j, best_v, best_i, largest)) {
+                best_v = v[i];
+                best_i = j;
+            }
+        }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const double ov = __shfl_xor(best_v, off, kWave);
+            const long oi = __shfl_xor(static_cast<int>(best_i), off, kWave);
+            if (oi >= 0 && (best_i < 0 || comes_before(ov, oi, best_v, best_i, largest))) {
+                best_v = ov;
+                best_i = oi;
+            }
+        }
+        if (lane == 0) {
+            // a row of NaNs has no element that "comes before" another: index -1, value 0, as the host engine
+            values[row * k + s] = best_i >= 0 ? xr[best_i] : E::from_f64(0.0);
+            indices[row * k + s] = best_i;
+        }
+        prev_v = best_v;
+        prev_i = best_i;
+    }
+}
+
 template <typename TI>
 int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, hipStream_t s) {
     using SI = typename Elem<TI>::store_t;
     const dim3 g(static_cast<unsigned>(rows)), b(kBlock);
+    if (n <= 4 * kWave) {
+        const dim3 gw(static_cast<unsigned>((rows + kWaves - 1) / kWaves));
+        const bool widen = dtype_out == PARAS_F32 && sizeof(SI) == 2;
+        const auto* xs = static_cast<const SI*>(x);
+        if (n <= kWave) {
+            if (widen) hipLaunchKernelGGL((softmax_rows_wave_kernel<TI, float, 1>), gw, b, 0, s, xs, static_cast<float*>(out), rows, (int)n);
+            else       hipLaunchKernelGGL((softmax_rows_wave_kernel<TI, TI, 1>), gw, b, 0, s, xs, static_cast<SI*>(out), rows, (int)n);
+        } else {
+            if (widen) hipLaunchKernelGGL((softmax_rows_wave_kernel<TI, float, 4>), gw, b, 0, s, xs, static_cast<float*>(out), rows, (int)n);
+            else       hipLaunchKernelGGL((softmax_rows_wave_kernel<TI, TI, 4>), gw, b, 0, s, xs, static_cast<SI*>(out), rows, (int)n);
+        }
+        PARAS_HIP_TRY(hipGetLastError());
+        return PARAS_OK;
+    }
     if (dtype_out == PARAS_F32 && sizeof(SI) == 2)
         hipLaunchKernelGGL((softmax_rows_kernel<TI, float>), g, b, 0, s, static_cast<const SI*>(x), static_cast<float*>(out), n);
     else
@@ -149,6 +251,15 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
 template <typename T>
 int launch_topk(const void* x, void* values, long* indices, long rows, long n, long k, int largest, hipStream_t s) {
     using S = typename Elem<T>::store_t;
+    if (n <= 4 * kWave) {
+        const dim3 gw(static_cast<unsigned>((rows + kWaves - 1) / kWaves)), b(kBlock);
+        if (n <= kWave)
+            hipLaunchKernelGGL((topk_rows_wave_kernel<T, 1>), gw, b, 0, s, static_cast<const S*>(x), static_cast<S*>(values), indices, rows, (int)n, (int)k, largest);
+        else
+            hipLaunchKernelGGL((topk_rows_wave_kernel<T, 4>), gw, b, 0, s, static_cast<const S*>(x), static_cast<S*>(values), indices, rows, (int)n, (int)k, largest);
+        PARAS_HIP_TRY(hipGetLastError());
+        return PARAS_OK;
+    }
     hipLaunchKernelGGL((topk_rows_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(kBlock), 0, s, static_cast<const S*>(x),
                        static_cast<S*>(values), indices, n, k, largest);
     PARAS_HIP_TRY(hipGetLastError());

@@ -27,7 +27,8 @@ def assert_gemm_close(out, ref, dtype):
     assert bool((err <= tol).all()), f"worst {err.max().item():.3e}, {(err > tol).sum().item()} beyond one ulp"
 
 
-SHAPES = [(128, 256, 64), (1, 8, 64), (130, 257, 128), (300, 100, 192), (512, 1024, 1024), (77, 4096, 320)]
+SHAPES = [(128, 256, 64), (1, 8, 64), (130, 257, 128), (300, 100, 192), (512, 1024, 1024), (77, 4096, 320),
+          (4100, 2100, 64)]     # the last one: 256-row tiles with a single k-tile
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

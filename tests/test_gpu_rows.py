@@ -14,7 +14,7 @@ FLOATS = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
 
 
 @pytest.mark.parametrize("dtype", FLOATS)
-@pytest.mark.parametrize("shape", [(1, 1), (7, 8), (33, 300), (4, 5000), (2, 3, 129)])
+@pytest.mark.parametrize("shape", [(1, 1), (7, 8), (33, 300), (4, 5000), (2, 3, 129), (1001, 64), (37, 65), (10, 256), (3, 257)])
 def test_softmax_matches_oracle(dtype, shape):
     torch.manual_seed(sum(shape))
     x = (3 * torch.randn(*shape)).to(dtype)
@@ -45,7 +45,8 @@ def test_softmax_half_to_float_and_extremes():
 @pytest.mark.parametrize("largest", [True, False])
 def test_topk_matches_oracle_bitwise(dtype, largest):
     torch.manual_seed(11)
-    for shape, k in (((5, 8), 2), ((9, 64), 8), ((3, 1000), 17), ((2, 2, 300), 300), ((4, 7), 0)):
+    for shape, k in (((5, 8), 2), ((9, 64), 8), ((3, 1000), 17), ((2, 2, 300), 300), ((4, 7), 0), ((1001, 64), 2),
+                     ((37, 65), 65), ((10, 256), 5), ((3, 257), 4)):
         x = torch.randn(*shape).to(dtype)
         x = (x * 4).round() / 4 if dtype != torch.float64 else x          # quantised: plenty of ties
         gv, gi = capi.topk_rows(x.cuda(), k, largest)
@@ -65,3 +66,16 @@ def test_topk_reference_tie_literal_and_torch_parity():
     assert torch.equal(i.cpu(), ti) and torch.equal(v.cpu(), tv)
     with pytest.raises(capi.ParasError, match="k out of range"):
         capi.topk_rows(y.cuda(), 300)
+
+
+def test_short_rows_with_nan_and_infinities():
+    """The one-wave-per-row kernels keep the host engine's conventions: a NaN never becomes the
+    row maximum of a softmax; a top-k slot with no candidate reports index -1 and value 0."""
+    x = torch.tensor([[1.0, float("nan"), 3.0, 2.0], [float("nan")] * 4, [float("inf"), 1.0, float("-inf"), 0.5]])
+    got, want = capi.softmax_rows(x.cuda()).cpu(), O.softmax_last(x)
+    assert torch.equal(got.isnan(), want.isnan())
+    assert torch.allclose(got.nan_to_num(7.0), want.nan_to_num(7.0), rtol=1e-6, atol=0)
+    gv, gi = capi.topk_rows(x.cuda(), 3)
+    wv, wi = O.topk_last(x, 3)
+    assert_bit_exact(gi, wi, "topk indices with NaN rows")
+    assert torch.equal(gv.cpu().isnan(), wv.isnan()) and torch.equal(gv.cpu().nan_to_num(7.0), wv.nan_to_num(7.0))
