@@ -69,6 +69,52 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const typename Ele
     for (long j = threadIdx.x; j < n; j += kBlock) outr[j] = EO::from_f64(exp(EI::to_f64(xr[j]) - m) / s);
 }
 
+// Rows of up to kBlock * EPT elements: the same, with each thread's exponentials kept in
+// registers between the sum and the division (one fp64 exp per element instead of two, one read
+// of the row instead of three).
+template <typename TI, typename TO, int EPT>
+__global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(const typename Elem<TI>::store_t* __restrict__ x,
+                                                                  typename Elem<TO>::store_t* __restrict__ out, int n) {
+    using EI = Elem<TI>;
+    using EO = Elem<TO>;
+    __shared__ double slots[2][kWaves];
+    const auto* xr = x + static_cast<long>(blockIdx.x) * n;
+    auto* outr = out + static_cast<long>(blockIdx.x) * n;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    double v[EPT];
+    double m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+        const int j = threadIdx.x + i * kBlock;
+        v[i] = j < n ? EI::to_f64(xr[j]) : -INFINITY;
+        if (j < n && v[i] > m) m = v[i];        // as the host: a NaN never replaces the max
+    }
+    m = wave_max_f64(m);
+    if (lane == 0) slots[0][wave] = m;
+    __syncthreads();
+    m = slots[0][0];
+#pragma unroll
+    for (int i = 1; i < kWaves; ++i) m = fmax(m, slots[0][i]);
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+        const int j = threadIdx.x + i * kBlock;
+        v[i] = j < n ? exp(v[i] - m) : 0.0;
+        sum += v[i];
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) slots[1][wave] = sum;
+    __syncthreads();
+    sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) sum += slots[1][i];
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+        const int j = threadIdx.x + i * kBlock;
+        if (j < n) outr[j] = EO::from_f64(v[i] / sum);
+    }
+}
+
 // (value, index) order of the reference: larger value first (smaller when !largest), then lower index.
 __device__ __forceinline__ bool comes_before(double va, long ia, double vb, long ib, bool largest) {
     return largest ? (va > vb || (va == vb && ia < ib)) : (va < vb || (va == vb && ia < ib));
@@ -236,6 +282,19 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
         } else {
             if (widen) hipLaunchKernelGGL((softmax_rows_wave_kernel<TI, float, 4>), gw, b, 0, s, xs, static_cast<float*>(out), rows, (int)n);
             else       hipLaunchKernelGGL((softmax_rows_wave_kernel<TI, TI, 4>), gw, b, 0, s, xs, static_cast<SI*>(out), rows, (int)n);
+        }
+        PARAS_HIP_TRY(hipGetLastError());
+        return PARAS_OK;
+    }
+    if (n <= 16 * kBlock) {
+        const bool widen = dtype_out == PARAS_F32 && sizeof(SI) == 2;
+        const auto* xs = static_cast<const SI*>(x);
+        if (n <= 4 * kBlock) {
+            if (widen) hipLaunchKernelGGL((softmax_rows_reg_kernel<TI, float, 4>), g, b, 0, s, xs, static_cast<float*>(out), (int)n);
+            else       hipLaunchKernelGGL((softmax_rows_reg_kernel<TI, TI, 4>), g, b, 0, s, xs, static_cast<SI*>(out), (int)n);
+        } else {
+            if (widen) hipLaunchKernelGGL((softmax_rows_reg_kernel<TI, float, 16>), g, b, 0, s, xs, static_cast<float*>(out), (int)n);
+            else       hipLaunchKernelGGL((softmax_rows_reg_kernel<TI, TI, 16>), g, b, 0, s, xs, static_cast<SI*>(out), (int)n);
         }
         PARAS_HIP_TRY(hipGetLastError());
         return PARAS_OK;

@@ -14,7 +14,7 @@ FLOATS = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
 
 
 @pytest.mark.parametrize("dtype", FLOATS)
-@pytest.mark.parametrize("shape", [(1, 1), (7, 8), (33, 300), (4, 5000), (2, 3, 129), (1001, 64), (37, 65), (10, 256), (3, 257)])
+@pytest.mark.parametrize("shape", [(1, 1), (7, 8), (33, 300), (4, 5000), (2, 3, 129), (1001, 64), (37, 65), (10, 256), (3, 257), (5, 1024), (3, 1025), (2, 4096), (2, 4097)])
 def test_softmax_matches_oracle(dtype, shape):
     torch.manual_seed(sum(shape))
     x = (3 * torch.randn(*shape)).to(dtype)
