@@ -102,6 +102,7 @@ struct FlashParams {
     // or additive values of the tensor dtype
     const unsigned char* mask;
     long ms_b, ms_h, ms_q, ms_k;
+    float inv_scale;   // the scores are kept unscaled: an additive mask value m enters as m / scale
 };
 
 template <typename T> struct Mma;
@@ -232,17 +233,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
         const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            // scale * log2(e) goes into q once (rounded back to the operand type), so the score
-            // accumulators are exponents of 2 as they leave the MFMA
-            const i16x8 raw = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
-            u32x4 sc4;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                sc4[e] = Mma<T>::pack2(Elem<T>::to_f32(static_cast<std::uint16_t>(raw[2 * e])) * p.scale_log2,
-                                       Elem<T>::to_f32(static_cast<std::uint16_t>(raw[2 * e + 1])) * p.scale_log2);
-            qreg[qb][ks] = __builtin_bit_cast(i16x8, sc4);
-        }
+        for (int ks = 0; ks < KSTEPS; ++ks) qreg[qb][ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
     }
 
     const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
@@ -293,20 +284,12 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         __syncthreads();
     };
 
-    // Online softmax state.  m_run is the reference exponent (scores are in units of log2 already):
-    // a score accumulator starts from sinit = -m_run in all its registers, so it comes out of the
-    // MFMAs as s - m_run, ready for v_exp.  m_run is finite from the start (0 until the first key
-    // with a finite score has been seen: `seen`, which then sets it to that block's maximum whatever
-    // its sign, so that uniformly very negative scores do not underflow).
-    float16_t oacc[QB][DBLK], sinit[QB];
+    float16_t oacc[QB][DBLK];
     float m_run[QB], l_run[QB];
-    bool seen = false;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-        m_run[qb] = 0.f;
+        m_run[qb] = -INFINITY;
         l_run[qb] = 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sinit[qb][r] = 0.f;
 #pragma unroll
         for (int i = 0; i < DBLK; ++i)
 #pragma unroll
@@ -327,7 +310,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         for (int db = 0; db < DBLK; ++db)
             v_rd[db] = vrow * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
     }
-    const float lazy_margin = 8.0f;   // exponent-of-2 units
+    const float lazy_margin = 8.0f / p.scale_log2;
 
     auto needs_mask = [&](int j, int qb) { return (kCausal && j * 32 + 31 > q0 + 32 * qb) || j * 32 + 32 > p.Lk; };
     auto apply_mask = [&](int j, int qb, float16_t& sc) {
@@ -381,7 +364,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const std::uint16_t bits = static_cast<std::uint16_t>(mr[r >> 1] >> (16 * (r & 1)));
-                sc[r] = fmaf(Elem<T>::to_f32(bits), 1.4426950408889634f, sc[r]);
+                sc[r] = fmaf(Elem<T>::to_f32(bits), p.inv_scale, sc[r]);
             }
         }
     };
@@ -391,35 +374,25 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
         return mx;
     };
-    // `mx` is the maximum of the finished scores `sc` of a block (this lane's half of the keys),
-    // relative to m_run.  Moves the reference up if a score exceeds it by more than the margin
-    // (rare after the first block): O and l are rescaled, and `sc` itself, which was formed
-    // against the old reference, is shifted to the new one.
-    auto raise_max = [&](float (&mx)[QB], float16_t (&sc)[QB]) {
-        // The test runs on each lane's own half of the keys; the two halves of a query are only
-        // brought together (and `seen` updated) inside the rare branch.
+    // Raise the running max of query block qb if block max `mx` (this lane's half) needs it.  The
+    // test runs on each lane's own half of the keys; the two halves of a query are only brought
+    // together inside the rare branch.
+    auto raise_max = [&](float (&mx)[QB]) {
         bool grow = false;
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) grow = grow || (seen ? mx[qb] > lazy_margin : mx[qb] > -INFINITY);
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // wave-uniform
+        for (int qb = 0; qb < QB; ++qb) grow = grow || (mx[qb] > m_run[qb] + lazy_margin);
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // wave-uniform, rare after block 0
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
-                const float mloc = half_swap_max(mx[qb]);
-                // lanes that need no move still take any upward one; an all-masked block moves nothing
-                const float delta = seen ? fmaxf(mloc, 0.f) : (mloc > -INFINITY ? mloc : 0.f);
-                const float alpha = __builtin_amdgcn_exp2f(-delta);
-                m_run[qb] += delta;
+                const float m_new = fmaxf(m_run[qb], half_swap_max(mx[qb]));
+                // (equal covers -inf on both sides: a query that has seen no key yet keeps its zeros)
+                const float alpha = m_run[qb] == m_new ? 1.f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.scale_log2);
+                m_run[qb] = m_new;
                 l_run[qb] *= alpha;
 #pragma unroll
                 for (int i = 0; i < DBLK; ++i)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) oacc[qb][i][r] *= alpha;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    sc[qb][r] -= delta;
-                    sinit[qb][r] = -m_run[qb];
-                }
-                if (qb == 0) seen = seen || mloc > -INFINITY;
             }
         }
     };
@@ -431,7 +404,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             if (needs_mask(j, qb)) apply_mask(j, qb, sc[qb]);
             if (kMask != 0 || needs_mask(j, qb)) mx[qb] = lane_max(sc[qb]);
         }
-        raise_max(mx, sc);
+        raise_max(mx);
     };
 
     // One block: exponentials of `cur` = S(j) and, if kNext, the MFMAs of S(j+1) into `nxt`,
@@ -441,7 +414,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     // block expects the operands of its first two slots in flight and, in its last two slots,
     // requests those of its successor (`tail`: KFirst = a block that starts with score MFMAs,
     // VFirst = one that only has PV left, NoTail = the successor's rows are not resident yet).
-    // The 8*QB exp pairs (2 exp + cvt + 2 add each) are spread between the MFMAs so the
+    // The 8*QB exp pairs (2 fma + 2 exp + cvt + 2 add each) are spread between the MFMAs so the
     // matrix pipe has an instruction in flight while the VALU works.  P(s2=0) is complete
     // before the first PV MFMA, P(s2=1) before the first PV MFMA that uses it; the row maxima
     // of S(j+1) are reduced as a tree in the slots after the last exp pair, so the rescale
@@ -475,13 +448,20 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         constexpr bool kTail = !std::is_same<decltype(tail), NoTail>::value;
         constexpr int S0 = kNext ? 0 : KSTEPS;           // first slot that exists
         static_assert(QB == 1, "the max tree below is written for one query block per wave");
+        float mc[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            mc[qb] = m_run[qb] * p.scale_log2;
+            // every key so far masked out: the reference point is arbitrary, and it must not be -inf
+            if constexpr (kMask != 0) mc[qb] = m_run[qb] == -INFINITY ? 0.f : mc[qb];
+        }
         std::uint32_t mnext[MREGS];
         if constexpr (kNext) mask_load(j + 1, mnext);
         u32x4 pw[QB][2];
         float mx[QB], t3[5], t2[2];
         auto exp_pair = [&](int qb, int i) {              // elements 2i, 2i+1 of cur[qb]
-            const float e0 = __builtin_amdgcn_exp2f(cur[qb][2 * i]);
-            const float e1 = __builtin_amdgcn_exp2f(cur[qb][2 * i + 1]);
+            const float e0 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i], p.scale_log2, -mc[qb]));
+            const float e1 = __builtin_amdgcn_exp2f(fmaf(cur[qb][2 * i + 1], p.scale_log2, -mc[qb]));
             const std::uint32_t w = Mma<T>::pack2(e0, e1);
             // Plain adds of the unrounded exponentials: v_dot2_f32_bf16 on the packed pair is one
             // instruction instead of two, but it runs on the matrix pipe's side and stalls the
@@ -507,7 +487,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             if (c < KSTEPS) {
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) {
-                    nxt[qb] = Mma<T>::run(frag[c % 4], qreg[qb][c], c == 0 ? sinit[qb] : nxt[qb]);
+                    if (c == 0) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) nxt[qb][r] = 0.f;
+                    }
+                    nxt[qb] = Mma<T>::run(frag[c % 4], qreg[qb][c], nxt[qb]);
                 }
             } else {
                 const int s2 = (c - KSTEPS) / DBLK, db = (c - KSTEPS) % DBLK;
@@ -548,9 +532,10 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
 #pragma unroll
+            for (int r = 0; r < 16; ++r) s_a[qb][r] = 0.f;
+#pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks)
-                s_a[qb] = Mma<T>::run(*reinterpret_cast<const i16x8*>(&k_lds0[32 * D + k_rd[ks]]), qreg[qb][ks],
-                                      ks == 0 ? sinit[qb] : s_a[qb]);
+                s_a[qb] = Mma<T>::run(*reinterpret_cast<const i16x8*>(&k_lds0[32 * D + k_rd[ks]]), qreg[qb][ks], s_a[qb]);
             mx[qb] = lane_max(s_a[qb]);
         }
         std::uint32_t m0[MREGS];
@@ -617,7 +602,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
                     *reinterpret_cast<u32x2*>(op + d) = w;
                 }
             if (p.lse != nullptr && lh == 0)
-                p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run[qb] * 0.6931471805599453f + logf(l_tot);
+                p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run[qb] * p.scale + logf(l_tot);
         }
     }
 }
@@ -679,6 +664,7 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     p.scale_log2 = static_cast<float>(a.scale * 1.4426950408889634);
     p.mask = static_cast<const unsigned char*>(a.mask);
     p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2]; p.ms_k = a.mask_strides[3];
+    p.inv_scale = static_cast<float>(1.0 / a.scale);
     const bool causal = a.is_causal != 0;
     const int mk = a.mask_kind;
     if (a.dtype == PARAS_BF16)

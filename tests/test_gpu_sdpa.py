@@ -114,12 +114,34 @@ def test_flash_matches_oracle(dtype, shape):
     s = (q.float() @ k.float().repeat_interleave(rep, 1).transpose(-1, -2)) / math.sqrt(D)
     if causal:
         s = s.masked_fill(~torch.ones(Lq, Lk).tril().bool(), -math.inf)
-    # The kernel sums the row denominator from the probabilities as rounded to the
-    # 16-bit MFMA operand (so numerator and denominator see the same rounding):
-    # one probability carries up to 2^-9 (bf16) / 2^-12 (f16) relative error, and
-    # a row dominated by one key passes that on to exp(lse).
-    tol = 4e-3 if dtype == torch.bfloat16 else 1e-3
+    # Scores are accumulated in fp32 from the unmodified operands and the row denominator is
+    # summed from the unrounded exponentials, so the log-sum-exp is good to fp32 round-off.
+    tol = 2e-4
     assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_flash_accuracy_with_large_scores(dtype):
+    """Inputs twice and four times the usual magnitude (score spread x4 / x16): the error against
+    the exact fp64 result must stay that of rounding P and O to the operand type.  Rounding a
+    pre-scaled q or k instead of scaling the fp32 scores would double it and show up in the
+    log-sum-exp first."""
+    torch.manual_seed(4)
+    B, H, S, D = 1, 4, 1024, 128
+    for mag, bar in ((2.0, 1.1e-3), (4.0, 1.3e-3)):          # mean absolute error, bf16; f16 an eighth of it
+        q, k = (mag * torch.randn(B, H, S, D)).to(dtype), (mag * torch.randn(B, H, S, D)).to(dtype)
+        v = torch.randn(B, H, S, D).to(dtype)
+        for causal in (True, False):
+            out, _, lse, kern = run(q, k, v, is_causal=causal, want_lse=True)
+            assert kern == "flash_mfma"
+            s = (q.double() @ k.double().transpose(-1, -2)) / math.sqrt(D)
+            if causal:
+                s = s.masked_fill(~torch.ones(S, S).tril().bool(), -math.inf)
+            want = torch.softmax(s, -1) @ v.double()
+            err = (out.double().cpu() - want).abs()
+            assert err.mean().item() <= (bar if dtype == torch.bfloat16 else bar / 8), f"mag {mag} causal {causal}: {err.mean().item()}"
+            assert err.max().item() <= (4e-2 if dtype == torch.bfloat16 else 5e-3)   # about one unit in the last place of |out| <= 4
+            assert torch.allclose(lse.double().cpu(), torch.logsumexp(s, -1), rtol=0, atol=5e-4)
 
 
 def test_flash_strided_inputs_and_explicit_scale():
