@@ -126,7 +126,8 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
     const int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
     const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
-    const bool use_wide = wide_tiles >= 128;       // measured: faster from half a round of one workgroup per CU upwards
+    // measured: faster from half a round of one workgroup per CU upwards (given rows to fill a tile)
+    const bool use_wide = wide_tiles >= 128 && M > gemm::kBM;
     const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
     const int64_t m_tiles = (M + bm - 1) / bm;
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
