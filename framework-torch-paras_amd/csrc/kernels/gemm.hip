@@ -97,6 +97,148 @@ __global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const Den
             }
 }
 
+// ---- few rows (M <= 128): the decode-time projections.  The product is bound by streaming the
+// weights once, so there is no tile and no LDS staging: a workgroup owns 16 weight rows, its eight
+// waves split the contraction (k-steps of 32 dealt round-robin, so the eight read adjacent 64-byte
+// pieces of each row), every wave feeds v_mfma_f32_16x16x32 straight from global memory (weights
+// as the row operand, non-temporal; the few activation rows from L2), and the eight partial
+// results meet in LDS in wave order.  Lane l of a 16x16 result holds activation row l%16 and
+// weight rows 4*(l/16) .. +3: four adjacent outputs, stored as one 8-byte piece when aligned.
+template <typename T> struct Mma16;
+template <> struct Mma16<bf16_t> {
+    __device__ static __forceinline__ float4_t run(u32x4 a, u32x4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma16<f16_t> {
+    __device__ static __forceinline__ float4_t run(u32x4 a, u32x4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+constexpr int kSkinnyWaves = 8;
+constexpr int kSkinnyMaxM = 128;
+
+template <typename T, int MB, int NB>   // MB = 16-row blocks of activations, NB = 16-row blocks of weights per workgroup
+__global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const DenseParams p) {
+    using El = Elem<T>;
+    __shared__ float4_t part[kSkinnyWaves][NB * MB][64];
+    const long bidx = blockIdx.y;
+    const std::uint16_t* A = p.a + bidx * p.sa;
+    const std::uint16_t* B = p.b + bidx * p.sb;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, kg = lane >> 4;
+    const long n0 = static_cast<long>(blockIdx.x) * (16 * NB);
+    const std::uint16_t* wp[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        long wrow = n0 + nb * 16 + r16;
+        if (wrow >= p.N) wrow = p.N - 1;                    // clamped rows are computed but never stored
+        wp[nb] = B + wrow * p.ldb + kg * 8;
+    }
+    const std::uint16_t* xp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        long xrow = mb * 16 + r16;
+        if (xrow >= p.M) xrow = p.M - 1;
+        xp[mb] = A + xrow * p.lda + kg * 8;
+    }
+    float4_t acc[NB][MB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const long ksteps = p.K / 32;
+    // A batch of k-steps: every load of the batch is requested before its first MFMA, so a wave
+    // pays the memory latency once per batch.
+    constexpr int kUnroll = MB <= 4 ? 4 : 2;
+    long ks = wave;
+    for (; ks + (kUnroll - 1) * kSkinnyWaves < ksteps; ks += kUnroll * kSkinnyWaves) {
+        u32x4 wv[kUnroll][NB], xv[kUnroll][MB];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) wv[u][nb] = load16_nt(wp[nb] + (ks + u * kSkinnyWaves) * 32);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) xv[u][mb] = load16(xp[mb] + (ks + u * kSkinnyWaves) * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[u][nb], xv[u][mb], acc[nb][mb]);
+    }
+    for (; ks < ksteps; ks += kSkinnyWaves) {
+        u32x4 wv[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) wv[nb] = load16_nt(wp[nb] + ks * 32);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const u32x4 xv = load16(xp[mb] + ks * 32);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[nb], xv, acc[nb][mb]);
+        }
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) part[wave][nb * MB + mb][lane] = acc[nb][mb];
+    __syncthreads();
+    // wave w finishes result blocks w, w + 8, ...
+    std::uint16_t* C = p.c + bidx * p.sc;
+    const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
+    const bool vec_ok = (p.ldc % 4 == 0) && (p.sc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
+    for (int blk = wave; blk < NB * MB; blk += kSkinnyWaves) {
+        const int nb = blk / MB, mb = blk % MB;
+        float4_t t = part[0][blk][lane];
+#pragma unroll
+        for (int w = 1; w < kSkinnyWaves; ++w) {
+            const float4_t o = part[w][blk][lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) t[r] += o[r];
+        }
+        const long row = mb * 16 + r16;
+        const long col = n0 + nb * 16 + 4 * kg;
+        if (row >= p.M) continue;
+        std::uint16_t o16[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = p.alpha * t[r];
+            if (ADD && col + r < p.N) v = fmaf(p.beta, El::to_f32(ADD[row * p.ld_add + col + r]), v);
+            o16[r] = El::from_f32(v);
+        }
+        if (vec_ok && col + 3 < p.N) {
+            u32x2 w2;
+            w2[0] = o16[0] | (static_cast<std::uint32_t>(o16[1]) << 16);
+            w2[1] = o16[2] | (static_cast<std::uint32_t>(o16[3]) << 16);
+            *reinterpret_cast<u32x2*>(C + row * p.ldc + col) = w2;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (col + r < p.N) C[row * p.ldc + col + r] = o16[r];
+        }
+    }
+}
+
+// Two blocks of weight rows per workgroup when that still leaves a workgroup for every CU: every
+// activation fragment then feeds two MFMAs, which halves the reads of the activations from L2.
+template <typename T>
+void launch_skinny(const DenseParams& p, long batch, hipStream_t s) {
+    const dim3 block(kSkinnyWaves * 64);
+    const int mb = static_cast<int>((p.M + 15) / 16);
+    const dim3 g1(static_cast<unsigned>((p.N + 15) / 16), static_cast<unsigned>(batch));
+    const dim3 g2(static_cast<unsigned>((p.N + 31) / 32), static_cast<unsigned>(batch));
+    const bool two = mb > 1 && static_cast<long>(g2.x) * batch >= 256;
+    if (mb <= 1)      hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 1, 1>), g1, block, 0, s, p);
+    else if (mb <= 2) { if (two) hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 2, 2>), g2, block, 0, s, p);
+                        else     hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 2, 1>), g1, block, 0, s, p); }
+    else if (mb <= 4) { if (two) hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 4, 2>), g2, block, 0, s, p);
+                        else     hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 4, 1>), g1, block, 0, s, p); }
+    else              { if (two) hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 8, 2>), g2, block, 0, s, p);
+                        else     hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 8, 1>), g1, block, 0, s, p); }
+}
+
 template <typename T, typename S>
 void launch_dense(const DenseParams& p, unsigned grid, hipStream_t s) {
     hipLaunchKernelGGL((dense_gemm_nt_kernel<T, S>), dim3(grid), dim3(S::kThreads), 0, s, p);
@@ -146,6 +288,12 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     p.sa = stride_a; p.sb = stride_b; p.sc = stride_c; p.sadd = stride_add;
     p.m_tiles = static_cast<int>(m_tiles); p.n_units = static_cast<int>(n_units);
     p.alpha = static_cast<float>(alpha); p.beta = static_cast<float>(beta);
+    if (M <= kSkinnyMaxM && batch <= 65535 && (N + 15) / 16 <= 0x7fffffffLL) {
+        if (dtype == PARAS_BF16) launch_skinny<bf16_t>(p, batch, s);
+        else                     launch_skinny<f16_t>(p, batch, s);
+        PARAS_HIP_TRY(hipGetLastError());
+        return PARAS_OK;
+    }
     const unsigned blocks = static_cast<unsigned>(m_tiles * n_units * batch);
     if (use_wide) {
         if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile256>(p, blocks, s);

@@ -6,6 +6,8 @@ in double and rounds once.  Bar: every element within one 16-bit ulp of the
 oracle (summation order is the only difference), and torch-CPU addmm / linear
 as the library check for the epilogue.
 """
+import math
+
 import pytest
 import torch
 
@@ -132,3 +134,36 @@ def test_gemm_nt_256_row_tiles_agree_with_128_row_tiles():
         assert torch.equal(whole[i], capi.gemm_nt(a[i], b[i])), f"batch {i}"
     ref = O.matmul_nt(a[3, -3:].cpu(), b[3].cpu())
     assert_gemm_close(whole[3, -3:], ref, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (16, 100, 64), (17, 1027, 320), (64, 4096, 1024), (100, 515, 192),
+                                   (128, 2050, 4096)])
+def test_gemm_nt_few_rows(shape, dtype):
+    """M <= 128 (decode-time projections) runs on the weight-streaming kernel: plain product,
+    bias + scaled addend, N with and without 8-byte aligned output rows."""
+    M, N, K = shape
+    torch.manual_seed(M + N + K)
+    a = torch.randn(M, K).to(dtype)
+    b = (torch.randn(N, K) / math.sqrt(K)).to(dtype)
+    assert_gemm_close(capi.gemm_nt(a.cuda(), b.cuda()), O.matmul_nt(a, b), dtype)
+    bias = torch.randn(N).to(dtype)
+    got = capi.gemm_nt(a.cuda(), b.cuda(), bias.cuda(), alpha=1.0, beta=1.0)
+    assert_gemm_close(got, torch.nn.functional.linear(a, b, bias), dtype)
+    addm = torch.randn(M, N).to(dtype)
+    got = capi.gemm_nt(a.cuda(), b.cuda(), addm.cuda(), alpha=0.5, beta=2.0)
+    want = torch.addmm(addm.float(), a.float(), b.float().t(), beta=2.0, alpha=0.5)
+    err = (got.float().cpu() - want).abs()
+    assert bool((err <= 2 * ulp16(want, dtype) + 1e-6).all())
+
+
+def test_gemm_nt_few_rows_batched():
+    torch.manual_seed(8)
+    a = torch.randn(6, 40, 256, device="cuda").bfloat16()
+    b = (0.1 * torch.randn(6, 72, 256, device="cuda")).bfloat16()
+    out = capi.gemm_nt(a, b)
+    for i in range(6):
+        assert_gemm_close(out[i], O.matmul_nt(a[i].cpu(), b[i].cpu()), torch.bfloat16)
+    shared = capi.gemm_nt(a, b[0])                      # one weight matrix for the whole batch
+    for i in range(6):
+        assert torch.equal(shared[i], capi.gemm_nt(a[i], b[0]))
