@@ -1,8 +1,10 @@
 // Tensor plumbing kernels for the `paras` device: strided copy with optional
 // float-type conversion, strided fill, and the two "composed" ops whose
 // reference implementations narrow to the tensor dtype after every step.
-// None of these is a performance target; they keep whole expressions on the
-// device so that the hot-path kernels are not surrounded by host bounces.
+// The copies keep whole expressions on the device so that the hot-path kernels
+// are not surrounded by host bounces; the two composed ops are what
+// F.rms_norm and torch_paras::swiglu reach on this device and stream at the
+// rate of their fused counterparts for the 16-bit dtypes.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -10,6 +12,7 @@
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
+#include "kernels/swiglu_math.h"
 
 namespace paras {
 namespace {
@@ -123,10 +126,131 @@ __global__ __launch_bounds__(kBlock) void swiglu_composed_kernel(const typename 
     }
 }
 
+// ---- 16-bit dtypes, 16-byte aligned rows: the same results at streaming speed.  Every product
+// of two 16-bit values is exact in fp32 (at most 22 significant bits), so "multiply in fp64, narrow"
+// is one fp32 multiply and one rounding; only the row sum needs fp64.  silu narrowed to T is the
+// fused SwiGLU element function with an up value of one.
+template <typename T, int NV>
+__global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_composed_vec(
+    const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w, std::uint16_t* __restrict__ out, long rows,
+    int H, double eps_narrowed) {
+    using E = Elem<T>;
+    constexpr int kWaves = kBlock / kWave;
+    __shared__ double slots[2 * kWaves];
+    const int nvec = H / 8;
+    u32x4 wv[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * kBlock;
+        if (w != nullptr && c < nvec) wv[i] = load16(w + static_cast<long>(c) * 8);
+    }
+    int calls = 0;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        u32x4 xv[NV];
+        double acc = 0.0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * kBlock;
+            if (c < nvec) {
+                xv[i] = load16_nt(x + r * H + static_cast<long>(c) * 8);
+                const std::uint16_t* e = reinterpret_cast<const std::uint16_t*>(&xv[i]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float v = E::to_f32(e[j]);
+                    acc += static_cast<double>(E::to_f32(E::from_f32(v * v)));
+                }
+            }
+        }
+        acc = wave_sum(acc);
+        double* set = slots + (calls++ & 1) * kWaves;        // alternating sets: one barrier per row
+        if ((threadIdx.x & (kWave - 1)) == 0) set[threadIdx.x / kWave] = acc;
+        __syncthreads();
+        double sum = 0.0;
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) sum += set[i];
+        const double s = narrow<T>(sum);
+        const double m = narrow<T>(s * (1.0 / static_cast<double>(H)));
+        const double a = narrow<T>(m + 1.0 * eps_narrowed);
+        const float inv = static_cast<float>(narrow<T>(1.0 / sqrt(a)));
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * kBlock;
+            if (c < nvec) {
+                const std::uint16_t* e = reinterpret_cast<const std::uint16_t*>(&xv[i]);
+                const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
+                u32x4 o;
+                std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    std::uint16_t y = E::from_f32(E::to_f32(e[j]) * inv);
+                    if (w != nullptr) y = E::from_f32(E::to_f32(y) * E::to_f32(we[j]));
+                    oe[j] = y;
+                }
+                store16_nt(out + r * H + static_cast<long>(c) * 8, o);
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_composed_vec(const std::uint16_t* __restrict__ x,
+                                                              const std::uint16_t* __restrict__ gate,
+                                                              std::uint16_t* __restrict__ out, long nvec) {
+    using E = Elem<T>;
+    const std::uint16_t one = E::from_f32(1.0f);
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += static_cast<long>(gridDim.x) * kBlock) {
+        const u32x4 xv = load16_nt(x + i * 8), gv = load16_nt(gate + i * 8);
+        const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv);
+        const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv);
+        u32x4 o;
+        std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) oe[j] = E::from_f32(E::to_f32(xe[j]) * E::to_f32(swiglu_one<T>(ge[j], one)));
+        store16_nt(out + i * 8, o);
+    }
+}
+
 unsigned grid_for(long n) {
     long g = (n + kBlock - 1) / kBlock;
     if (g > 65536) g = 65536;
     return static_cast<unsigned>(g < 1 ? 1 : g);
+}
+
+// Launches the register-resident kernel if the row shape allows it; false = use the general one.
+template <typename T>
+bool launch_rms_composed_vec(const void* x, const void* w, void* out, long rows, long H, double eps_narrowed, dim3 g,
+                             hipStream_t st) {
+    const bool aligned = H % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
+                                         reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const long nvec = H / 8;
+    if (!aligned || nvec > 4 * kBlock) return false;
+    const auto* xs = static_cast<const std::uint16_t*>(x);
+    const auto* ws = static_cast<const std::uint16_t*>(w);
+    auto* os = static_cast<std::uint16_t*>(out);
+    const dim3 b(kBlock);
+    if (nvec <= kBlock)          hipLaunchKernelGGL((rms_norm_composed_vec<T, 1>), g, b, 0, st, xs, ws, os, rows, (int)H, eps_narrowed);
+    else if (nvec <= 2 * kBlock) hipLaunchKernelGGL((rms_norm_composed_vec<T, 2>), g, b, 0, st, xs, ws, os, rows, (int)H, eps_narrowed);
+    else                         hipLaunchKernelGGL((rms_norm_composed_vec<T, 4>), g, b, 0, st, xs, ws, os, rows, (int)H, eps_narrowed);
+    return true;
+}
+
+// 16-byte vectors on the streaming kernel, the last n % 8 elements (or everything, if unaligned) on the scalar one.
+template <typename T>
+void launch_swiglu_composed16(const void* x, const void* gate, void* out, long n, hipStream_t st) {
+    const auto* xs = static_cast<const std::uint16_t*>(x);
+    const auto* gs = static_cast<const std::uint16_t*>(gate);
+    auto* os = static_cast<std::uint16_t*>(out);
+    long done = 0;
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 && n >= 8) {
+        const long nvec = n / 8;
+        long blocks = (nvec + kBlock - 1) / kBlock;
+        if (blocks > 0x7fffffffL) blocks = 0x7fffffffL;      // the kernel grid-strides beyond that
+        hipLaunchKernelGGL((swiglu_composed_vec<T>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, st, xs, gs, os, nvec);
+        done = nvec * 8;
+    }
+    if (done < n)
+        hipLaunchKernelGGL((swiglu_composed_kernel<T>), dim3(grid_for(n - done)), dim3(kBlock), 0, st, xs + done, gs + done,
+                           os + done, n - done);
 }
 
 int make_spec(int ndim, const int64_t* sizes, const int64_t* ss, const int64_t* ds, Strided* s, long* n) {
@@ -291,15 +415,17 @@ int paras_rms_norm_composed_fwd(const void* x, const void* w, void* out, int64_t
             u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
             float en;
             __builtin_memcpy(&en, &u, 4);
-            hipLaunchKernelGGL((rms_norm_composed_kernel<bf16_t>), g, b, 0, st, static_cast<const uint16_t*>(x),
-                               static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), (long)rows, (long)H,
-                               static_cast<double>(en));
+            if (!launch_rms_composed_vec<bf16_t>(x, w, out, rows, H, static_cast<double>(en), g, st))
+                hipLaunchKernelGGL((rms_norm_composed_kernel<bf16_t>), g, b, 0, st, static_cast<const uint16_t*>(x),
+                                   static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), (long)rows, (long)H,
+                                   static_cast<double>(en));
             break;
         }
         case PARAS_F16: {
             const double en = static_cast<double>(static_cast<float>(static_cast<_Float16>(static_cast<float>(eps))));
-            hipLaunchKernelGGL((rms_norm_composed_kernel<f16_t>), g, b, 0, st, static_cast<const uint16_t*>(x),
-                               static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), (long)rows, (long)H, en);
+            if (!launch_rms_composed_vec<f16_t>(x, w, out, rows, H, en, g, st))
+                hipLaunchKernelGGL((rms_norm_composed_kernel<f16_t>), g, b, 0, st, static_cast<const uint16_t*>(x),
+                                   static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), (long)rows, (long)H, en);
             break;
         }
         default: return fail(PARAS_ERR_INVALID, "paras_rms_norm_composed_fwd: unknown dtype %d", dtype);
@@ -320,8 +446,8 @@ int paras_swiglu_composed_fwd(const void* x, const void* gate, void* out, int64_
     switch (dtype) {
         case PARAS_F32:  hipLaunchKernelGGL((swiglu_composed_kernel<float>), g, b, 0, st, static_cast<const float*>(x), static_cast<const float*>(gate), static_cast<float*>(out), (long)n); break;
         case PARAS_F64:  hipLaunchKernelGGL((swiglu_composed_kernel<double>), g, b, 0, st, static_cast<const double*>(x), static_cast<const double*>(gate), static_cast<double*>(out), (long)n); break;
-        case PARAS_BF16: hipLaunchKernelGGL((swiglu_composed_kernel<bf16_t>), g, b, 0, st, static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(out), (long)n); break;
-        case PARAS_F16:  hipLaunchKernelGGL((swiglu_composed_kernel<f16_t>), g, b, 0, st, static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(out), (long)n); break;
+        case PARAS_BF16: launch_swiglu_composed16<bf16_t>(x, gate, out, n, st); break;
+        case PARAS_F16:  launch_swiglu_composed16<f16_t>(x, gate, out, n, st); break;
         default: return fail(PARAS_ERR_INVALID, "paras_swiglu_composed_fwd: unknown dtype %d", dtype);
     }
     PARAS_HIP_TRY(hipGetLastError());

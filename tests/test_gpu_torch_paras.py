@@ -209,6 +209,34 @@ def test_composed_ops_narrow_like_the_host_engine(device):
         assert_bit_exact(got.cpu(), O.swiglu_composed(u, g), f"torch_paras::swiglu {dt}")
 
 
+def test_composed_ops_streaming_kernels_are_exact(device):
+    """The 16-bit streaming forms of aten::rms_norm and torch_paras::swiglu against the oracle's
+    step-by-step narrowing: row sizes on each register tier and on the general kernel, with and
+    without weight, every representable bf16 gate, tiny and huge magnitudes."""
+    for dt in (torch.bfloat16, torch.float16):
+        for H in (8, 264, 2048, 4096, 8192, 1000, 8200):
+            x, w = (2 * torch.randn(19, H)).to(dt), (1 + 0.1 * torch.randn(H)).to(dt)
+            got = torch.ops.aten.rms_norm(x.to(device), [H], w.to(device), 1e-6)
+            assert_bit_exact(got.cpu(), O.rms_norm_composed(x, [H], w, 1e-6), f"aten::rms_norm {dt} H={H}")
+            got = torch.ops.aten.rms_norm(x.to(device), [H], None, 1e-6)
+            assert_bit_exact(got.cpu(), O.rms_norm_composed(x, [H], None, 1e-6), f"aten::rms_norm no weight {dt} H={H}")
+        scale = 1e-18 if dt == torch.bfloat16 else 1e-3
+        x = (scale * torch.randn(5, 512)).to(dt)
+        got = torch.ops.aten.rms_norm(x.to(device), [512], None, 1e-6)
+        assert_bit_exact(got.cpu(), O.rms_norm_composed(x, [512], None, 1e-6), f"aten::rms_norm tiny {dt}")
+        g = (4 * torch.randn(5, 1031)).to(dt)
+        u = (torch.randn(5, 1031) * torch.tensor([1e-30, 1.0, 1e3, 1e-3, 30.0]).view(5, 1)).to(dt)
+        got = torch.ops.torch_paras.swiglu(u.to(device), g.to(device))
+        assert_bit_exact(got.cpu(), O.swiglu_composed(u, g), f"torch_paras::swiglu {dt}")
+    gate = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    for xv in (1.0, -0.3, 7.25):
+        x = torch.full_like(gate, xv)
+        got = torch.ops.torch_paras.swiglu(x.to(device), gate.to(device))
+        want = O.swiglu_composed(x, gate)
+        both_nan = got.cpu().isnan() & want.isnan()
+        assert torch.equal(got.cpu().view(torch.int16)[~both_nan], want.view(torch.int16)[~both_nan]), f"all gates, x={xv}"
+
+
 def test_swiglu(device):
     x, gate = torch.randn(4, 32), torch.randn(4, 32)
     assert_close(torch.ops.torch_paras.swiglu(x.to(device), gate.to(device)), torch.ops.torch_paras.swiglu(x, gate), "swiglu")
