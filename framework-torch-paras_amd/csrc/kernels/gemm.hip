@@ -31,14 +31,14 @@ struct DenseParams {
     long M, N, K;
     long lda, ldb, ldc, ld_add;
     long sa, sb, sc, sadd;      // batch strides (elements)
-    int  m_tiles, n_units;      // row tiles (128 or 256 rows), 256-column units
+    int  m_tiles, n_units;      // row tiles (128 or 256 rows), column units (128 or 256 columns)
     float alpha, beta;
 };
 
 // S = Tile128 (4 waves, 128 rows) or Tile256 (8 waves, 256 rows; for problems with at least
 // 128 tiles of 256 x 256).
 template <typename T, typename S>
-__global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const DenseParams p) {
+__global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_gemm_nt_kernel(const DenseParams p) {
     using El = Elem<T>;
     __shared__ __attribute__((aligned(16))) typename S::Lds lds;
 
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const Den
     const long per_batch = static_cast<long>(p.m_tiles) * p.n_units;
     const long bidx = blockIdx.x / per_batch, rem = blockIdx.x % per_batch;
     const int mt = static_cast<int>(rem / p.n_units), nu = static_cast<int>(rem % p.n_units);
-    const long row0 = static_cast<long>(mt) * S::kBM, n0 = static_cast<long>(nu) * 2 * kBN;
+    const long row0 = static_cast<long>(mt) * S::kBM, n0 = static_cast<long>(nu) * S::kGroups * kBN;
     const std::uint16_t* A = p.a + bidx * p.sa;
     const std::uint16_t* B = p.b + bidx * p.sb;
 
@@ -55,7 +55,8 @@ __global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const Den
     const int lr = lane & 31, lh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
 
-    unsigned a_off[4], b_off[2][S::kBChunks];
+    constexpr int G = S::kGroups;
+    unsigned a_off[4], b_off[G][S::kBChunks];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int c = tid + i * S::kThreads;
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const Den
         a_off[i] = static_cast<unsigned>(arow * p.lda + (c & 7) * 8);
     }
 #pragma unroll
-    for (int g = 0; g < 2; ++g)
+    for (int g = 0; g < G; ++g)
 #pragma unroll
         for (int i = 0; i < S::kBChunks; ++i) {
             const int c = tid + i * S::kThreads;
@@ -72,14 +73,16 @@ __global__ __launch_bounds__(S::kThreads, 2) void dense_gemm_nt_kernel(const Den
             if (brow >= p.N) brow = p.N - 1;
             b_off[g][i] = static_cast<unsigned>(brow * p.ldb + (c & 7) * 8);
         }
-    const std::uint16_t* const b_base[2] = {B, B};
-    float16_t acc[2][2][2];
+    const std::uint16_t* b_base[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) b_base[g] = B;
+    float16_t acc[G][2][2];
     S::template mainloop<T>(A, a_off, b_base, b_off, p.K, lds, acc);
 
     std::uint16_t* C = p.c + bidx * p.sc;
     const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
 #pragma unroll
-    for (int g = 0; g < 2; ++g)
+    for (int g = 0; g < G; ++g)
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
@@ -266,12 +269,15 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) != 0 || lda % 8 != 0 || ldb % 8 != 0 ||
         stride_a % 8 != 0 || stride_b % 8 != 0)
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
-    const int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
+    int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
     const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
     // measured: faster from half a round of one workgroup per CU upwards (given rows to fill a tile)
     const bool use_wide = wide_tiles >= 128 && M > gemm::kBM;
     const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
     const int64_t m_tiles = (M + bm - 1) / bm;
+    // fewer 128 x 256 tiles than the chip holds at once (two per CU): 128 x 128 tiles, twice as many
+    const bool use_square = !use_wide && m_tiles * n_units * batch < 512 && N > gemm::kBN;
+    if (use_square) n_units = (N + gemm::kBN - 1) / gemm::kBN;
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
     if (M * lda >= (1LL << 32) || N * ldb >= (1LL << 32))
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: an operand matrix spans 2^32 elements or more");
@@ -298,6 +304,9 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     if (use_wide) {
         if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile256>(p, blocks, s);
         else                     launch_dense<f16_t, gemm::Tile256>(p, blocks, s);
+    } else if (use_square) {
+        if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile128x128>(p, blocks, s);
+        else                     launch_dense<f16_t, gemm::Tile128x128>(p, blocks, s);
     } else {
         if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile128>(p, blocks, s);
         else                     launch_dense<f16_t, gemm::Tile128>(p, blocks, s);

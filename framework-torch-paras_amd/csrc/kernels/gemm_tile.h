@@ -43,10 +43,12 @@ template <> struct MmaT<f16_t> {
 };
 
 
-struct TileLds {
+template <int G>     // G column groups of 128
+struct TileLdsG {
     std::uint16_t a[kBM * kLS];
-    std::uint16_t b[2][kBN * kLS];
+    std::uint16_t b[G][kBN * kLS];
 };
+using TileLds = TileLdsG<2>;
 
 // a_off[i] / b_off[g][i]: element offsets (from the uniform bases a_base / b_base[g]) of this
 // thread's four 16-byte chunks per operand row set at k = 0 (chunk c = tid + i*256 -> tile row
@@ -54,21 +56,21 @@ struct TileLds {
 // vector registers; callers check that every operand spans fewer than 2^32 elements.
 // Accumulates into acc[g][mi][ni]; lane (column lr = lane%32, half lh = lane/32) of
 // block (mi, ni) ends up holding rows (r/4)*8 + 4*lh + r%4, r = 0..15.
-template <typename T>
+template <typename T, int G>
 __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
-                                              const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][4],
-                                              long K, TileLds& lds, float16_t (&acc)[2][2][2]) {
+                                              const std::uint16_t* const (&b_base)[G], const unsigned (&b_off)[G][4],
+                                              long K, TileLdsG<G>& lds, float16_t (&acc)[G][2][2]) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
     std::uint16_t* a_lds = lds.a;
     std::uint16_t (*b_lds)[kBN * kLS] = lds.b;
-    u32x4 a_st[4], b_st[2][4];
+    u32x4 a_st[4], b_st[G][4];
     auto load_tile = [&](long k0) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) a_st[i] = load16(a_base + k0 + a_off[i]);
 #pragma unroll
-        for (int g = 0; g < 2; ++g)
+        for (int g = 0; g < G; ++g)
 #pragma unroll
             for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_base[g] + k0 + b_off[g][i]);
     };
@@ -78,13 +80,13 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
             const int c = tid + i * kThreads;
             const int off = (c >> 3) * kLS + (c & 7) * 8;
             *reinterpret_cast<u32x4*>(&a_lds[off]) = a_st[i];
-            *reinterpret_cast<u32x4*>(&b_lds[0][off]) = b_st[0][i];
-            *reinterpret_cast<u32x4*>(&b_lds[1][off]) = b_st[1][i];
+#pragma unroll
+            for (int g = 0; g < G; ++g) *reinterpret_cast<u32x4*>(&b_lds[g][off]) = b_st[g][i];
         }
     };
 
 #pragma unroll
-    for (int g = 0; g < 2; ++g)
+    for (int g = 0; g < G; ++g)
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
@@ -104,7 +106,8 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
         // k-step requested while the current one computes (A into a second register pair right
         // away, each B fragment back into its own registers as soon as its two MFMAs have
         // issued), so an operand is asked for about six MFMAs before it is used.
-        i16x8 af[2][2], bf[4];
+        constexpr int Q = 2 * G;               // B fragments per k-step
+        i16x8 af[2][2], bf[Q];
         auto read_a = [&](int buf, int ks) {
 #pragma unroll
             for (int mi = 0; mi < 2; ++mi)
@@ -115,13 +118,13 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
         };
         read_a(0, 0);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) read_b(q, 0);
+        for (int q = 0; q < Q; ++q) read_b(q, 0);
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) {
             const int cur = ks & 1;
             const bool more = ks + 1 < kBK / 16;
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
+            for (int q = 0; q < Q; ++q)
 #pragma unroll
                 for (int mi = 0; mi < 2; ++mi) {
                     acc[q >> 1][mi][q & 1] = MmaT<T>::run(af[cur][mi], bf[q], acc[q >> 1][mi][q & 1]);
@@ -255,18 +258,21 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
 }  // namespace wide
 
 // The two tile shapes as a kernel sees them.
-struct Tile128 {
-    static constexpr int kBM = gemm::kBM, kThreads = gemm::kThreads, kBChunks = 4;
-    using Lds = TileLds;
+template <int G>
+struct Tile128G {
+    static constexpr int kBM = gemm::kBM, kThreads = gemm::kThreads, kBChunks = 4, kGroups = G;
+    using Lds = TileLdsG<G>;
     template <typename T>
     __device__ static __forceinline__ void mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
-                                                    const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][4],
-                                                    long K, Lds& lds, float16_t (&acc)[2][2][2]) {
-        tile_mainloop<T>(a_base, a_off, b_base, b_off, K, lds, acc);
+                                                    const std::uint16_t* const (&b_base)[G], const unsigned (&b_off)[G][4],
+                                                    long K, Lds& lds, float16_t (&acc)[G][2][2]) {
+        tile_mainloop<T, G>(a_base, a_off, b_base, b_off, K, lds, acc);
     }
 };
+using Tile128 = Tile128G<2>;
+using Tile128x128 = Tile128G<1>;     // one column group: twice the workgroups for problems that would not fill the chip
 struct Tile256 {
-    static constexpr int kBM = wide::kBM, kThreads = wide::kThreads, kBChunks = 2;
+    static constexpr int kBM = wide::kBM, kThreads = wide::kThreads, kBChunks = 2, kGroups = 2;
     using Lds = wide::TileLds;
     template <typename T>
     __device__ static __forceinline__ void mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
