@@ -35,8 +35,8 @@ struct DenseParams {
     float alpha, beta;
 };
 
-// S = Tile128 (4 waves, 128 rows) or Tile256 (8 waves, 256 rows; for problems with at least
-// 128 tiles of 256 x 256).
+// S = Tile256 (8 waves, 256 x 256; for problems with at least 144 such tiles), Tile128 (4 waves,
+// 128 x 256) or Tile128x128 (4 waves, one column group; when there would be fewer than 512 tiles of 128 x 256).
 template <typename T, typename S>
 __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_gemm_nt_kernel(const DenseParams p) {
     using El = Elem<T>;
@@ -271,8 +271,9 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
         return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
     int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
     const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
-    // measured: faster from half a round of one workgroup per CU upwards (given rows to fill a tile)
-    const bool use_wide = wide_tiles >= 128 && M > gemm::kBM;
+    // measured: faster from a little over half a round of one workgroup per CU upwards (at exactly 128
+    // tiles the 128 x 128 tiling below wins by 10-25 %, at 160 the 256-row tiles win by 20 %)
+    const bool use_wide = wide_tiles >= 144 && M > gemm::kBM;
     const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
     const int64_t m_tiles = (M + bm - 1) / bm;
     // fewer 128 x 256 tiles than the chip holds at once (two per CU): 128 x 128 tiles, twice as many

@@ -125,7 +125,7 @@ def test_gemm_nt_256_row_tiles_agree_with_128_row_tiles():
     both forms add the same products in the same order, so they agree bit for bit (ragged M and
     N, strided batch)."""
     torch.manual_seed(21)
-    Bt, M, N, K = 4, 2100, 2100, 128      # 81 tiles of 256 x 256 each, 324 together
+    Bt, M, N, K = 4, 2100, 2100, 128      # 81 tiles of 256 x 256 each (-> 128 x 128 tiles), 324 together (-> 256-row tiles)
     a = torch.randn(Bt, M, K, device="cuda").bfloat16()
     b = (0.1 * torch.randn(Bt, N, K, device="cuda")).bfloat16()
     whole = capi.gemm_nt(a, b)
