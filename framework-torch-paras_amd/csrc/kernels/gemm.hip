@@ -12,6 +12,8 @@
 // (a bias) over all rows.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
@@ -33,6 +35,7 @@ struct DenseParams {
     long sa, sb, sc, sadd;      // batch strides (elements)
     int  m_tiles, n_units;      // row tiles (128 or 256 rows), column units (128 or 256 columns)
     float alpha, beta;
+    double alpha64, beta64;     // the same, for fp64 tensors
 };
 
 // S = Tile256 (8 waves, 256 x 256; for problems with at least 144 such tiles), Tile128 (4 waves,
@@ -242,6 +245,92 @@ void launch_skinny(const DenseParams& p, long batch, hipStream_t s) {
                         else     hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 8, 1>), g1, block, 0, s, p); }
 }
 
+// ---- any float dtype, any contraction size, any alignment: the product for what the MFMA kernels
+// do not take (fp32 / fp64 tensors, K not a multiple of 64, rows that are not 16-byte aligned), so
+// that no GEMM leaves the device.  64 x 64 outputs per workgroup, 4 x 4 per thread, k-tiles of 16
+// through LDS; fp32 accumulation (fp64 for fp64 tensors) and one rounding, as ATen-CPU does.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_nt_any_kernel(const typename Elem<T>::store_t* __restrict__ a,
+                                                          const typename Elem<T>::store_t* __restrict__ b,
+                                                          const typename Elem<T>::store_t* __restrict__ add,
+                                                          typename Elem<T>::store_t* __restrict__ c, const DenseParams p) {
+    using El = Elem<T>;
+    using Acc = typename std::conditional<sizeof(typename El::store_t) == 8, double, float>::type;
+    constexpr int BM = 64, BN = 64, BKK = 16;
+    __shared__ Acc as[BKK][BM + 1], bs[BKK][BN + 1];
+    const long bidx = blockIdx.z;
+    const auto* A = a + bidx * p.sa;
+    const auto* B = b + bidx * p.sb;
+    const long row0 = static_cast<long>(blockIdx.y) * BM, col0 = static_cast<long>(blockIdx.x) * BN;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int lrow = threadIdx.x >> 2, lk = (threadIdx.x & 3) * 4;     // staging: 64 rows x 16 k, 4 k per thread
+    auto widen = [](typename El::store_t v) -> Acc {
+        if constexpr (sizeof(typename El::store_t) == 8) return El::to_f64(v);
+        else return El::to_f32(v);
+    };
+    Acc acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0;
+    for (long k0 = 0; k0 < p.K; k0 += BKK) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const long k = k0 + lk + e;
+            const long ar = row0 + lrow, br = col0 + lrow;
+            as[lk + e][lrow] = (ar < p.M && k < p.K) ? widen(A[ar * p.lda + k]) : Acc(0);
+            bs[lk + e][lrow] = (br < p.N && k < p.K) ? widen(B[br * p.ldb + k]) : Acc(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BKK; ++kk) {
+            Acc av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = as[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bv[j] = bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+        }
+        __syncthreads();
+    }
+    auto* C = c + bidx * p.sc;
+    const auto* ADD = add ? add + bidx * p.sadd : nullptr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const long row = row0 + ty * 4 + i;
+        if (row >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long col = col0 + tx * 4 + j;
+            if (col >= p.N) continue;
+            if constexpr (sizeof(typename El::store_t) == 8) {
+                double v = static_cast<double>(p.alpha64) * acc[i][j];
+                if (ADD) v += p.beta64 * El::to_f64(ADD[row * p.ld_add + col]);
+                C[row * p.ldc + col] = El::from_f64(v);
+            } else {
+                float v = p.alpha * acc[i][j];
+                if (ADD) v = fmaf(p.beta, El::to_f32(ADD[row * p.ld_add + col]), v);
+                C[row * p.ldc + col] = El::from_f32(v);
+            }
+        }
+    }
+}
+
+template <typename T>
+int launch_any(const DenseParams& p, const void* a, const void* b, const void* add, void* c, long batch, hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    const long gx = (p.N + 63) / 64, gy = (p.M + 63) / 64;
+    PARAS_REQUIRE(gx <= 0x7fffffffL && gy <= 65535 && batch <= 65535, "paras_gemm_nt: shape too large for the general kernel");
+    hipLaunchKernelGGL((gemm_nt_any_kernel<T>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy), static_cast<unsigned>(batch)),
+                       dim3(256), 0, s, static_cast<const S*>(a), static_cast<const S*>(b), static_cast<const S*>(add),
+                       static_cast<S*>(c), p);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
 template <typename T, typename S>
 void launch_dense(const DenseParams& p, unsigned grid, hipStream_t s) {
     hipLaunchKernelGGL((dense_gemm_nt_kernel<T, S>), dim3(grid), dim3(S::kThreads), 0, s, p);
@@ -259,29 +348,11 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     using namespace paras;
     PARAS_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "paras_gemm_nt: negative shape");
     if (M == 0 || N == 0 || batch == 0) return PARAS_OK;
-    PARAS_REQUIRE(dtype == PARAS_BF16 || dtype == PARAS_F16, "paras_gemm_nt: dtype must be bf16 or f16");
-    if (K == 0 || K % gemm::kBK != 0)
-        return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: the contraction size (%lld) must be a positive multiple of %d",
-                    (long long)K, gemm::kBK);
-    PARAS_REQUIRE(a && b && c, "paras_gemm_nt: null pointer");
+    PARAS_REQUIRE(dtype == PARAS_BF16 || dtype == PARAS_F16 || dtype == PARAS_F32 || dtype == PARAS_F64,
+                  "paras_gemm_nt: unknown dtype");
+    PARAS_REQUIRE(c && (K == 0 || (a && b)), "paras_gemm_nt: null pointer");   // an empty contraction has no operands to read
     PARAS_REQUIRE(lda >= K && ldb >= K && ldc >= N && (addend == nullptr || ld_add == 0 || ld_add >= N),
                   "paras_gemm_nt: a leading dimension is smaller than its row");
-    if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) != 0 || lda % 8 != 0 || ldb % 8 != 0 ||
-        stride_a % 8 != 0 || stride_b % 8 != 0)
-        return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: operand rows must be 16-byte aligned");
-    int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
-    const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
-    // measured: faster from a little over half a round of one workgroup per CU upwards (at exactly 128
-    // tiles the 128 x 128 tiling below wins by 10-25 %, at 160 the 256-row tiles win by 20 %)
-    const bool use_wide = wide_tiles >= 144 && M > gemm::kBM;
-    const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
-    const int64_t m_tiles = (M + bm - 1) / bm;
-    // fewer 128 x 256 tiles than the chip holds at once (two per CU): 128 x 128 tiles, twice as many
-    const bool use_square = !use_wide && m_tiles * n_units * batch < 512 && N > gemm::kBN;
-    if (use_square) n_units = (N + gemm::kBN - 1) / gemm::kBN;
-    PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
-    if (M * lda >= (1LL << 32) || N * ldb >= (1LL << 32))
-        return fail(PARAS_ERR_UNSUPPORTED, "paras_gemm_nt: an operand matrix spans 2^32 elements or more");
     hipStream_t s = nullptr;
     int rc = resolve_stream(stream, &s);
     if (rc != PARAS_OK) return rc;
@@ -293,8 +364,33 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     p.M = M; p.N = N; p.K = K;
     p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.ld_add = ld_add;
     p.sa = stride_a; p.sb = stride_b; p.sc = stride_c; p.sadd = stride_add;
-    p.m_tiles = static_cast<int>(m_tiles); p.n_units = static_cast<int>(n_units);
     p.alpha = static_cast<float>(alpha); p.beta = static_cast<float>(beta);
+    p.alpha64 = alpha; p.beta64 = beta;
+    // What the MFMA kernels take: 16-bit floats, K a positive multiple of 64, 16-byte aligned operand
+    // rows, operands of fewer than 2^32 elements.  Everything else runs on the general kernel.
+    const bool mfma_ok = (dtype == PARAS_BF16 || dtype == PARAS_F16) && K > 0 && K % gemm::kBK == 0 &&
+                         ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0 && lda % 8 == 0 &&
+                         ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0 && M * lda < (1LL << 32) && N * ldb < (1LL << 32);
+    if (!mfma_ok) {
+        switch (dtype) {
+            case PARAS_F32:  return launch_any<float>(p, a, b, addend, c, batch, s);
+            case PARAS_F64:  return launch_any<double>(p, a, b, addend, c, batch, s);
+            case PARAS_BF16: return launch_any<bf16_t>(p, a, b, addend, c, batch, s);
+            default:         return launch_any<f16_t>(p, a, b, addend, c, batch, s);
+        }
+    }
+    int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
+    const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
+    // measured: faster from a little over half a round of one workgroup per CU upwards (at exactly 128
+    // tiles the 128 x 128 tiling below wins by 10-25 %, at 160 the 256-row tiles win by 20 %)
+    const bool use_wide = wide_tiles >= 144 && M > gemm::kBM;
+    const int64_t bm = use_wide ? gemm::wide::kBM : gemm::kBM;
+    const int64_t m_tiles = (M + bm - 1) / bm;
+    // fewer 128 x 256 tiles than the chip holds at once (two per CU): 128 x 128 tiles, twice as many
+    const bool use_square = !use_wide && m_tiles * n_units * batch < 512 && N > gemm::kBN;
+    if (use_square) n_units = (N + gemm::kBN - 1) / gemm::kBN;
+    PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
+    p.m_tiles = static_cast<int>(m_tiles); p.n_units = static_cast<int>(n_units);
     if (M <= kSkinnyMaxM && batch <= 65535 && (N + 15) / 16 <= 0x7fffffffLL) {
         if (dtype == PARAS_BF16) launch_skinny<bf16_t>(p, batch, s);
         else                     launch_skinny<f16_t>(p, batch, s);

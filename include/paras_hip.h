@@ -279,9 +279,11 @@ PARAS_API int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up,
 /* A [M, K] rows lda apart, B [N, K] rows ldb apart (both contiguous along K:  */
 /* x W^T of nn.Linear, q k^T), C [M, N] rows ldc apart; batch strides in       */
 /* elements (0 = shared).  addend may be NULL; ld_add = 0 broadcasts one row   */
-/* (a bias) over the M rows.  bf16 / f16 on MFMA; K must be a multiple of 64   */
-/* and operand rows 16-byte aligned (PARAS_ERR_UNSUPPORTED otherwise: the      */
-/* caller keeps its host path for those).                                      */
+/* (a bias) over the M rows.  All four float dtypes.  bf16 / f16 with K a       */
+/* multiple of 64 and 16-byte aligned operand rows run on the MFMA kernels     */
+/* (fp32 accumulation, one rounding); everything else -- fp32 / fp64 tensors,  */
+/* other K, other alignments -- on a general kernel (fp32 accumulation, fp64   */
+/* for fp64 tensors), so no product needs a host path.                         */
 /* ------------------------------------------------------------------------- */
 PARAS_API int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c,
                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,

@@ -76,11 +76,38 @@ def test_gemm_nt_batched_strided_and_shared_operand():
 
 def test_gemm_nt_errors_and_empty():
     z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(capi.ParasError, match="multiple of 64"):
-        capi.gemm_nt(z(8, 72), z(8, 72))
-    with pytest.raises(capi.ParasError, match="bf16 or f16"):
-        capi.gemm_nt(torch.zeros(8, 64, device="cuda"), torch.zeros(8, 64, device="cuda"))
+    with pytest.raises(capi.ParasError, match="leading dimension"):
+        a = z(8, 64)
+        capi.check(capi.lib().paras_gemm_nt(a.data_ptr(), a.data_ptr(), None, a.data_ptr(), 8, 8, 64, 32, 64, 8, 0, 1, 0, 0, 0, 0,
+                                            1.0, 0.0, capi.BF16, capi._stream()))
     assert capi.gemm_nt(z(0, 64), z(8, 64)).shape == (0, 8)
+    assert torch.equal(capi.gemm_nt(z(4, 0), z(8, 0)), z(4, 8))          # empty contraction: zeros
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16, torch.float16])
+def test_gemm_nt_general_kernel(dtype):
+    """What the MFMA kernels do not take -- fp32 / fp64 tensors, contraction sizes that are not a
+    multiple of 64, rows that are not 16-byte aligned -- runs on the general device kernel."""
+    torch.manual_seed(13)
+    for (M, N, K) in [(1, 1, 1), (17, 9, 30), (70, 130, 65), (64, 64, 16), (129, 65, 200)]:
+        a, b = torch.randn(M, K).to(dtype), (torch.randn(N, K) / math.sqrt(K)).to(dtype)
+        got = capi.gemm_nt(a.cuda(), b.cuda())
+        if dtype in (torch.bfloat16, torch.float16):
+            assert_gemm_close(got, O.matmul_nt(a, b), dtype)
+        else:
+            want = a.double() @ b.double().t()
+            tol = 1e-5 if dtype == torch.float32 else 1e-13
+            assert torch.allclose(got.double().cpu(), want, rtol=tol, atol=tol)
+        bias = torch.randn(N).to(dtype)
+        got = capi.gemm_nt(a.cuda(), b.cuda(), bias.cuda(), alpha=0.5, beta=2.0)
+        want = 0.5 * (a.double() @ b.double().t()) + 2.0 * bias.double()
+        tol = {torch.float32: 1e-5, torch.float64: 1e-13}.get(dtype, 2e-2)
+        assert torch.allclose(got.double().cpu(), want, rtol=tol, atol=tol)
+    if dtype == torch.bfloat16:                                              # a multiple of 64, but rows 2 bytes off alignment
+        buf = torch.randn(40 * 128 + 1).to(dtype).cuda()
+        a = buf[1:].view(40, 128)
+        b = (0.1 * torch.randn(24, 128)).to(dtype).cuda()
+        assert_gemm_close(capi.gemm_nt(a, b), O.matmul_nt(a.cpu(), b.cpu()), dtype)
 
 
 def test_gemm_nt_linearity_at_projection_size():

@@ -394,14 +394,28 @@ def test_linear_mm_bmm_addmm_on_device(device, dtype):
     _one_ulp(torch.matmul(q.to(device), k.to(device).transpose(-1, -2)), torch.matmul(q, k.transpose(-1, -2)), dtype)
 
 
-def test_gemm_other_dtypes_and_shapes_take_the_host_route(device):
+def test_gemm_other_dtypes_and_shapes_stay_on_the_device(device):
+    """fp32 / fp64 products and contraction sizes the MFMA kernels do not take run on the general
+    device kernel (reference tolerance against torch-CPU; fp32 accumulation and one rounding for the
+    16-bit dtypes, so those agree with ATen-CPU to one unit in the last place)."""
     torch.manual_seed(1)
     a, b = torch.randn(17, 30), torch.randn(30, 9)
     assert_close(torch.mm(a.to(device), b.to(device)), torch.mm(a, b), "fp32 mm")          # reference tolerance
-    a16, b16 = torch.randn(8, 24).bfloat16(), torch.randn(24, 8).bfloat16()                 # K not a multiple of 64
-    assert_bit_exact(torch.mm(a16.to(device), b16.to(device)), torch.mm(a16, b16), "bf16 mm, host route")
+    ad, bd = torch.randn(70, 130, dtype=torch.float64), torch.randn(130, 65, dtype=torch.float64)
+    assert torch.allclose(torch.mm(ad.to(device), bd.to(device)).cpu(), torch.mm(ad, bd), rtol=1e-12, atol=1e-12)
+    x, w, bias = torch.randn(5, 33, 100), torch.randn(77, 100), torch.randn(77)
+    assert_close(F.linear(x.to(device), w.to(device), bias.to(device)), F.linear(x, w, bias), "fp32 linear")
+    a3, b3 = torch.randn(3, 20, 31), torch.randn(3, 31, 12)
+    assert_close(torch.bmm(a3.to(device), b3.to(device)), torch.bmm(a3, b3), "fp32 bmm")
+    s_ = torch.randn(17, 9)
+    assert_close(torch.addmm(s_.to(device), a.to(device), b.to(device), beta=0.5, alpha=2.0), torch.addmm(s_, a, b, beta=0.5, alpha=2.0), "fp32 addmm")
+    for dt in (torch.bfloat16, torch.float16):
+        a16, b16 = torch.randn(8, 24).to(dt), torch.randn(24, 8).to(dt)                       # K not a multiple of 64
+        _one_ulp(torch.mm(a16.to(device), b16.to(device)), torch.mm(a16, b16), dt)
     with pytest.raises(RuntimeError):
         torch.mm(a.to(device), torch.randn(31, 9).to(device))
+    with pytest.raises(RuntimeError, match="float dtypes"):
+        torch.mm(torch.ones(4, 4, dtype=torch.int32).to(device), torch.ones(4, 4, dtype=torch.int32).to(device))
 
 
 def test_linear_backward_through_device_gemm(device):
