@@ -446,3 +446,42 @@ def test_softmax_and_topk_ops_on_device(device):
         assert torch.equal(i.cpu(), ti) and torch.equal(v.cpu(), tv)
     v, i = torch.topk(torch.tensor([[5, 3, 5, 5, 1, 3]]).to(device), 4)  # integer dtype: host route
     assert v.cpu().tolist() == [[5, 5, 5, 3]]
+
+
+def test_covered_ops_never_take_the_host_fallback():
+    """With PARAS_LOG=1 the device prints every op that goes through the dispatcher's CPU fallback:
+    none of the ops this build covers may appear there, in any dtype it registers."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, torch, torch.nn.functional as F
+sys.path.insert(0, sys.argv[1])
+import torch_paras
+dev = "paras:0"
+for dt in (torch.bfloat16, torch.float16, torch.float32):
+    q, k, v = (torch.randn(2, 4, 64, 64).to(dt).to(dev) for _ in range(3))
+    F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    F.scaled_dot_product_attention(q, k, v, attn_mask=(torch.rand(64, 64) > 0.3).to(dev))
+    x, w = torch.randn(8, 256).to(dt).to(dev), torch.randn(256).to(dt).to(dev)
+    F.rms_norm(x, (256,), w, 1e-6)
+    torch.ops.paras.rms_norm(x, w, 1e-6)
+    torch.ops.paras.swiglu(x, x)
+    torch.ops.torch_paras.swiglu(x, x)
+    W = torch.randn(128, 256).to(dt).to(dev)
+    F.linear(x, W)
+    torch.mm(x, W.t())
+    torch.bmm(x.view(2, 4, 256), W.t().expand(2, 256, 128))
+    torch.softmax(x, -1)
+    torch.topk(x, 2)
+torch_paras.synchronize()
+print("done")
+"""
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "framework-torch-paras_amd")
+    env = dict(os.environ, PARAS_LOG="1")
+    r = subprocess.run([sys.executable, "-c", code, root], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0 and "done" in r.stdout, r.stderr[-2000:]
+    fell = sorted({line.split("for ", 1)[1].strip() for line in r.stderr.splitlines() if "falling back to CPU for" in line})
+    covered = ("scaled_dot_product", "rms_norm", "swiglu", "linear", "mm", "softmax", "topk")
+    bad = [op for op in fell if any(c in op for c in covered)]
+    assert not bad, f"covered ops went through the host fallback: {bad} (all fallbacks: {fell})"
