@@ -83,6 +83,57 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_any(
     }
 }
 
+// 16-bit tensors, 16-byte aligned: eight elements per lane and access.  Every element goes through
+// the fp32 fast tier; the few whose result sits next to a rounding boundary (or outside the fast
+// tier's range) are collected in a bit mask and redone in fp64 in a loop that runs as often as the
+// lane with the most of them needs -- usually not at all, sometimes once.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_vec(const std::uint16_t* __restrict__ go,
+                                                         const std::uint16_t* __restrict__ gate,
+                                                         const std::uint16_t* __restrict__ up,
+                                                         std::uint16_t* __restrict__ ggate,
+                                                         std::uint16_t* __restrict__ gup, long nvec) {
+    using E = Elem<T>;
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += static_cast<long>(gridDim.x) * kBlock) {
+        const u32x4 dv = load16_nt(go + i * 8), gv = load16_nt(gate + i * 8), uv = load16_nt(up + i * 8);
+        const std::uint16_t* de = reinterpret_cast<const std::uint16_t*>(&dv);
+        const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv);
+        const std::uint16_t* ue = reinterpret_cast<const std::uint16_t*>(&uv);
+        std::uint16_t og[8], ou[8];
+        unsigned redo = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float yg, yu;
+            bool ok_g, ok_u;
+            swiglu_bwd_fast<T>(E::to_f32(de[j]), E::to_f32(ge[j]), E::to_f32(ue[j]), yg, yu, ok_g, ok_u);
+            og[j] = E::from_f32_finite(yg);
+            ou[j] = E::from_f32_finite(yu);
+            redo |= (ok_g && ok_u) ? 0u : (1u << j);
+        }
+        while (redo != 0) {
+            const int j = __builtin_ctz(redo);
+            redo &= redo - 1;
+            std::uint16_t d16 = 0, g16 = 0, u16 = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (k == j) { d16 = de[k]; g16 = ge[k]; u16 = ue[k]; }
+            std::uint16_t xg, xu;
+            swiglu_bwd_exact<T>(E::to_f32(d16), E::to_f32(g16), E::to_f32(u16), xg, xu);
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (k == j) { og[k] = xg; ou[k] = xu; }
+        }
+        u32x4 wg, wu;
+#pragma unroll
+        for (int p2 = 0; p2 < 4; ++p2) {
+            wg[p2] = og[2 * p2] | (static_cast<std::uint32_t>(og[2 * p2 + 1]) << 16);
+            wu[p2] = ou[2 * p2] | (static_cast<std::uint32_t>(ou[2 * p2 + 1]) << 16);
+        }
+        store16_nt(ggate + i * 8, wg);
+        store16_nt(gup + i * 8, wu);
+    }
+}
+
 // rotate_half (csrc/ops/fused_ops.cpp:254-263, 290-299): out[.., c] takes
 // x[.., c+half] (negated for forward) when c < half, else x[.., c-half]
 // (negated for backward).  Negation flips the sign bit, which is what
@@ -162,10 +213,29 @@ template <typename T>
 int launch_swiglu_bwd(const void* go, const void* gate, const void* up, void* ggate, void* gup, long n,
                       hipStream_t s) {
     using S = typename Elem<T>::store_t;
-    hipLaunchKernelGGL((swiglu_bwd_any<T>), dim3(stream_grid(kBlock, n)), dim3(kBlock), 0, s,
-                       static_cast<const S*>(go), static_cast<const S*>(gate), static_cast<const S*>(up),
-                       static_cast<S*>(ggate), static_cast<S*>(gup), n);
-    PARAS_HIP_TRY(hipGetLastError());
+    const auto* d = static_cast<const S*>(go);
+    const auto* g = static_cast<const S*>(gate);
+    const auto* u = static_cast<const S*>(up);
+    auto* og = static_cast<S*>(ggate);
+    auto* ou = static_cast<S*>(gup);
+    long done = 0;
+    if constexpr (sizeof(S) == 2) {
+        const bool aligned = ((reinterpret_cast<uintptr_t>(go) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) |
+                               reinterpret_cast<uintptr_t>(ggate) | reinterpret_cast<uintptr_t>(gup)) % 16) == 0;
+        if (aligned && n >= 8) {
+            const long nvec = n / 8;
+            long blocks = (nvec + kBlock - 1) / kBlock;
+            if (blocks > 0x7fffffffL) blocks = 0x7fffffffL;  // the kernel grid-strides beyond that
+            hipLaunchKernelGGL((swiglu_bwd_vec<T>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, s, d, g, u, og, ou, nvec);
+            PARAS_HIP_TRY(hipGetLastError());
+            done = nvec * 8;
+        }
+    }
+    if (done < n) {
+        hipLaunchKernelGGL((swiglu_bwd_any<T>), dim3(stream_grid(kBlock, n - done)), dim3(kBlock), 0, s, d + done, g + done,
+                           u + done, og + done, ou + done, n - done);
+        PARAS_HIP_TRY(hipGetLastError());
+    }
     return PARAS_OK;
 }
 

@@ -86,6 +86,54 @@ __device__ __forceinline__ typename Elem<T>::store_t swiglu_one(typename Elem<T>
     }
 }
 
+// ---- SwiGLU backward -----------------------------------------------------------
+// Host definition (csrc/ops/fused_ops.cpp:218-226), in fp64:
+//   s = 1/(1+exp(-g));  dup = (dy*g)*s;  dgate = (dy*u) * (s * (1 + g*(1-s)))
+// Fast tier in fp32 with e = exp2(-g*log2e), r = rcp(1+e) (= s), e*r (= 1-s, formed without the
+// cancellation of 1-s), q = 1 + g*(e*r).  Error bounds in units of 2^-24 relative (one rounding
+// = 1, v_exp_f32 / v_rcp_f32 = 2), with w = 1-s and Ee = 2|g| + 2 the error of e (argument
+// rounding, amplified by |g|, plus the instruction's own):
+//   r:      w*Ee + 3            (the error of e enters 1+e damped by w)
+//   dup:    w*Ee + 5
+//   e*r:    s*Ee + 4            (the errors of e in e and in r partly cancel)
+//   q:      absolute |g e r| (s*Ee + 5) + |q|, i.e. relative rho (s*Ee + 5) + 1, rho = |g e r| / |q|
+//   dgate:  w*Ee + 7 + rho (s*Ee + 5)
+// q crosses zero near g = -1.278: rho grows without bound there and those elements take the exact
+// tier.  The bounds are used with a factor 1.5 and 3 units of margin.  A relative error of E units
+// is less than E fp32 ulps of the result, which is what narrow_is_safe takes.
+template <typename T>
+__device__ __forceinline__ void swiglu_bwd_exact(float dy, float g, float u, typename Elem<T>::store_t& dgate,
+                                                 typename Elem<T>::store_t& dup) {
+    const double dyd = static_cast<double>(dy), gd = static_cast<double>(g), ud = static_cast<double>(u);
+    const double s = 1.0 / (1.0 + exp(-gd));
+    dup = Elem<T>::from_f64(dyd * gd * s);
+    dgate = Elem<T>::from_f64(dyd * ud * (s * (1.0 + gd * (1.0 - s))));
+}
+
+// Fast tier for one element of a 16-bit tensor: the fp32 results and whether each may be narrowed.
+template <typename T>
+__device__ __forceinline__ void swiglu_bwd_fast(float dy, float g, float u, float& yg, float& yu, bool& ok_g, bool& ok_u) {
+    const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
+    const float r = __builtin_amdgcn_rcpf(1.0f + e);
+    const float er = e * r;
+    yu = (dy * g) * r;
+    const float ger = g * er;
+    const float q = 1.0f + ger;
+    yg = (dy * u) * (r * q);
+    const float ee = fmaf(2.0f, fabsf(g), 2.0f);
+    const float eu = fmaf(er, ee, 5.0f);
+    const float rho = fabsf(ger) * __builtin_amdgcn_rcpf(fabsf(q));
+    const float eg = fmaf(rho, fmaf(r, ee, 5.0f), eu + 2.0f);
+    const bool in_range = (fabsf(g - 26.0f) <= 34.0f) && (rho < 4096.0f);     // -8 <= g <= 60, q well away from zero; false for NaN
+    const std::uint32_t ulps_u = static_cast<std::uint32_t>(fmaf(1.5f, eu, 3.0f));
+    const std::uint32_t ulps_g = static_cast<std::uint32_t>(fmaf(1.5f, in_range ? eg : 0.0f, 3.0f));
+    ok_u = in_range && narrow_is_safe<T>(yu, ulps_u);
+    ok_g = in_range && narrow_is_safe<T>(yg, ulps_g);
+    // exact signed zeros need no fp64 (zero padding stays on the fast tier)
+    ok_u = ok_u || (yu == 0.0f && (dy == 0.0f || g == 0.0f));
+    ok_g = ok_g || (yg == 0.0f && (dy == 0.0f || u == 0.0f) && in_range);
+}
+
 // ---- RMSNorm output ------------------------------------------------------------
 // out = T(x * rstd * w).  fp32: fl(fl(x*fl(rstd))*w) is within 3 * 2^-24
 // relative of the exact product (three roundings), i.e. at most 3 fp32 ulps; 4 is used.

@@ -167,3 +167,39 @@ def test_rotate_half_vector_path_and_fallbacks(dtype):
     xr = buf[1:].view(4, 128)
     got = capi.rotate_half(dev(buf)[1:].view(4, 128))
     assert_bit_exact(got, O.rotate_half(xr.contiguous()), "rotate_half unaligned")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_swiglu_backward_every_gate_value(dtype):
+    """The two-tier backward (fp32 with an error bound, fp64 next to rounding boundaries and around
+    the zero of silu' at g = -1.278) against the oracle for every representable gate, with grad_out /
+    up values of several magnitudes and signs, zeros included."""
+    gate = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(dtype)
+    for dyv, uv in ((1.0, 1.0), (-0.3, 7.25), (1e-3, -2.5), (3.0, 0.0), (0.0, 1.0), (-250.0, 0.015625), (1.7, -1e-2)):
+        dy, up = torch.full_like(gate, dyv), torch.full_like(gate, uv)
+        gg, gu = capi.swiglu_backward(dev(dy), dev(gate), dev(up))
+        wgg, wgu = O.swiglu_backward(dy, gate, up)
+        for got, want, name in ((gg, wgg, "grad_gate"), (gu, wgu, "grad_up")):
+            got = got.cpu()
+            assert torch.equal(got.isnan(), want.isnan()), f"{name}: NaN positions, dy={dyv} up={uv}"
+            keep = ~want.isnan()                       # (a NaN's sign and payload are not part of the contract)
+            bad = int((got.view(torch.int16)[keep] != want.view(torch.int16)[keep]).sum())
+            assert bad == 0, f"{name} for every gate, dy={dyv} up={uv}: {bad} elements differ bitwise"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_swiglu_backward_random_and_ragged(dtype):
+    torch.manual_seed(17)
+    for n, scale in ((8, 1.0), (1000003, 1.0), (4099, 6.0), (65536, 0.05)):
+        gate, up, dy = (scale * torch.randn(n)).to(dtype), torch.randn(n).to(dtype), torch.randn(n).to(dtype)
+        gg, gu = capi.swiglu_backward(dev(dy), dev(gate), dev(up))
+        wgg, wgu = O.swiglu_backward(dy, gate, up)
+        assert_bit_exact(gg, wgg, f"grad_gate n={n}")
+        assert_bit_exact(gu, wgu, f"grad_up n={n}")
+    # a view 2 bytes into its allocation: the element-wise kernel
+    buf = torch.randn(3, 1025).to(dtype)
+    g2, u2, d2 = buf[0, 1:], buf[1, 1:], buf[2, 1:]
+    gg, gu = capi.swiglu_backward(dev(buf)[2, 1:], dev(buf)[0, 1:], dev(buf)[1, 1:])
+    wgg, wgu = O.swiglu_backward(d2.contiguous(), g2.contiguous(), u2.contiguous())
+    assert_bit_exact(gg, wgg, "grad_gate unaligned")
+    assert_bit_exact(gu, wgu, "grad_up unaligned")
