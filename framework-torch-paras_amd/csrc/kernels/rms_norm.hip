@@ -218,19 +218,20 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final(
     gw[j] = E::from_f64(acc);
 }
 
-// 16-bit tensors with 16-byte aligned rows of at most kBlock*NV vectors: dx and the partial
+// 16-bit tensors with 16-byte aligned rows of at most BLOCK*NV vectors: dx and the partial
 // column sums in ONE pass over grad_out and x.  A workgroup owns a slab of kDwSlabRows rows; each
 // thread keeps the same NV vectors of every row (and of w), so its 8*NV column sums live in
 // registers across the slab, and the next row's vectors are requested before the current row's
 // reduction.  Arithmetic in fp64 in the host's order of operations.  (NV = 2 needs 136 registers:
 // three workgroups per CU.  Re-reading w per row to fit four measured 20 % slower.)
-template <typename T, int NV>
-__global__ __launch_bounds__(kBlock, (NV == 1 ? 4 : 3)) void rms_norm_bwd_fused(
+template <typename T, int NV, int BLOCK>
+__global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? 2 : (NV == 1 ? 4 : 3))) void rms_norm_bwd_fused(
     const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
     const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
     using E = Elem<T>;
     constexpr int V = 8;
-    __shared__ double slots[2 * kWavesPerBlock];
+    constexpr int kWaves = BLOCK / kWave;
+    __shared__ double slots[2 * kWaves];
     const int nvec = H / V;
     const long slab = blockIdx.x;
     const long r0 = slab * kDwSlabRows;
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(kBlock, (NV == 1 ? 4 : 3)) void rms_norm_bwd_fused(
     double dw[NV][V];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int c = threadIdx.x + i * kBlock;
+        const int c = threadIdx.x + i * BLOCK;
         have[i] = c < nvec;
         if (have[i]) {
             wv[i] = load16(w + static_cast<long>(c) * V);
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(kBlock, (NV == 1 ? 4 : 3)) void rms_norm_bwd_fused(
             gv[i] = gn[i];
             xv[i] = xn[i];
             if (have[i] && r + 1 < r1) {
-                const int c = threadIdx.x + i * kBlock;
+                const int c = threadIdx.x + i * BLOCK;
                 gn[i] = load16_nt(go + (r + 1) * H + static_cast<long>(c) * V);
                 xn[i] = load16_nt(x + (r + 1) * H + static_cast<long>(c) * V);
             }
@@ -277,7 +278,15 @@ __global__ __launch_bounds__(kBlock, (NV == 1 ? 4 : 3)) void rms_norm_bwd_fused(
                     dw[i][j] += g * xj * rr;
                 }
             }
-        dot = block_sum(dot, slots, sum_calls++);
+        {   // sum over the workgroup; two alternating slot sets, so one barrier per row
+            dot = wave_sum(dot);
+            double* set = slots + (sum_calls++ & 1) * kWaves;
+            if ((threadIdx.x & (kWave - 1)) == 0) set[threadIdx.x / kWave] = dot;
+            __syncthreads();
+            dot = 0.0;
+#pragma unroll
+            for (int i = 0; i < kWaves; ++i) dot += set[i];
+        }
         const double coef = rr * rr * rr / static_cast<double>(H);
 #pragma unroll
         for (int i = 0; i < NV; ++i)
@@ -290,13 +299,13 @@ __global__ __launch_bounds__(kBlock, (NV == 1 ? 4 : 3)) void rms_norm_bwd_fused(
 #pragma unroll
                 for (int j = 0; j < V; ++j)
                     oe[j] = E::from_f64(E::to_f64(ge[j]) * E::to_f64(we[j]) * rr - coef * E::to_f64(xe[j]) * dot);
-                store16_nt(gx + r * H + static_cast<long>(threadIdx.x + i * kBlock) * V, o);
+                store16_nt(gx + r * H + static_cast<long>(threadIdx.x + i * BLOCK) * V, o);
             }
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i)
         if (have[i]) {
-            double* dst = partial + slab * H + static_cast<long>(threadIdx.x + i * kBlock) * V;
+            double* dst = partial + slab * H + static_cast<long>(threadIdx.x + i * BLOCK) * V;
 #pragma unroll
             for (int j = 0; j < V; ++j) dst[j] = dw[i][j];
         }
@@ -367,16 +376,19 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
         const bool aligned = (H % 8 == 0) && ((reinterpret_cast<uintptr_t>(go) | reinterpret_cast<uintptr_t>(x) |
                                                reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gx)) % 16 == 0);
         const long nvec = H / 8;
-        if (aligned && nvec <= kBlock * 2) {
+        if (aligned && nvec <= 512 * 2) {
             const auto* g16 = static_cast<const std::uint16_t*>(go);
             const auto* x16 = static_cast<const std::uint16_t*>(x);
             const auto* w16 = static_cast<const std::uint16_t*>(w);
             auto* gx16 = static_cast<std::uint16_t*>(gx);
             auto* part = static_cast<double*>(workspace);
+            const dim3 grid(static_cast<unsigned>(slabs));
             if (nvec <= kBlock)
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1>), dim3(static_cast<unsigned>(slabs)), dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
-            else
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 2>), dim3(static_cast<unsigned>(slabs)), dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, kBlock>), grid, dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            else if (nvec <= kBlock * 2)
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 2, kBlock>), grid, dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            else   // rows of up to 8192 elements: the same two vectors per thread on 512 threads
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 2, 512>), grid, dim3(512), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
             PARAS_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + 7) / 8)), dim3(kBlock), 0, s,
                                part, static_cast<S*>(gw), slabs, H);

@@ -142,10 +142,10 @@ def test_full_size_rms_norm_and_swiglu_bf16():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("shape", [(70, 4096), (33, 2048), (16, 520), (300, 1024), (5, 8)])
+@pytest.mark.parametrize("shape", [(70, 4096), (33, 2048), (16, 520), (300, 1024), (5, 8), (37, 8192), (20, 5120), (9, 8200)])
 def test_rms_norm_backward_one_pass_kernel(shape, dtype):
-    """Row sizes the one-pass backward kernel takes (16-byte aligned rows of up to 4096 elements),
-    with slabs of rows that are full, ragged and single."""
+    """Row sizes the one-pass backward kernel takes (16-byte aligned rows of up to 8192 elements; the
+    last shape is beyond it), with slabs of rows that are full, ragged and single."""
     rows, H = shape
     torch.manual_seed(rows + H)
     x, w, go = torch.randn(rows, H).to(dtype), (1 + 0.1 * torch.randn(H)).to(dtype), torch.randn(rows, H).to(dtype)
