@@ -105,8 +105,8 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
 
 // ---- few rows (M <= 128): the decode-time projections.  The product is bound by streaming the
 // weights once, so there is no tile and no LDS staging: a workgroup owns 16 weight rows, its eight
-// waves split the contraction (k-steps of 32 dealt round-robin, so the eight read adjacent 64-byte
-// pieces of each row), every wave feeds v_mfma_f32_16x16x32 straight from global memory (weights
+// waves split the contraction (pieces of 64 dealt round-robin, so the eight read adjacent 128-byte
+// lines of each row), every wave feeds v_mfma_f32_16x16x32 straight from global memory (weights
 // as the row operand, non-temporal; the few activation rows from L2), and the eight partial
 // results meet in LDS in wave order.  Lane l of a 16x16 result holds activation row l%16 and
 // weight rows 4*(l/16) .. +3: four adjacent outputs, stored as one 8-byte piece when aligned.
@@ -140,50 +140,62 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const
     for (int nb = 0; nb < NB; ++nb) {
         long wrow = n0 + nb * 16 + r16;
         if (wrow >= p.N) wrow = p.N - 1;                    // clamped rows are computed but never stored
-        wp[nb] = B + wrow * p.ldb + kg * 8;
+        wp[nb] = B + wrow * p.ldb + kg * 16;
     }
     const std::uint16_t* xp[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         long xrow = mb * 16 + r16;
         if (xrow >= p.M) xrow = p.M - 1;
-        xp[mb] = A + xrow * p.lda + kg * 8;
+        xp[mb] = A + xrow * p.lda + kg * 16;
     }
     float4_t acc[NB][MB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
-    const long ksteps = p.K / 32;
-    // A batch of k-steps: every load of the batch is requested before its first MFMA, so a wave
-    // pays the memory latency once per batch.
-    constexpr int kUnroll = MB <= 4 ? 4 : 2;
-    long ks = wave;
-    for (; ks + (kUnroll - 1) * kSkinnyWaves < ksteps; ks += kUnroll * kSkinnyWaves) {
-        u32x4 wv[kUnroll][NB], xv[kUnroll][MB];
+    // The contraction is walked in pieces of 64 (two MFMAs): lane group kg supplies elements
+    // 16 kg .. 16 kg + 7 of a piece to the first MFMA and the next eight to the second -- any
+    // assignment works as long as both operands use the same one -- so that the four groups
+    // together read whole 128-byte lines of a row.  A batch is kPieces pieces: every load of the
+    // batch is requested before its first MFMA, so a wave pays the memory latency once per batch.
+    const long pieces = p.K / 64;
+    constexpr int kPieces = MB <= 4 ? 2 : 1;
+    long pc = wave;
+    for (; pc + (kPieces - 1) * kSkinnyWaves < pieces; pc += kPieces * kSkinnyWaves) {
+        u32x4 wv[kPieces][2][NB], xv[kPieces][2][MB];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
+        for (int u = 0; u < kPieces; ++u)
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) wv[u][nb] = load16_nt(wp[nb] + (ks + u * kSkinnyWaves) * 32);
+            for (int h = 0; h < 2; ++h) {
+                const long k = (pc + u * kSkinnyWaves) * 64 + h * 8;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) xv[u][mb] = load16(xp[mb] + (ks + u * kSkinnyWaves) * 32);
-        }
+                for (int nb = 0; nb < NB; ++nb) wv[u][h][nb] = load16_nt(wp[nb] + k);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+                for (int mb = 0; mb < MB; ++mb) xv[u][h][mb] = load16(xp[mb] + k);
+            }
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+        for (int u = 0; u < kPieces; ++u)
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[u][nb], xv[u][mb], acc[nb][mb]);
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[u][h][nb], xv[u][h][mb], acc[nb][mb]);
     }
-    for (; ks < ksteps; ks += kSkinnyWaves) {
-        u32x4 wv[NB];
+    for (; pc < pieces; pc += kSkinnyWaves) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) wv[nb] = load16_nt(wp[nb] + ks * 32);
+        for (int h = 0; h < 2; ++h) {
+            const long k = pc * 64 + h * 8;
+            u32x4 wv[NB];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            const u32x4 xv = load16(xp[mb] + ks * 32);
+            for (int nb = 0; nb < NB; ++nb) wv[nb] = load16_nt(wp[nb] + k);
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[nb], xv, acc[nb][mb]);
+            for (int mb = 0; mb < MB; ++mb) {
+                const u32x4 xv = load16(xp[mb] + k);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[nb], xv, acc[nb][mb]);
+            }
         }
     }
 #pragma unroll
