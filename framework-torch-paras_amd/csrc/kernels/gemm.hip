@@ -107,7 +107,8 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
 // weights once, so there is no tile and no LDS staging: a workgroup owns 16 weight rows, its eight
 // waves split the contraction (pieces of 64 dealt round-robin, so the eight read adjacent 128-byte
 // lines of each row), every wave feeds v_mfma_f32_16x16x32 straight from global memory (weights
-// as the row operand, non-temporal; the few activation rows from L2), and the eight partial
+// as the row operand, with plain loads: non-temporal ones measured 5-18 % slower here, each
+// 128-byte line being touched by two instructions; the few activation rows from L2), and the eight partial
 // results meet in LDS in wave order.  Lane l of a 16x16 result holds activation row l%16 and
 // weight rows 4*(l/16) .. +3: four adjacent outputs, stored as one 8-byte piece when aligned.
 template <typename T> struct Mma16;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const
             for (int h = 0; h < 2; ++h) {
                 const long k = (pc + u * kSkinnyWaves) * 64 + h * 8;
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) wv[u][h][nb] = load16_nt(wp[nb] + k);
+                for (int nb = 0; nb < NB; ++nb) wv[u][h][nb] = load16(wp[nb] + k);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) xv[u][h][mb] = load16(xp[mb] + k);
             }
@@ -189,7 +190,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const
             const long k = pc * 64 + h * 8;
             u32x4 wv[NB];
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) wv[nb] = load16_nt(wp[nb] + k);
+            for (int nb = 0; nb < NB; ++nb) wv[nb] = load16(wp[nb] + k);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const u32x4 xv = load16(xp[mb] + k);
@@ -255,6 +256,144 @@ void launch_skinny(const DenseParams& p, long batch, hipStream_t s) {
                         else     hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 4, 1>), g1, block, 0, s, p); }
     else              { if (two) hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 8, 2>), g2, block, 0, s, p);
                         else     hipLaunchKernelGGL((skinny_gemm_nt_kernel<T, 8, 1>), g1, block, 0, s, p); }
+}
+
+// ---- few rows with a workspace: the same product with the activations read once per 128 weight
+// rows instead of once per 16.  In the kernel above every workgroup re-reads all M x K activations
+// from L2, which -- not the weights -- bounds it from M = 32 upwards.  Here the eight waves of a
+// workgroup own eight blocks of 16 weight rows and walk the SAME part of the contraction, so a slab
+// of activations (M rows x 256 elements) is brought into LDS once and shared; the contraction is
+// split over workgroups instead (grid.x), each writes its fp32 partial result to the workspace, and
+// a second kernel adds the partials in split order and applies the epilogue: deterministic, and
+// 128 / 16 = 8 times fewer activation reads for a workspace of splits x M x N floats.
+constexpr int kSlab = 256;                 // contraction elements per LDS slab (4 pieces of 64)
+constexpr int kSlabLd = kSlab + 8;         // LDS row stride (elements): 16 consecutive rows hit distinct banks
+
+template <typename T, int MB>
+__global__ __launch_bounds__(512) void skinny_splitk_kernel(const DenseParams p, float* __restrict__ partial, int pieces_per_split) {
+    __shared__ __attribute__((aligned(16))) std::uint16_t xs[2][MB * 16 * kSlabLd];
+    const long bidx = blockIdx.z;
+    const std::uint16_t* A = p.a + bidx * p.sa;
+    const std::uint16_t* B = p.b + bidx * p.sb;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, kg = lane >> 4;
+    // grid.x = split, grid.y = block of 128 weight rows: workgroups that run together read adjacent
+    // parts of the same weight rows
+    const long n0 = static_cast<long>(blockIdx.y) * 128 + wave * 16;
+    long wrow = n0 + r16;
+    if (wrow >= p.N) wrow = p.N - 1;                        // clamped rows are computed but never stored
+    const std::uint16_t* wp = B + wrow * p.ldb + kg * 16;
+    const long pieces = p.K / 64;
+    const long pc0 = static_cast<long>(blockIdx.x) * pieces_per_split;
+    const long pc1 = pc0 + pieces_per_split < pieces ? pc0 + pieces_per_split : pieces;
+    // staging of a slab: MB*16 rows x 32 chunks of 16 bytes, 512 threads -> MB chunks per thread
+    u32x4 stage[MB];
+    auto load_slab = [&](long pc) {                         // pieces pc .. pc+3 (clamped to the split's end)
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+            const int c = tid + i * 512;
+            long row = c >> 5;
+            const long k = pc * 64 + (c & 31) * 8;
+            if (row >= p.M) row = p.M - 1;
+            stage[i] = k < pc1 * 64 ? load16(A + row * p.lda + k) : u32x4{0, 0, 0, 0};
+        }
+    };
+    auto store_slab = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+            const int c = tid + i * 512;
+            *reinterpret_cast<u32x4*>(&xs[buf][(c >> 5) * kSlabLd + (c & 31) * 8]) = stage[i];
+        }
+    };
+    float4_t acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    // Weights and activations of slab s+1 are requested before the MFMAs of slab s, so that two
+    // slabs' worth of loads are in flight per wave and a split of two slabs pays the memory latency
+    // about once.
+    u32x4 wv[4][2], wn[4][2];
+    auto load_w = [&](long pc, u32x4 (&dst)[4][2]) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                dst[u][h] = pc + u < pc1 ? load16(wp + (pc + u) * 64 + h * 8) : u32x4{0, 0, 0, 0};
+    };
+    if (pc0 < pc1) {
+        load_slab(pc0);
+        load_w(pc0, wv);
+        store_slab(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (long pc = pc0; pc < pc1; pc += 4, buf ^= 1) {
+        const bool more = pc + 4 < pc1;
+        if (more) {
+            load_slab(pc + 4);
+            load_w(pc + 4, wn);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const u32x4 xv = *reinterpret_cast<const u32x4*>(&xs[buf][(mb * 16 + r16) * kSlabLd + u * 64 + kg * 16 + h * 8]);
+                    acc[mb] = Mma16<T>::run(wv[u][h], xv, acc[mb]);
+                }
+        if (more) {
+            store_slab(buf ^ 1);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) wv[u][h] = wn[u][h];
+        }
+        __syncthreads();
+    }
+    // partial[(batch, split)][row][col]: lane holds row mb*16 + r16, columns n0 + 4 kg .. + 3
+    float* dst = partial + (bidx * gridDim.x + blockIdx.x) * (p.M * p.N);
+    const long col = n0 + 4 * kg;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const long row = mb * 16 + r16;
+        if (row >= p.M) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (col + r < p.N) dst[row * p.N + col + r] = acc[mb][r];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void skinny_splitk_finish_kernel(const DenseParams p, const float* __restrict__ partial, int splits) {
+    using El = Elem<T>;
+    const long mn = p.M * p.N;
+    const long i = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= mn) return;
+    const long bidx = blockIdx.y;
+    const float* src = partial + bidx * splits * mn + i;
+    float t = 0.f;
+    for (int sp = 0; sp < splits; ++sp) t += src[sp * mn];
+    const long row = i / p.N, col = i % p.N;
+    float v = p.alpha * t;
+    if (p.add) v = fmaf(p.beta, El::to_f32((p.add + bidx * p.sadd)[row * p.ld_add + col]), v);
+    (p.c + bidx * p.sc)[row * p.ldc + col] = El::from_f32(v);
+}
+
+// Splits of the contraction for the workspace kernel (0 = it does not apply): enough workgroups to
+// fill the chip twice, at least two slabs each.
+int splitk_plan(long M, long N, long K, long batch, int* pieces_per_split) {
+    if (M < 32 || M > kSkinnyMaxM || K % 64 != 0 || N < 512) return 0;   // up to 16 rows the activations are no load
+    const long pieces = K / 64;
+    const long groups = (N + 127) / 128 * batch;
+    long splits = (512 + groups - 1) / groups;
+    if (splits > pieces / 8) splits = pieces / 8;
+    if (splits < 2) return 0;
+    long per = (pieces + splits - 1) / splits;
+    per = (per + 3) / 4 * 4;                                  // whole slabs
+    splits = (pieces + per - 1) / per;
+    if (splits < 2 || (N + 127) / 128 > 65535) return 0;
+    *pieces_per_split = static_cast<int>(per);
+    return static_cast<int>(splits);
 }
 
 // ---- any float dtype, any contraction size, any alignment: the product for what the MFMA kernels
@@ -353,10 +492,26 @@ void launch_dense(const DenseParams& p, unsigned grid, hipStream_t s) {
 
 extern "C" {
 
+size_t paras_gemm_nt_workspace(int64_t M, int64_t N, int64_t K, int64_t batch, int dtype) {
+    using namespace paras;
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || (dtype != PARAS_BF16 && dtype != PARAS_F16)) return 0;
+    int per = 0;
+    const int splits = splitk_plan(M, N, K, batch, &per);
+    return static_cast<size_t>(splits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+}
+
 int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int64_t M, int64_t N, int64_t K,
                   int64_t lda, int64_t ldb, int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
                   int64_t stride_b, int64_t stride_c, int64_t stride_add, double alpha, double beta, int dtype,
                   void* stream) {
+    return paras_gemm_nt_ws(a, b, addend, c, M, N, K, lda, ldb, ldc, ld_add, batch, stride_a, stride_b, stride_c, stride_add,
+                            alpha, beta, dtype, nullptr, 0, stream);
+}
+
+int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, int64_t M, int64_t N, int64_t K,
+                     int64_t lda, int64_t ldb, int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
+                     int64_t stride_b, int64_t stride_c, int64_t stride_add, double alpha, double beta, int dtype,
+                     void* workspace, size_t workspace_bytes, void* stream) {
     using namespace paras;
     PARAS_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "paras_gemm_nt: negative shape");
     if (M == 0 || N == 0 || batch == 0) return PARAS_OK;
@@ -403,6 +558,29 @@ int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c, int
     if (use_square) n_units = (N + gemm::kBN - 1) / gemm::kBN;
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
     p.m_tiles = static_cast<int>(m_tiles); p.n_units = static_cast<int>(n_units);
+    if (workspace != nullptr && batch <= 65535) {
+        int per = 0;
+        const int splits = splitk_plan(M, N, K, batch, &per);
+        const size_t need = static_cast<size_t>(splits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+        if (splits >= 2 && workspace_bytes >= need && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+            const dim3 grid(static_cast<unsigned>(splits), static_cast<unsigned>((N + 127) / 128), static_cast<unsigned>(batch));
+            const int mb = static_cast<int>((M + 15) / 16);
+            float* part = static_cast<float*>(workspace);
+            const bool bf = dtype == PARAS_BF16;
+            if (mb <= 2)      { if (bf) hipLaunchKernelGGL((skinny_splitk_kernel<bf16_t, 2>), grid, dim3(512), 0, s, p, part, per);
+                                else    hipLaunchKernelGGL((skinny_splitk_kernel<f16_t, 2>), grid, dim3(512), 0, s, p, part, per); }
+            else if (mb <= 4) { if (bf) hipLaunchKernelGGL((skinny_splitk_kernel<bf16_t, 4>), grid, dim3(512), 0, s, p, part, per);
+                                else    hipLaunchKernelGGL((skinny_splitk_kernel<f16_t, 4>), grid, dim3(512), 0, s, p, part, per); }
+            else              { if (bf) hipLaunchKernelGGL((skinny_splitk_kernel<bf16_t, 8>), grid, dim3(512), 0, s, p, part, per);
+                                else    hipLaunchKernelGGL((skinny_splitk_kernel<f16_t, 8>), grid, dim3(512), 0, s, p, part, per); }
+            PARAS_HIP_TRY(hipGetLastError());
+            const dim3 fgrid(static_cast<unsigned>((M * N + 255) / 256), static_cast<unsigned>(batch));
+            if (bf) hipLaunchKernelGGL((skinny_splitk_finish_kernel<bf16_t>), fgrid, dim3(256), 0, s, p, part, splits);
+            else    hipLaunchKernelGGL((skinny_splitk_finish_kernel<f16_t>), fgrid, dim3(256), 0, s, p, part, splits);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
+    }
     if (M <= kSkinnyMaxM && batch <= 65535 && (N + 15) / 16 <= 0x7fffffffLL) {
         if (dtype == PARAS_BF16) launch_skinny<bf16_t>(p, batch, s);
         else                     launch_skinny<f16_t>(p, batch, s);

@@ -60,9 +60,14 @@ Tensor run_gemm(const Tensor& a_in, const Tensor& mat2, const c10::optional<Tens
         ld_add = add.stride(-2);
     }
     const int64_t nb = batch > 0 ? batch : 1;
-    check(paras_gemm_nt(a.data_ptr(), bt.data_ptr(), add_ptr, out.data_ptr(), M, N, K, a.stride(-2), bt.stride(-2), N, ld_add,
-                        nb, batch > 0 ? a.stride(0) : 0, batch > 0 ? bt.stride(0) : 0, M * N, s_add, alpha, beta,
-                        require_float_code(a, "paras gemm"), stream_for(a)));
+    const int code = require_float_code(a, "paras gemm");
+    // few-row products (decode-time projections) run faster with a workspace for split partial sums
+    const size_t ws_bytes = paras_gemm_nt_workspace(M, N, K, nb, code);
+    Tensor ws;
+    if (ws_bytes > 0) ws = at::empty({static_cast<int64_t>(ws_bytes)}, a.options().dtype(c10::kByte));
+    check(paras_gemm_nt_ws(a.data_ptr(), bt.data_ptr(), add_ptr, out.data_ptr(), M, N, K, a.stride(-2), bt.stride(-2), N, ld_add,
+                           nb, batch > 0 ? a.stride(0) : 0, batch > 0 ? bt.stride(0) : 0, M * N, s_add, alpha, beta, code,
+                           ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, stream_for(a)));
     return out;
 }
 

@@ -290,6 +290,21 @@ PARAS_API int paras_gemm_nt(const void* a, const void* b, const void* addend, vo
                             int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
                             int64_t stride_b, int64_t stride_c, int64_t stride_add,
                             double alpha, double beta, int dtype, void* stream);
+/* The same product with a caller-provided workspace of                        */
+/* paras_gemm_nt_workspace(M, N, K, batch, dtype) bytes (0 for shapes that     */
+/* need none; 16-byte aligned).  With it, bf16 / f16 products of 32 to 128     */
+/* rows (decode-time projections) split the contraction over workgroups and    */
+/* read the activations once per 128 weight rows; the partial sums are added   */
+/* in a fixed order.  Without it (NULL) the call is paras_gemm_nt.  (Same      */
+/* reference lines as above.)                                                  */
+PARAS_API size_t paras_gemm_nt_workspace(int64_t M, int64_t N, int64_t K, int64_t batch,
+                                         int dtype);
+PARAS_API int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c,
+                               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                               int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
+                               int64_t stride_b, int64_t stride_c, int64_t stride_add,
+                               double alpha, double beta, int dtype, void* workspace,
+                               size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Row softmax and row top-k (replace softmax_out / topk_out,                  */

@@ -63,6 +63,8 @@ SIGNATURES = {
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
     "paras_gemm_nt": (i32, [vp, vp, vp, vp] + [i64] * 12 + [f64, f64, i32, vp]),
+    "paras_gemm_nt_workspace": (sz, [i64, i64, i64, i64, i32]),
+    "paras_gemm_nt_ws": (i32, [vp, vp, vp, vp] + [i64] * 12 + [f64, f64, i32, vp, sz, vp]),
     "paras_softmax_rows": (i32, [vp, vp, i64, i64, i32, i32, vp]),
     "paras_topk_rows": (i32, [vp, vp, vp, i64, i64, i64, i32, i32, vp]),
 }
@@ -223,9 +225,10 @@ def moe_ffn(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, k, workspa
     return out
 
 
-def gemm_nt(a, b, addend=None, alpha=1.0, beta=1.0):
+def gemm_nt(a, b, addend=None, alpha=1.0, beta=1.0, workspace=False):
     """C = alpha * a @ b^T (+ beta * addend); a [.., M, K], b [.., N, K] (2-D or batched 3-D,
-    last dim contiguous); addend [N] (bias), [M, N] or [B, M, N]."""
+    last dim contiguous); addend [N] (bias), [M, N] or [B, M, N].  workspace=True hands the
+    library the workspace it asks for (paras_gemm_nt_ws)."""
     batched = a.dim() == 3
     B = a.shape[0] if batched else 1
     M, K = a.shape[-2:]
@@ -239,6 +242,13 @@ def gemm_nt(a, b, addend=None, alpha=1.0, beta=1.0):
             ld_add = addend.stride(-2)
         if addend.dim() == 3:
             sadd = addend.stride(0)
+    if workspace:
+        nbytes = lib().paras_gemm_nt_workspace(M, N, K, B, DT[a.dtype])
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=a.device)
+        check(lib().paras_gemm_nt_ws(_ptr(a), _ptr(b), _ptr(addend) if addend is not None else None, _ptr(c), M, N, K,
+                                     a.stride(-2), b.stride(-2), N, ld_add, B, sa, sb, M * N, sadd, alpha, beta,
+                                     DT[a.dtype], _ptr(ws), nbytes, _stream()))
+        return c
     check(lib().paras_gemm_nt(_ptr(a), _ptr(b), _ptr(addend) if addend is not None else None, _ptr(c), M, N, K,
                               a.stride(-2), b.stride(-2), N, ld_add, B, sa, sb, M * N, sadd, alpha, beta,
                               DT[a.dtype], _stream()))

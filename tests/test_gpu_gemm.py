@@ -194,3 +194,43 @@ def test_gemm_nt_few_rows_batched():
     shared = capi.gemm_nt(a, b[0])                      # one weight matrix for the whole batch
     for i in range(6):
         assert torch.equal(shared[i], capi.gemm_nt(a[i], b[0]))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(32, 4096, 4096), (64, 4096, 1024), (64, 1027, 4096), (100, 1536, 2048), (128, 2050, 4096),
+                                   (33, 640, 1088)])
+def test_gemm_nt_few_rows_with_workspace(shape, dtype):
+    """32 to 128 rows with the workspace the library asks for: the contraction is split over
+    workgroups and the partial sums are added in a fixed order -- same bar as every other GEMM
+    kernel, same result on every call, with bias / scaled addend and ragged N and K splits."""
+    M, N, K = shape
+    torch.manual_seed(M + N + K)
+    a = torch.randn(M, K).to(dtype)
+    b = (torch.randn(N, K) / math.sqrt(K)).to(dtype)
+    assert capi.lib().paras_gemm_nt_workspace(M, N, K, 1, capi.DT[dtype]) > 0
+    got = capi.gemm_nt(a.cuda(), b.cuda(), workspace=True)
+    assert_gemm_close(got, O.matmul_nt(a, b), dtype)
+    assert torch.equal(got, capi.gemm_nt(a.cuda(), b.cuda(), workspace=True))          # deterministic
+    bias = torch.randn(N).to(dtype)
+    got = capi.gemm_nt(a.cuda(), b.cuda(), bias.cuda(), alpha=1.0, beta=1.0, workspace=True)
+    assert_gemm_close(got, torch.nn.functional.linear(a, b, bias), dtype)
+    addm = torch.randn(M, N).to(dtype)
+    got = capi.gemm_nt(a.cuda(), b.cuda(), addm.cuda(), alpha=0.5, beta=2.0, workspace=True)
+    want = torch.addmm(addm.float(), a.float(), b.float().t(), beta=2.0, alpha=0.5)
+    assert bool(((got.float().cpu() - want).abs() <= 2 * ulp16(want, dtype) + 1e-6).all())
+
+
+def test_gemm_nt_workspace_batched_and_shapes_that_need_none():
+    torch.manual_seed(6)
+    a = torch.randn(3, 48, 1024, device="cuda").bfloat16()
+    b = (0.05 * torch.randn(3, 768, 1024, device="cuda")).bfloat16()
+    out = capi.gemm_nt(a, b, workspace=True)
+    for i in range(3):
+        assert_gemm_close(out[i], O.matmul_nt(a[i].cpu(), b[i].cpu()), torch.bfloat16)
+    L = capi.lib()
+    assert L.paras_gemm_nt_workspace(8, 4096, 4096, 1, capi.BF16) == 0        # up to 16 rows: nothing to share
+    assert L.paras_gemm_nt_workspace(4096, 4096, 4096, 1, capi.BF16) == 0     # tile kernels
+    assert L.paras_gemm_nt_workspace(64, 4096, 4096, 1, capi.F32) == 0        # general kernel
+    x = torch.randn(8, 256, device="cuda").bfloat16()
+    w = torch.randn(64, 256, device="cuda").bfloat16()
+    assert torch.equal(capi.gemm_nt(x, w, workspace=True), capi.gemm_nt(x, w))
