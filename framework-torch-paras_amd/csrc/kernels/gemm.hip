@@ -162,14 +162,23 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const
     // batch is requested before its first MFMA, so a wave pays the memory latency once per batch.
     const long pieces = p.K / 64;
     constexpr int kPieces = MB <= 4 ? 2 : 1;
-    long pc = wave;
-    for (; pc + (kPieces - 1) * kSkinnyWaves < pieces; pc += kPieces * kSkinnyWaves) {
+    // this wave's pieces are wave, wave + W, ...; each workgroup starts at a different one of them and
+    // wraps around, so that the workgroups do not all read the same part of every weight row at once
+    const long mine = pieces > wave ? (pieces - wave + kSkinnyWaves - 1) / kSkinnyWaves : 0;
+    const long first = mine > 0 ? (static_cast<long>(blockIdx.x) * 3) % mine : 0;
+    auto piece_at = [&](long t) {
+        long r = t + first;
+        if (r >= mine) r -= mine;
+        return (wave + r * kSkinnyWaves) * 64;
+    };
+    long t = 0;
+    for (; t + kPieces <= mine; t += kPieces) {
         u32x4 wv[kPieces][2][NB], xv[kPieces][2][MB];
 #pragma unroll
         for (int u = 0; u < kPieces; ++u)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const long k = (pc + u * kSkinnyWaves) * 64 + h * 8;
+                const long k = piece_at(t + u) + h * 8;
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) wv[u][h][nb] = load16(wp[nb] + k);
 #pragma unroll
@@ -184,10 +193,10 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16<T>::run(wv[u][h][nb], xv[u][h][mb], acc[nb][mb]);
     }
-    for (; pc < pieces; pc += kSkinnyWaves) {
+    for (; t < mine; ++t) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const long k = pc * 64 + h * 8;
+            const long k = piece_at(t) + h * 8;
             u32x4 wv[NB];
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) wv[nb] = load16(wp[nb] + k);
