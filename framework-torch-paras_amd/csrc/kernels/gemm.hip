@@ -328,18 +328,28 @@ __global__ __launch_bounds__(512) void skinny_splitk_kernel(const DenseParams p,
             for (int h = 0; h < 2; ++h)
                 dst[u][h] = pc + u < pc1 ? load16(wp + (pc + u) * 64 + h * 8) : u32x4{0, 0, 0, 0};
     };
-    if (pc0 < pc1) {
-        load_slab(pc0);
-        load_w(pc0, wv);
+    // The slabs of the split are walked from a different starting slab in every block of weight rows
+    // (and wrap around), so that the workgroups of one split do not read the same part of their rows
+    // at the same time.
+    const long nslabs = pc1 > pc0 ? (pc1 - pc0 + 3) / 4 : 0;
+    const long rot = nslabs > 0 ? static_cast<long>(blockIdx.y) % nslabs : 0;
+    auto slab_pc = [&](long i) {
+        long r = i + rot;
+        if (r >= nslabs) r -= nslabs;
+        return pc0 + 4 * r;
+    };
+    if (nslabs > 0) {
+        load_slab(slab_pc(0));
+        load_w(slab_pc(0), wv);
         store_slab(0);
     }
     __syncthreads();
     int buf = 0;
-    for (long pc = pc0; pc < pc1; pc += 4, buf ^= 1) {
-        const bool more = pc + 4 < pc1;
+    for (long i = 0; i < nslabs; ++i, buf ^= 1) {
+        const bool more = i + 1 < nslabs;
         if (more) {
-            load_slab(pc + 4);
-            load_w(pc + 4, wn);
+            load_slab(slab_pc(i + 1));
+            load_w(slab_pc(i + 1), wn);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
