@@ -50,6 +50,10 @@ struct DecodeParams {
     int B, Hq, Hkv, Lq, Lk, G, R;
     int splits, chunk;  // keys per workgroup
     float scale_log2, scale;
+    // optional mask (element strides; 0 = broadcast): bytes that are zero / non-zero, or additive values of the tensor dtype
+    const unsigned char* mask;
+    long ms_b, ms_h, ms_q, ms_k;
+    float inv_scale;    // the scores are kept unscaled: an additive mask value m enters as m / scale
 };
 
 template <typename T> struct Mma16;
@@ -86,7 +90,8 @@ __device__ __forceinline__ float group_sum(float x) {
     return x + __shfl_xor(x, 32, kWave);
 }
 
-template <typename T>
+// kMask: 0 = none, 1 = bool (true = attend), 2 = additive values of dtype T
+template <typename T, int kMask>
 __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeParams p) {
     // Per-wave V tiles (double buffered); reused as fp32 merge space at the end.
     __shared__ __attribute__((aligned(16))) std::uint16_t v_lds[kWaves][2][kTile * kVS];
@@ -108,6 +113,14 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
             i16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
             qreg[ks] = live ? *reinterpret_cast<const i16x8*>(qp + 32 * ks + 8 * lg) : z;
         }
+    }
+
+    // ---- this lane's mask row (query row lq): the 8 keys it scores per tile are 4 lg .. 4 lg + 3 of each 16-key block
+    const unsigned char* mrow = nullptr;
+    if constexpr (kMask != 0) {
+        const bool live = lq < p.R;
+        const int gi = live ? lq / p.Lq : 0, qi = live ? lq % p.Lq : 0;
+        mrow = p.mask + (static_cast<long>(b) * p.ms_b + static_cast<long>(hkv * p.G + gi) * p.ms_h + static_cast<long>(qi) * p.ms_q) * (kMask == 1 ? 1 : 2);
     }
 
     // ---- this wave's key range
@@ -179,6 +192,21 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
             for (int ks = 0; ks < 4; ++ks) sacc[kb] = Mma16<T>::run(kcur[kb][ks], qreg[ks], sacc[kb]);
         }
         const int key0 = k_begin + t * kTile;
+        if constexpr (kMask != 0) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int key = key0 + kb * 16 + 4 * lg + r;
+                    key = key < p.Lk ? key : p.Lk - 1;                       // keys past the end are masked below anyway
+                    if constexpr (kMask == 1) {
+                        if (mrow[static_cast<long>(key) * p.ms_k] == 0) sacc[kb][r] = -INFINITY;
+                    } else {
+                        const std::uint16_t bits = *reinterpret_cast<const std::uint16_t*>(mrow + static_cast<long>(key) * p.ms_k * 2);
+                        sacc[kb][r] = fmaf(Elem<T>::to_f32(bits), p.inv_scale, sacc[kb][r]);
+                    }
+                }
+        }
         if (key0 + kTile > k_end) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
@@ -190,8 +218,10 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
                            fmaxf(fmaxf(sacc[1][0], sacc[1][1]), fmaxf(sacc[1][2], sacc[1][3])));
         mloc = group_max(mloc);
         const float m_new = fmaxf(m_run, mloc);
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2);
-        const float mc = m_new * p.scale_log2;
+        // (with a mask every key so far may be masked out: -inf on both sides keeps the zeros, and the
+        // reference point of the exponentials must not be -inf)
+        const float alpha = m_run == m_new ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2);
+        const float mc = m_new == -INFINITY ? 0.f : m_new * p.scale_log2;
         m_run = m_new;
         float lsum = 0.f;
 #pragma unroll
@@ -327,7 +357,8 @@ void plan(const paras_sdpa_args& a, int* splits, int* chunk) {
 bool decode_supported(const paras_sdpa_args& a) {
     if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
     if (a.D != kD || a.Dv != kD) return false;
-    if (a.mask_kind != 0 || a.attn != nullptr || a.is_causal) return false;
+    if (a.attn != nullptr || a.is_causal) return false;
+    if (a.mask_kind != 0 && (a.mask == nullptr || a.mask_kind > 2)) return false;
     if (a.Hkv < 1 || a.Hq % a.Hkv != 0) return false;
     const int64_t rows = a.Lq * (a.Hq / a.Hkv);
     if (rows < 1 || rows > kMaxRows) return false;
@@ -366,9 +397,21 @@ int launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s) {
     p.part_o = static_cast<float*>(workspace);
     p.part_ml = p.part_o ? p.part_o + slots * kMaxRows * kD : nullptr;
     const dim3 grid(p.splits, static_cast<unsigned>(a.B * a.Hkv));
+    p.mask = static_cast<const unsigned char*>(a.mask);
+    p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2]; p.ms_k = a.mask_strides[3];
+    p.inv_scale = static_cast<float>(1.0 / a.scale);
     const bool bf = a.dtype == PARAS_BF16;
-    if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t>), grid, dim3(kThreads), 0, s, p);
-    else    hipLaunchKernelGGL((decode_split_kernel<f16_t>), grid, dim3(kThreads), 0, s, p);
+    const dim3 block(kThreads);
+    if (a.mask_kind == 0) {
+        if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t, 0>), grid, block, 0, s, p);
+        else    hipLaunchKernelGGL((decode_split_kernel<f16_t, 0>), grid, block, 0, s, p);
+    } else if (a.mask_kind == 1) {
+        if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t, 1>), grid, block, 0, s, p);
+        else    hipLaunchKernelGGL((decode_split_kernel<f16_t, 1>), grid, block, 0, s, p);
+    } else {
+        if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t, 2>), grid, block, 0, s, p);
+        else    hipLaunchKernelGGL((decode_split_kernel<f16_t, 2>), grid, block, 0, s, p);
+    }
     PARAS_HIP_TRY(hipGetLastError());
     if (p.splits > 1) {
         const dim3 g2(static_cast<unsigned>(a.B * a.Hkv), p.R);

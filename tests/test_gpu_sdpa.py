@@ -302,6 +302,42 @@ def test_decode_matches_oracle(dtype, shape):
     assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=1e-3, atol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decode_with_masks_matches_oracle(dtype):
+    """Ragged batches: decode with a key-padding mask [B,1,1,Lk], a per-head additive bias
+    [B,Hq,1,Lk], a [Lq,Lk] mask for two query positions, a sequence whose first 3000 keys are all
+    masked (whole tiles, whole waves and whole splits without a visible key) and one with no visible
+    key at all (NaN, as the reference's softmax gives)."""
+    torch.manual_seed(31)
+    B, Hq, Hkv, Lk = 3, 8, 2, 4000
+    q, k, v = torch.randn(B, Hq, 1, 128).to(dtype), torch.randn(B, Hkv, Lk, 128).to(dtype), torch.randn(B, Hkv, Lk, 128).to(dtype)
+    lengths = [4000, 1234, 77]
+    keep = torch.zeros(B, 1, 1, Lk, dtype=torch.bool)
+    for i, n in enumerate(lengths):
+        keep[i, ..., :n] = True
+    out, _, _, kern = run(q, k, v, mask=keep)
+    want, _ = O.sdpa_math(q, k, v, attn_mask=keep, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split" and max_abs(out, want) <= ABS_16BIT
+    bias = (2 * torch.randn(B, Hq, 1, Lk)).masked_fill(~keep, -math.inf).to(dtype)
+    out, _, _, kern = run(q, k, v, mask=bias)
+    want, _ = O.sdpa_math(q, k, v, attn_mask=bias, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split" and max_abs(out, want) <= 2 * ABS_16BIT
+    q2 = torch.randn(B, Hq, 2, 128).to(dtype)
+    m2 = torch.rand(2, Lk) > 0.5
+    m2[:, 0] = True
+    out, _, _, kern = run(q2, k, v, mask=m2)
+    want, _ = O.sdpa_math(q2, k, v, attn_mask=m2, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split" and max_abs(out, want) <= ABS_16BIT
+    late = torch.ones(B, 1, 1, Lk, dtype=torch.bool)
+    late[0, ..., :3000] = False
+    late[1] = False
+    out, _, _, kern = run(q, k, v, mask=late)
+    want, _ = O.sdpa_math(q, k, v, attn_mask=late, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split"
+    assert bool(out[1].isnan().all()) and bool(want[1].isnan().all())
+    assert max_abs(out[[0, 2]], want[[0, 2]]) <= ABS_16BIT
+
+
 def test_generic_handles_odd_heads_masks_and_all_masked_rows():
     q, k, v = torch.randn(1, 3, 5, 24), torch.randn(1, 3, 9, 24), torch.randn(1, 3, 9, 40)
     out, attn, _, kern = run(q, k, v, want_attn=True)                # Dv != D
