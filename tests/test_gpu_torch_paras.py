@@ -485,3 +485,44 @@ print("done")
     covered = ("scaled_dot_product", "rms_norm", "swiglu", "linear", "mm", "softmax", "topk")
     bad = [op for op in fell if any(c in op for c in covered)]
     assert not bad, f"covered ops went through the host fallback: {bad} (all fallbacks: {fell})"
+
+
+def test_llama_block_forward_matches_cpu(device):
+    """One decoder block assembled from the ops of this build (RMSNorm, QKV / output / MLP projections,
+    RoPE through rotate_half, causal GQA attention, SwiGLU), the glue (elementwise arithmetic,
+    reshapes) going wherever the dispatcher sends it: the same code on `paras:0` and on the CPU."""
+    from torch_paras import nn as paras_nn
+    torch.manual_seed(11)
+    B, S, Hd, nh, nkv, hd, I = 2, 96, 256, 4, 2, 64, 512
+    dt = torch.bfloat16
+    W = {n: (torch.randn(*shp) * 0.05).to(dt) for n, shp in
+         dict(q=(nh * hd, Hd), k=(nkv * hd, Hd), v=(nkv * hd, Hd), o=(Hd, nh * hd), g=(I, Hd), u=(I, Hd), d=(Hd, I)).items()}
+    n1, n2 = (1 + 0.1 * torch.randn(Hd)).to(dt), (1 + 0.1 * torch.randn(Hd)).to(dt)
+    x = torch.randn(B, S, Hd).to(dt)
+    pos = torch.arange(S, dtype=torch.float32)
+    inv = 1.0 / (10000 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    ang = torch.cat([pos[:, None] * inv[None, :]] * 2, -1)
+    cos, sin = ang.cos().to(dt), ang.sin().to(dt)
+
+    def block(x, W, n1, n2, cos, sin, rot):
+        h = F.rms_norm(x, (Hd,), n1, 1e-6)
+        q = F.linear(h, W["q"]).view(B, S, nh, hd).transpose(1, 2)
+        k = F.linear(h, W["k"]).view(B, S, nkv, hd).transpose(1, 2)
+        v = F.linear(h, W["v"]).view(B, S, nkv, hd).transpose(1, 2)
+        q = q * cos + rot(q) * sin
+        k = k * cos + rot(k) * sin
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        x = x + F.linear(a.transpose(1, 2).reshape(B, S, nh * hd), W["o"])
+        h = F.rms_norm(x, (Hd,), n2, 1e-6)
+        m = torch.ops.torch_paras.swiglu(F.linear(h, W["u"]), F.linear(h, W["g"]))
+        return x + F.linear(m, W["d"])
+
+    def rot_cpu(t):
+        return torch.cat([-t[..., hd // 2:], t[..., : hd // 2]], -1)
+
+    want = block(x, W, n1, n2, cos, sin, rot_cpu)
+    to = lambda t: t.to(device)
+    got = block(to(x), {n: to(w) for n, w in W.items()}, to(n1), to(n2), to(cos), to(sin), paras_nn.rotate_half)
+    err = (got.cpu().float() - want.float()).abs()
+    assert got.dtype == dt and got.shape == want.shape
+    assert err.max().item() <= 6e-2 and err.mean().item() <= 4e-3, (err.max().item(), err.mean().item())
