@@ -192,21 +192,38 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_composed_v
     }
 }
 
+constexpr int kComposedUnroll = 4;   // 16-byte vectors per stream in flight per lane
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void swiglu_composed_vec(const std::uint16_t* __restrict__ x,
                                                               const std::uint16_t* __restrict__ gate,
                                                               std::uint16_t* __restrict__ out, long nvec) {
     using E = Elem<T>;
     const std::uint16_t one = E::from_f32(1.0f);
-    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < nvec; i += static_cast<long>(gridDim.x) * kBlock) {
-        const u32x4 xv = load16_nt(x + i * 8), gv = load16_nt(gate + i * 8);
-        const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv);
-        const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv);
-        u32x4 o;
-        std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+    const long stride = static_cast<long>(gridDim.x) * kBlock * kComposedUnroll;
+    for (long base = static_cast<long>(blockIdx.x) * kBlock * kComposedUnroll + threadIdx.x; base < nvec; base += stride) {
+        u32x4 xv[kComposedUnroll], gv[kComposedUnroll];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) oe[j] = E::from_f32(E::to_f32(xe[j]) * E::to_f32(swiglu_one<T>(ge[j], one)));
-        store16_nt(out + i * 8, o);
+        for (int k = 0; k < kComposedUnroll; ++k) {
+            const long i = base + static_cast<long>(k) * kBlock;
+            if (i < nvec) {
+                xv[k] = load16_nt(x + i * 8);
+                gv[k] = load16_nt(gate + i * 8);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kComposedUnroll; ++k) {
+            const long i = base + static_cast<long>(k) * kBlock;
+            if (i < nvec) {
+                const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv[k]);
+                const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv[k]);
+                u32x4 o;
+                std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) oe[j] = E::from_f32(E::to_f32(xe[j]) * E::to_f32(swiglu_one<T>(ge[j], one)));
+                store16_nt(out + i * 8, o);
+            }
+        }
     }
 }
 
@@ -243,7 +260,7 @@ void launch_swiglu_composed16(const void* x, const void* gate, void* out, long n
     long done = 0;
     if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 && n >= 8) {
         const long nvec = n / 8;
-        long blocks = (nvec + kBlock - 1) / kBlock;
+        long blocks = (nvec + kBlock * kComposedUnroll - 1) / (kBlock * kComposedUnroll);
         if (blocks > 0x7fffffffL) blocks = 0x7fffffffL;      // the kernel grid-strides beyond that
         hipLaunchKernelGGL((swiglu_composed_vec<T>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, st, xs, gs, os, nvec);
         done = nvec * 8;
