@@ -311,16 +311,54 @@ __global__ __launch_bounds__(kBlock) void copy_dense_kernel(const u32x4* __restr
     if (i < nvec) store16_nt(dst + i, load16_nt(src + i));
 }
 
+// Both sides dense and suitably aligned: eight elements per thread, one wide load and one wide store.
+template <typename TS, typename TD>
+__global__ __launch_bounds__(kBlock) void convert_dense_kernel(const typename Elem<TS>::store_t* __restrict__ src,
+                                                              typename Elem<TD>::store_t* __restrict__ dst, long n8) {
+    using SS = typename Elem<TS>::store_t;
+    using SD = typename Elem<TD>::store_t;
+    struct alignas(sizeof(SS) * 8 > 16 ? 16 : sizeof(SS) * 8) PackS { SS v[8]; };
+    struct alignas(sizeof(SD) * 8 > 16 ? 16 : sizeof(SD) * 8) PackD { SD v[8]; };
+    const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n8) return;
+    const PackS in = reinterpret_cast<const PackS*>(src)[i];
+    PackD o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if constexpr (sizeof(SS) == 8) o.v[j] = Elem<TD>::from_f64(Elem<TS>::to_f64(in.v[j]));
+        else                           o.v[j] = Elem<TD>::from_f32(Elem<TS>::to_f32(in.v[j]));
+    }
+    reinterpret_cast<PackD*>(dst)[i] = o;
+}
+
+template <typename TS, typename TD>
+void launch_convert(const typename Elem<TS>::store_t* sp, void* dst, long n, const Strided& s, hipStream_t st) {
+    using SD = typename Elem<TD>::store_t;
+    auto* dp = static_cast<SD*>(dst);
+    const bool dense = s.ndim == 0 || (s.ndim == 1 && s.src_strides[0] == 1 && s.dst_strides[0] == 1);
+    long done = 0;
+    if (dense && n >= 8 && ((reinterpret_cast<uintptr_t>(sp) | reinterpret_cast<uintptr_t>(dp)) & 15) == 0) {
+        const long n8 = n / 8;
+        hipLaunchKernelGGL((convert_dense_kernel<TS, TD>), dim3(static_cast<unsigned>((n8 + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, sp, dp, n8);
+        done = n8 * 8;
+        if (done == n) return;
+        Strided t = s;
+        t.ndim = 1; t.sizes[0] = n - done; t.src_strides[0] = 1; t.dst_strides[0] = 1;
+        hipLaunchKernelGGL((copy_convert_kernel<TS, TD>), dim3(grid_for(n - done)), dim3(kBlock), 0, st, sp + done, dp + done, n - done, t);
+        return;
+    }
+    hipLaunchKernelGGL((copy_convert_kernel<TS, TD>), dim3(grid_for(n)), dim3(kBlock), 0, st, sp, dp, n, s);
+}
+
 template <typename TS>
 int convert_from(const void* src, void* dst, long n, const Strided& s, int dst_dtype, hipStream_t st) {
     using SS = typename Elem<TS>::store_t;
     const auto* sp = static_cast<const SS*>(src);
-    const dim3 g(grid_for(n)), b(kBlock);
     switch (dst_dtype) {
-        case PARAS_F32:  hipLaunchKernelGGL((copy_convert_kernel<TS, float>), g, b, 0, st, sp, static_cast<float*>(dst), n, s); break;
-        case PARAS_F64:  hipLaunchKernelGGL((copy_convert_kernel<TS, double>), g, b, 0, st, sp, static_cast<double*>(dst), n, s); break;
-        case PARAS_BF16: hipLaunchKernelGGL((copy_convert_kernel<TS, bf16_t>), g, b, 0, st, sp, static_cast<uint16_t*>(dst), n, s); break;
-        case PARAS_F16:  hipLaunchKernelGGL((copy_convert_kernel<TS, f16_t>), g, b, 0, st, sp, static_cast<uint16_t*>(dst), n, s); break;
+        case PARAS_F32:  launch_convert<TS, float>(sp, dst, n, s, st); break;
+        case PARAS_F64:  launch_convert<TS, double>(sp, dst, n, s, st); break;
+        case PARAS_BF16: launch_convert<TS, bf16_t>(sp, dst, n, s, st); break;
+        case PARAS_F16:  launch_convert<TS, f16_t>(sp, dst, n, s, st); break;
         default: return fail(PARAS_ERR_INVALID, "paras_copy_strided: unknown dtype %d", dst_dtype);
     }
     PARAS_HIP_TRY(hipGetLastError());
@@ -360,6 +398,25 @@ int paras_copy_strided(const void* src, void* dst, int ndim, const int64_t* size
             dst = static_cast<char*>(dst) + nvec * 16;
             n -= done;
             s.ndim = 1; s.sizes[0] = n; s.src_strides[0] = 1; s.dst_strides[0] = 1;
+        }
+        // Rows contiguous on both sides (innermost strides 1) whose length, strides and bases are
+        // multiples of 16 bytes: the same copy with 16-byte elements (head transposes, slices of a fused
+        // projection): an eighth of the index arithmetic for 16-bit tensors, and wide accesses.
+        if (s.ndim >= 2 && elem_size < 16 && s.src_strides[s.ndim - 1] == 1 && s.dst_strides[s.ndim - 1] == 1 &&
+            ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0) {
+            const long per = 16 / elem_size;
+            bool ok = s.sizes[s.ndim - 1] % per == 0;
+            for (int d = 0; d + 1 < s.ndim; ++d) ok = ok && s.src_strides[d] % per == 0 && s.dst_strides[d] % per == 0;
+            if (ok) {
+                Strided w = s;
+                w.sizes[s.ndim - 1] /= per;
+                for (int d = 0; d + 1 < s.ndim; ++d) { w.src_strides[d] /= per; w.dst_strides[d] /= per; }
+                const long nw = n / per;
+                hipLaunchKernelGGL((copy_same_kernel<u32x4>), dim3(grid_for(nw)), b, 0, st, static_cast<const u32x4*>(src),
+                                   static_cast<u32x4*>(dst), nw, w);
+                PARAS_HIP_TRY(hipGetLastError());
+                return PARAS_OK;
+            }
         }
         const dim3 g(grid_for(n));
         switch (elem_size) {

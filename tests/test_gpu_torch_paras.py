@@ -526,3 +526,30 @@ def test_llama_block_forward_matches_cpu(device):
     err = (got.cpu().float() - want.float()).abs()
     assert got.dtype == dt and got.shape == want.shape
     assert err.max().item() <= 6e-2 and err.mean().item() <= 4e-3, (err.max().item(), err.mean().item())
+
+
+def test_strided_copies_and_conversions_wide_paths(device):
+    """Copies whose rows are contiguous run with 16-byte elements, dense conversions eight elements
+    per thread; shapes on and off those paths (odd row lengths, views that start off alignment,
+    broadcast sources) must all give what the CPU gives."""
+    torch.manual_seed(23)
+    for dt in (torch.bfloat16, torch.float32, torch.float16):
+        a = torch.randn(2, 4, 33, 64).to(dt)
+        d = a.to(device)
+        assert torch.equal(d.transpose(1, 2).contiguous().cpu(), a.transpose(1, 2).contiguous())      # head transpose
+        assert torch.equal(d[..., 8:40].contiguous().cpu(), a[..., 8:40].contiguous())                # slice of rows
+        assert torch.equal(d[..., 3:40].contiguous().cpu(), a[..., 3:40].contiguous())                # rows off alignment
+        assert torch.equal(d[:, :, ::2].contiguous().cpu(), a[:, :, ::2].contiguous())                # strided rows
+        assert torch.equal(d.permute(3, 0, 1, 2).contiguous().cpu(), a.permute(3, 0, 1, 2).contiguous())   # no contiguous rows
+        assert torch.equal(d[:, :1].expand(2, 4, 33, 64).contiguous().cpu(), a[:, :1].expand(2, 4, 33, 64).contiguous())
+        for to in (torch.float32, torch.bfloat16, torch.float16, torch.float64):
+            assert torch.equal(d.to(to).cpu(), a.to(to)), f"{dt} -> {to}"
+            b = torch.randn(1003).to(dt)
+            assert torch.equal(b.to(device).to(to).cpu(), b.to(to))
+            assert torch.equal(b.to(device)[1:].to(to).cpu(), b[1:].to(to))                            # unaligned start
+    dst = torch.zeros(4, 6, 16, dtype=torch.bfloat16).to(device)
+    src = torch.randn(4, 3, 16).bfloat16()
+    dst[:, 1::2] = src.to(device)                                                                        # strided destination
+    ref = torch.zeros(4, 6, 16, dtype=torch.bfloat16)
+    ref[:, 1::2] = src
+    assert torch.equal(dst.cpu(), ref)
