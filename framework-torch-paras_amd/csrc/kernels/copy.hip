@@ -227,6 +227,75 @@ __global__ __launch_bounds__(kBlock) void swiglu_composed_vec(const std::uint16_
     }
 }
 
+// ---- elementwise add / sub / mul / div with broadcasting (the reference's binary_kernel,
+// csrc/ops/pointwise_ops.cpp:63-85 with add_out :262-268, sub_out :271-277, mul_out :280-283,
+// div_out :299-302): out = T(a op alpha*b) evaluated in double.  For 16-bit tensors with alpha = 1
+// add, sub and mul in fp32 give the same bits: a product of two such values is exact in fp32, and a
+// sum is either exact in double (then fp32's correctly rounded sum is what double -> float gives)
+// or one operand is below a quarter unit in the last place of the other in both.
+enum { kOpAdd = 0, kOpSub = 1, kOpMul = 2, kOpDiv = 3 };
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::store_t binary_one(int op, typename Elem<T>::store_t as, typename Elem<T>::store_t bs,
+                                                                 double alpha, bool unit_alpha) {
+    using E = Elem<T>;
+    if constexpr (sizeof(typename E::store_t) == 2) {
+        if (unit_alpha && op != kOpDiv) {
+            const float x = E::to_f32(as), y = E::to_f32(bs);
+            return E::from_f32(op == kOpAdd ? x + y : op == kOpSub ? x - y : x * y);
+        }
+    }
+    const double x = E::to_f64(as), y = E::to_f64(bs);
+    double r;
+    switch (op) {
+        case kOpAdd: r = x + alpha * y; break;
+        case kOpSub: r = x - alpha * y; break;
+        case kOpMul: r = x * y; break;
+        default:     r = x / y; break;
+    }
+    return E::from_f64(r);
+}
+
+// general form: `s` carries a's strides as src_strides and b's as dst_strides; out is dense
+template <typename T>
+__global__ __launch_bounds__(kBlock) void binary_strided_kernel(int op, const typename Elem<T>::store_t* __restrict__ a,
+                                                                const typename Elem<T>::store_t* __restrict__ b,
+                                                                typename Elem<T>::store_t* __restrict__ out, long n, const Strided s,
+                                                                double alpha) {
+    const bool unit = alpha == 1.0;
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * kBlock) {
+        long ao, bo;
+        offsets(s, i, &ao, &bo);
+        out[i] = binary_one<T>(op, a[ao], b[bo], alpha, unit);
+    }
+}
+
+// 16-bit tensors, out and a dense, b dense or one value or one row repeated (period `brow` vectors,
+// 0 = one value): eight elements per thread
+template <typename T>
+__global__ __launch_bounds__(kBlock) void binary_vec16_kernel(int op, const std::uint16_t* __restrict__ a,
+                                                              const std::uint16_t* __restrict__ b, std::uint16_t* __restrict__ out,
+                                                              long nvec, long brow, double alpha) {
+    const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= nvec) return;
+    const bool unit = alpha == 1.0;
+    const u32x4 av = load16_nt(a + i * 8);
+    u32x4 bv;
+    if (brow == 0) {
+        const std::uint32_t w = b[0] | (static_cast<std::uint32_t>(b[0]) << 16);
+        bv = u32x4{w, w, w, w};
+    } else {
+        bv = brow == nvec ? load16_nt(b + i * 8) : load16(b + (i % brow) * 8);
+    }
+    const std::uint16_t* ae = reinterpret_cast<const std::uint16_t*>(&av);
+    const std::uint16_t* be = reinterpret_cast<const std::uint16_t*>(&bv);
+    u32x4 o;
+    std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) oe[j] = binary_one<T>(op, ae[j], be[j], alpha, unit);
+    store16_nt(out + i * 8, o);
+}
+
 unsigned grid_for(long n) {
     long g = (n + kBlock - 1) / kBlock;
     if (g > 65536) g = 65536;
@@ -457,6 +526,53 @@ int paras_fill_strided(void* dst, int ndim, const int64_t* sizes, const int64_t*
         case 4: hipLaunchKernelGGL((fill_kernel<uint32_t>), g, b, 0, st, static_cast<uint32_t*>(dst), n, s, static_cast<uint32_t>(value_bits)); break;
         case 8: hipLaunchKernelGGL((fill_kernel<uint64_t>), g, b, 0, st, static_cast<uint64_t*>(dst), n, s, value_bits); break;
         default: return fail(PARAS_ERR_UNSUPPORTED, "paras_fill_strided: element size %d", elem_size);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+int paras_binary_strided(int op, const void* a, const void* b, void* out, int ndim, const int64_t* sizes,
+                         const int64_t* a_strides, const int64_t* b_strides, double alpha, int dtype, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(op >= kOpAdd && op <= kOpDiv, "paras_binary_strided: unknown op %d", op);
+    Strided s;
+    long n = 0;
+    int rc = make_spec(ndim, sizes, a_strides, b_strides, &s, &n);
+    if (rc != PARAS_OK) return rc;
+    if (n == 0) return PARAS_OK;
+    PARAS_REQUIRE(a && b && out, "paras_binary_strided: null pointer");
+    hipStream_t st = nullptr;
+    rc = resolve_stream(stream, &st);
+    if (rc != PARAS_OK) return rc;
+    const dim3 g(grid_for(n)), blk(kBlock);
+    if (dtype == PARAS_BF16 || dtype == PARAS_F16) {
+        // a dense; b dense, a single value, or a trailing block repeated over the leading dims
+        long brow = -1;
+        if (s.ndim <= 1 && (s.ndim == 0 || s.src_strides[0] == 1)) {
+            if (s.ndim == 0 || s.dst_strides[0] == 1) brow = n;
+            else if (s.dst_strides[0] == 0) brow = 0;
+        } else if (s.ndim == 2 && s.src_strides[1] == 1 && s.src_strides[0] == s.sizes[1] && s.dst_strides[1] == 1 &&
+                   s.dst_strides[0] == 0) {
+            brow = s.sizes[1];
+        }
+        const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+        if (brow >= 0 && aligned && n % 8 == 0 && brow % 8 == 0) {
+            const long nvec = n / 8;
+            const dim3 gv(static_cast<unsigned>((nvec + kBlock - 1) / kBlock));
+            if (dtype == PARAS_BF16)
+                hipLaunchKernelGGL((binary_vec16_kernel<bf16_t>), gv, blk, 0, st, op, static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b), static_cast<uint16_t*>(out), nvec, brow / 8, alpha);
+            else
+                hipLaunchKernelGGL((binary_vec16_kernel<f16_t>), gv, blk, 0, st, op, static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b), static_cast<uint16_t*>(out), nvec, brow / 8, alpha);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
+    }
+    switch (dtype) {
+        case PARAS_F32:  hipLaunchKernelGGL((binary_strided_kernel<float>), g, blk, 0, st, op, static_cast<const float*>(a), static_cast<const float*>(b), static_cast<float*>(out), n, s, alpha); break;
+        case PARAS_F64:  hipLaunchKernelGGL((binary_strided_kernel<double>), g, blk, 0, st, op, static_cast<const double*>(a), static_cast<const double*>(b), static_cast<double*>(out), n, s, alpha); break;
+        case PARAS_BF16: hipLaunchKernelGGL((binary_strided_kernel<bf16_t>), g, blk, 0, st, op, static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b), static_cast<uint16_t*>(out), n, s, alpha); break;
+        case PARAS_F16:  hipLaunchKernelGGL((binary_strided_kernel<f16_t>), g, blk, 0, st, op, static_cast<const uint16_t*>(a), static_cast<const uint16_t*>(b), static_cast<uint16_t*>(out), n, s, alpha); break;
+        default: return fail(PARAS_ERR_INVALID, "paras_binary_strided: unknown dtype %d", dtype);
     }
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;

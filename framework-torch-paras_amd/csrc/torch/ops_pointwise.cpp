@@ -1,0 +1,93 @@
+// aten::add / sub / mul / div (Tensor overloads and their in-place forms) for
+// the `paras` device: the residual adds, RoPE products and scalings between
+// the fused ops of a decoder block.  The reference evaluates them in its host
+// engine's binary_kernel (csrc/ops/pointwise_ops.cpp:63-85, 262-302: both
+// operands in the output dtype, a wrapped scalar narrowed to it first,
+// result = T(a op alpha*b) in double); paras_binary_strided does the same on the
+// GPU for float tensors of one dtype, with broadcasting.  Anything else
+// (integer tensors, mixed dtypes that promote) takes ATen on host copies.
+#include "paras_torch.h"
+
+#include <ATen/ExpandUtils.h>
+
+namespace paras_torch {
+namespace {
+
+using at::Tensor;
+
+enum Op { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3 };
+
+bool is_host_number(const Tensor& t) { return !is_paras(t) && t.dim() == 0; }
+
+// The device computes when `self` is a float paras tensor and `other` is a paras tensor of the
+// same dtype or a zero-dim host tensor (a Python number, or a scalar tensor: neither promotes a
+// float tensor's dtype unless it is complex).
+bool device_takes(const Tensor& self, const Tensor& other) {
+    if (!is_paras(self) || float_code(self.scalar_type()) < 0) return false;
+    if (is_paras(other)) return other.scalar_type() == self.scalar_type() && other.device() == self.device();
+    return is_host_number(other) && !other.is_complex();
+}
+
+Tensor on_host(const Tensor& t) { return is_paras(t) ? t.to(c10::Device(c10::kCPU)) : t; }
+
+Tensor host_route(int op, const Tensor& self, const Tensor& other, const at::Scalar& alpha) {
+    const Tensor a = on_host(self), b = on_host(other);
+    Tensor r = op == kAdd ? at::add(a, b, alpha) : op == kSub ? at::sub(a, b, alpha) : op == kMul ? at::mul(a, b) : at::div(a, b);
+    return r.to(is_paras(self) ? self.device() : other.device());
+}
+
+Tensor run(int op, const Tensor& self, const Tensor& other, double alpha) {
+    Tensor b = other;
+    if (!is_paras(other)) {
+        // the number, narrowed to the tensor's dtype as the reference does, as a one-element device tensor
+        b = at::empty({}, self.options());
+        b.fill_(other.to(self.scalar_type()).item());
+    }
+    const std::vector<int64_t> shape = at::infer_size(self.sizes(), b.sizes());
+    TORCH_CHECK(shape.size() <= 8, "paras: tensor rank ", shape.size(), " exceeds kernel limit of 8");
+    const Tensor a = self.expand(shape), bb = b.expand(shape);
+    Tensor out = at::empty(shape, self.options());
+    if (out.numel() == 0) return out;
+    check(paras_binary_strided(op, a.data_ptr(), bb.data_ptr(), out.data_ptr(), static_cast<int>(shape.size()), shape.data(),
+                               a.strides().data(), bb.strides().data(), alpha, require_float_code(self, "paras binary op"),
+                               stream_for(self)));
+    return out;
+}
+
+Tensor binary(int op, const Tensor& self, const Tensor& other, const at::Scalar& alpha) {
+    if (device_takes(self, other)) return run(op, self, other, alpha.toDouble());
+    // number (op) tensor: add and mul commute; the others go to the host
+    if ((op == kAdd || op == kMul) && is_host_number(self) && device_takes(other, self)) return run(op, other, self, alpha.toDouble());
+    return host_route(op, self, other, alpha);
+}
+
+Tensor& binary_(int op, Tensor& self, const Tensor& other, const at::Scalar& alpha) {
+    Tensor r = binary(op, self, other, alpha);
+    TORCH_CHECK(r.sizes() == self.sizes(), "paras: output with shape ", self.sizes(), " doesn't match the broadcast shape ", r.sizes());
+    self.copy_(r);
+    return self;
+}
+
+Tensor add(const Tensor& self, const Tensor& other, const at::Scalar& alpha) { return binary(kAdd, self, other, alpha); }
+Tensor sub(const Tensor& self, const Tensor& other, const at::Scalar& alpha) { return binary(kSub, self, other, alpha); }
+Tensor mul(const Tensor& self, const Tensor& other) { return binary(kMul, self, other, 1); }
+Tensor div(const Tensor& self, const Tensor& other) { return binary(kDiv, self, other, 1); }
+Tensor& add_(Tensor& self, const Tensor& other, const at::Scalar& alpha) { return binary_(kAdd, self, other, alpha); }
+Tensor& sub_(Tensor& self, const Tensor& other, const at::Scalar& alpha) { return binary_(kSub, self, other, alpha); }
+Tensor& mul_(Tensor& self, const Tensor& other) { return binary_(kMul, self, other, 1); }
+Tensor& div_(Tensor& self, const Tensor& other) { return binary_(kDiv, self, other, 1); }
+
+}  // namespace
+
+TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
+    m.impl("add.Tensor", add);
+    m.impl("sub.Tensor", sub);
+    m.impl("mul.Tensor", mul);
+    m.impl("div.Tensor", div);
+    m.impl("add_.Tensor", add_);
+    m.impl("sub_.Tensor", sub_);
+    m.impl("mul_.Tensor", mul_);
+    m.impl("div_.Tensor", div_);
+}
+
+}  // namespace paras_torch

@@ -125,6 +125,16 @@ PARAS_API int paras_copy_strided(const void* src, void* dst, int ndim, const int
 PARAS_API int paras_fill_strided(void* dst, int ndim, const int64_t* sizes, const int64_t* strides,
                                  int elem_size, uint64_t value_bits, void* stream);
 
+/* Elementwise out = T(a op alpha*b) with broadcasting, evaluated as the host
+ * engine does (replaces binary_kernel, csrc/ops/pointwise_ops.cpp:63-85, with
+ * add_out :262-268, sub_out :271-277, mul_out :280-283, div_out :299-302).
+ * op: 0 add, 1 sub, 2 mul, 3 div (alpha is used by add and sub only).  a and b
+ * are views of the output's shape (element strides, 0 = broadcast); out is
+ * dense; all three of the same paras_dtype float type. */
+PARAS_API int paras_binary_strided(int op, const void* a, const void* b, void* out, int ndim,
+                                   const int64_t* sizes, const int64_t* a_strides,
+                                   const int64_t* b_strides, double alpha, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Fused RMSNorm (replaces ptsycl::rms_norm, csrc/ops/fused_ops.cpp:43-88)    */
 /*   ss = sum_j x[r][j]^2 ; rstd[r] = 1/sqrt(ss/H + eps)                      */

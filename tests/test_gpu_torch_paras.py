@@ -553,3 +553,37 @@ def test_strided_copies_and_conversions_wide_paths(device):
     ref = torch.zeros(4, 6, 16, dtype=torch.bfloat16)
     ref[:, 1::2] = src
     assert torch.equal(dst.cpu(), ref)
+
+
+def test_elementwise_binary_ops_on_device_match_the_host_engine(device):
+    """add / sub / mul / div of float tensors run on the device and give the bits of the reference's
+    binary_kernel (double evaluation, one narrowing): same shape, broadcast rows, broadcast single
+    values, Python numbers, alpha, general strides, in-place forms; wide exponent gaps for the
+    fp32 add that stands in for the double one."""
+    torch.manual_seed(29)
+    ops = ((torch.add, O.OP_ADD), (torch.sub, O.OP_SUB), (torch.mul, O.OP_MUL), (torch.div, O.OP_DIV))
+    for dt in (torch.bfloat16, torch.float16, torch.float32, torch.float64):
+        a = torch.randn(3, 5, 16, 64).to(dt)
+        scale = torch.tensor([1e-6, 1.0, 3e4]).view(3, 1, 1, 1) if dt != torch.float16 else torch.tensor([1e-3, 1.0, 30.0]).view(3, 1, 1, 1)
+        b = (torch.randn(3, 5, 16, 64) * scale).to(dt)
+        row = torch.randn(16, 64).to(dt)
+        col = torch.randn(5, 1, 1).to(dt)
+        odd = torch.randn(3, 5, 16, 7).to(dt)
+        for fn, code in ops:
+            for x, y in ((a, b), (a, row), (a, col), (odd, odd.flip(-1)), (a.transpose(1, 2), b.transpose(1, 2))):
+                got = fn(x.to(device), y.to(device)).cpu()
+                assert_bit_exact(got, O.binary(code, x, y), f"{fn.__name__} {dt} {tuple(x.shape)} {tuple(y.shape)}")
+            got = fn(a.to(device), 0.3).cpu()
+            assert_bit_exact(got, O.binary_scalar(code, a, 0.3), f"{fn.__name__} {dt} with a number")
+        assert_bit_exact(torch.add(a.to(device), b.to(device), alpha=0.25).cpu(), O.binary(O.OP_ADD, a, b, 0.25), f"add alpha {dt}")
+        assert_bit_exact((2.0 * a.to(device)).cpu(), O.binary_scalar(O.OP_MUL, a, 2.0), f"number * tensor {dt}")
+        d = a.to(device).clone()
+        d += b.to(device)
+        d *= row.to(device)
+        assert_bit_exact(d.cpu(), O.binary(O.OP_MUL, O.binary(O.OP_ADD, a, b), row), f"in-place {dt}")
+    # integer tensors and promoting mixes are not part of the device surface: host route, same values as the CPU
+    i = torch.arange(12).view(3, 4)
+    assert torch.equal((i.to(device) + i.to(device)).cpu(), i + i)
+    m = torch.randn(4, 4).bfloat16()
+    f = torch.randn(4, 4)
+    assert torch.equal((m.to(device) + f.to(device)).cpu(), m + f)
