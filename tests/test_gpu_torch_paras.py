@@ -587,3 +587,46 @@ def test_elementwise_binary_ops_on_device_match_the_host_engine(device):
     m = torch.randn(4, 4).bfloat16()
     f = torch.randn(4, 4)
     assert torch.equal((m.to(device) + f.to(device)).cpu(), m + f)
+
+
+def test_decoder_block_runs_without_any_host_fallback():
+    """Between its inputs and its output a bf16 decoder block (norms, projections, RoPE, causal GQA
+    attention, SwiGLU MLP, residuals) must not send a single op through the CPU fallback."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, torch, torch.nn.functional as F
+sys.path.insert(0, sys.argv[1])
+import torch_paras
+from torch_paras import nn as pn
+dev = "paras:0"
+torch.manual_seed(0)
+B, S, Hd, nh, nkv, hd, I = 2, 96, 256, 4, 2, 64, 512
+to = lambda t: t.to(torch.bfloat16).to(dev)
+W = {n: to(torch.randn(*shp) * 0.05) for n, shp in dict(q=(nh*hd, Hd), k=(nkv*hd, Hd), v=(nkv*hd, Hd), o=(Hd, nh*hd), g=(I, Hd), u=(I, Hd), d=(Hd, I)).items()}
+n1, n2 = to(torch.ones(Hd)), to(torch.ones(Hd))
+x, cos, sin = to(torch.randn(B, S, Hd)), to(torch.randn(S, hd)), to(torch.randn(S, hd))
+print("=== block starts", file=sys.stderr, flush=True)
+h = F.rms_norm(x, (Hd,), n1, 1e-6)
+q = F.linear(h, W["q"]).view(B, S, nh, hd).transpose(1, 2)
+k = F.linear(h, W["k"]).view(B, S, nkv, hd).transpose(1, 2)
+v = F.linear(h, W["v"]).view(B, S, nkv, hd).transpose(1, 2)
+q = q * cos + pn.rotate_half(q) * sin
+k = k * cos + pn.rotate_half(k) * sin
+a = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+x = x + F.linear(a.transpose(1, 2).reshape(B, S, nh * hd), W["o"])
+h = F.rms_norm(x, (Hd,), n2, 1e-6)
+m = torch.ops.torch_paras.swiglu(F.linear(h, W["u"]), F.linear(h, W["g"]))
+y = x * 0.5 + F.linear(m, W["d"])
+torch_paras.synchronize()
+print("=== block ends", file=sys.stderr, flush=True)
+print("done")
+"""
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "framework-torch-paras_amd")
+    r = subprocess.run([sys.executable, "-c", code, root], capture_output=True, text=True, env=dict(os.environ, PARAS_LOG="1"), timeout=300)
+    assert r.returncode == 0 and "done" in r.stdout, r.stderr[-2000:]
+    err = r.stderr
+    inside = err[err.index("=== block starts"):err.index("=== block ends")]
+    fell = sorted({line.split("for ", 1)[1].strip() for line in inside.splitlines() if "falling back to CPU for" in line})
+    assert not fell, f"ops of the block went through the host: {fell}"
