@@ -296,6 +296,22 @@ __global__ __launch_bounds__(kBlock) void binary_vec16_kernel(int op, const std:
     store16_nt(out + i * 8, o);
 }
 
+// ---- index_select along one dim of a dense tensor seen as [outer, n_src, inner]:
+// dst[o, i, :] = src[o, idx[i], :] (the reference's index_select, csrc/ops/indexing_ops.cpp:96-150;
+// embedding lookups arrive here as dim 0).  `inner` is counted in W-byte units.  An index outside
+// [0, n_src) is clamped into it: the reference does not check either, and a clamp cannot fault.
+template <typename W>
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(const W* __restrict__ src, const long* __restrict__ idx,
+                                                             W* __restrict__ dst, long total, long n_src, long n_idx, long inner) {
+    for (long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x; i < total; i += static_cast<long>(gridDim.x) * kBlock) {
+        const long c = i % inner, r = i / inner;
+        const long sel = r % n_idx, o = r / n_idx;
+        long j = idx[sel];
+        j = j < 0 ? 0 : (j >= n_src ? n_src - 1 : j);
+        dst[i] = src[(o * n_src + j) * inner + c];
+    }
+}
+
 unsigned grid_for(long n) {
     long g = (n + kBlock - 1) / kBlock;
     if (g > 65536) g = 65536;
@@ -526,6 +542,32 @@ int paras_fill_strided(void* dst, int ndim, const int64_t* sizes, const int64_t*
         case 4: hipLaunchKernelGGL((fill_kernel<uint32_t>), g, b, 0, st, static_cast<uint32_t*>(dst), n, s, static_cast<uint32_t>(value_bits)); break;
         case 8: hipLaunchKernelGGL((fill_kernel<uint64_t>), g, b, 0, st, static_cast<uint64_t*>(dst), n, s, value_bits); break;
         default: return fail(PARAS_ERR_UNSUPPORTED, "paras_fill_strided: element size %d", elem_size);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+int paras_index_select(const void* src, const int64_t* index, void* dst, int64_t outer, int64_t n_src, int64_t n_index,
+                       int64_t inner_bytes, void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(outer >= 0 && n_src >= 0 && n_index >= 0 && inner_bytes >= 0, "paras_index_select: negative shape");
+    if (outer == 0 || n_index == 0 || inner_bytes == 0) return PARAS_OK;
+    PARAS_REQUIRE(n_src > 0, "paras_index_select: cannot select from an empty dimension");
+    PARAS_REQUIRE(src && index && dst, "paras_index_select: null pointer");
+    hipStream_t st = nullptr;
+    int rc = resolve_stream(stream, &st);
+    if (rc != PARAS_OK) return rc;
+    const long* idx = reinterpret_cast<const long*>(index);
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | static_cast<uintptr_t>(inner_bytes);
+    const int w = (bits % 16 == 0) ? 16 : (bits % 8 == 0) ? 8 : (bits % 4 == 0) ? 4 : (bits % 2 == 0) ? 2 : 1;
+    const long inner = inner_bytes / w, total = outer * n_index * inner;
+    const dim3 g(grid_for(total)), b(kBlock);
+    switch (w) {
+        case 16: hipLaunchKernelGGL((gather_rows_kernel<u32x4>), g, b, 0, st, static_cast<const u32x4*>(src), idx, static_cast<u32x4*>(dst), total, (long)n_src, (long)n_index, inner); break;
+        case 8:  hipLaunchKernelGGL((gather_rows_kernel<uint64_t>), g, b, 0, st, static_cast<const uint64_t*>(src), idx, static_cast<uint64_t*>(dst), total, (long)n_src, (long)n_index, inner); break;
+        case 4:  hipLaunchKernelGGL((gather_rows_kernel<uint32_t>), g, b, 0, st, static_cast<const uint32_t*>(src), idx, static_cast<uint32_t*>(dst), total, (long)n_src, (long)n_index, inner); break;
+        case 2:  hipLaunchKernelGGL((gather_rows_kernel<uint16_t>), g, b, 0, st, static_cast<const uint16_t*>(src), idx, static_cast<uint16_t*>(dst), total, (long)n_src, (long)n_index, inner); break;
+        default: hipLaunchKernelGGL((gather_rows_kernel<uint8_t>), g, b, 0, st, static_cast<const uint8_t*>(src), idx, static_cast<uint8_t*>(dst), total, (long)n_src, (long)n_index, inner); break;
     }
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;

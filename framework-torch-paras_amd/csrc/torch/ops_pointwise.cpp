@@ -1,5 +1,5 @@
-// aten::add / sub / mul / div (Tensor overloads and their in-place forms) for
-// the `paras` device: the residual adds, RoPE products and scalings between
+// aten::add / sub / mul / div (Tensor overloads and their in-place forms), cat and
+// index_select (and through it embedding) for the `paras` device: the residual adds, RoPE products and scalings between
 // the fused ops of a decoder block.  The reference evaluates them in its host
 // engine's binary_kernel (csrc/ops/pointwise_ops.cpp:63-85, 262-302: both
 // operands in the output dtype, a wrapped scalar narrowed to it first,
@@ -77,9 +77,62 @@ Tensor& sub_(Tensor& self, const Tensor& other, const at::Scalar& alpha) { retur
 Tensor& mul_(Tensor& self, const Tensor& other) { return binary_(kMul, self, other, 1); }
 Tensor& div_(Tensor& self, const Tensor& other) { return binary_(kDiv, self, other, 1); }
 
+// cat as the reference composes it (csrc/ops/pointwise_ops.cpp:1558-1590): the inputs are copied
+// into slices of the result by the device's strided copy.
+Tensor cat(const at::ITensorListRef& tensors, int64_t dim) {
+    auto list = tensors.materialize();
+    TORCH_CHECK(!list.empty(), "cat: expected non-empty tensor list");
+    const Tensor* first = nullptr;
+    for (const auto& r : list)
+        if (!(r.get().dim() == 1 && r.get().numel() == 0)) { first = &r.get(); break; }    // legacy empty tensors are skipped
+    if (first == nullptr) return at::empty({0}, list[0].get().options());
+    const int64_t d = c10::maybe_wrap_dim(dim, first->dim());
+    std::vector<int64_t> shape = first->sizes().vec();
+    shape[d] = 0;
+    for (const auto& r : list) {
+        const Tensor& t = r.get();
+        if (t.dim() == 1 && t.numel() == 0) continue;
+        TORCH_CHECK(t.dim() == first->dim() && t.scalar_type() == first->scalar_type() && is_paras(t),
+                    "paras cat: tensors must share rank, dtype and device");
+        for (int64_t k = 0; k < t.dim(); ++k)
+            TORCH_CHECK(k == d || t.size(k) == first->size(k), "paras cat: sizes must match except in dimension ", d);
+        shape[d] += t.size(d);
+    }
+    Tensor out = at::empty(shape, first->options());
+    int64_t off = 0;
+    for (const auto& r : list) {
+        const Tensor& t = r.get();
+        if (t.numel() == 0) continue;
+        out.narrow(d, off, t.size(d)).copy_(t);
+        off += t.size(d);
+    }
+    return out;
+}
+
+Tensor index_select(const Tensor& self, int64_t dim, const Tensor& index) {
+    TORCH_CHECK(index.dim() <= 1, "paras index_select: index must be 0-D or 1-D");
+    TORCH_CHECK(index.scalar_type() == c10::kLong || index.scalar_type() == c10::kInt, "paras index_select: index must be int32 or int64");
+    const int64_t d = c10::maybe_wrap_dim(dim, self.dim());
+    Tensor idx = (index.dim() == 0 ? index.unsqueeze(0) : index).to(self.device(), c10::kLong).contiguous();
+    Tensor src = self.dim() == 0 ? self.reshape({1}) : self.contiguous();
+    std::vector<int64_t> shape = src.sizes().vec();
+    int64_t outer = 1, inner = 1;
+    for (int64_t k = 0; k < d; ++k) outer *= shape[k];
+    for (int64_t k = d + 1; k < src.dim(); ++k) inner *= shape[k];
+    const int64_t n_src = shape[d];
+    shape[d] = idx.numel();
+    Tensor out = at::empty(shape, src.options());
+    if (out.numel() > 0)
+        check(paras_index_select(src.data_ptr(), idx.data_ptr<int64_t>(), out.data_ptr(), outer, n_src, idx.numel(),
+                                 inner * static_cast<int64_t>(src.element_size()), stream_for(self)));
+    return self.dim() == 0 ? out.reshape({}) : out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY_IMPL(aten, PrivateUse1, m) {
+    m.impl("cat", cat);
+    m.impl("index_select", index_select);
     m.impl("add.Tensor", add);
     m.impl("sub.Tensor", sub);
     m.impl("mul.Tensor", mul);

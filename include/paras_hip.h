@@ -125,6 +125,13 @@ PARAS_API int paras_copy_strided(const void* src, void* dst, int ndim, const int
 PARAS_API int paras_fill_strided(void* dst, int ndim, const int64_t* sizes, const int64_t* strides,
                                  int elem_size, uint64_t value_bits, void* stream);
 
+/* dst[o, i, :] = src[o, index[i], :] for a dense src seen as [outer, n_src,
+ * inner_bytes] and int64 device indices (replaces index_select_out,
+ * csrc/ops/indexing_ops.cpp:96-150; embedding lookups are dim 0).  Indices
+ * outside [0, n_src) are clamped into it. */
+PARAS_API int paras_index_select(const void* src, const int64_t* index, void* dst, int64_t outer,
+                                 int64_t n_src, int64_t n_index, int64_t inner_bytes, void* stream);
+
 /* Elementwise out = T(a op alpha*b) with broadcasting, evaluated as the host
  * engine does (replaces binary_kernel, csrc/ops/pointwise_ops.cpp:63-85, with
  * add_out :262-268, sub_out :271-277, mul_out :280-283, div_out :299-302).

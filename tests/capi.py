@@ -62,6 +62,7 @@ SIGNATURES = {
     "paras_moe_route": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp]),
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
+    "paras_index_select": (i32, [vp, vp, vp, i64, i64, i64, i64, vp]),
     "paras_binary_strided": (i32, [i32, vp, vp, vp, i32, vp, vp, vp, f64, i32, vp]),
     "paras_gemm_nt": (i32, [vp, vp, vp, vp] + [i64] * 12 + [f64, f64, i32, vp]),
     "paras_gemm_nt_workspace": (sz, [i64, i64, i64, i64, i32]),

@@ -630,3 +630,31 @@ print("done")
     inside = err[err.index("=== block starts"):err.index("=== block ends")]
     fell = sorted({line.split("for ", 1)[1].strip() for line in inside.splitlines() if "falling back to CPU for" in line})
     assert not fell, f"ops of the block went through the host: {fell}"
+
+
+def test_cat_index_select_and_embedding_on_device(device):
+    """KV-cache appends, row gathers and embedding lookups stay on the device and equal the CPU's."""
+    torch.manual_seed(37)
+    for dt in (torch.bfloat16, torch.float32, torch.int64):
+        mk = (lambda *s: torch.randn(*s).to(dt)) if dt.is_floating_point else (lambda *s: torch.randint(-50, 50, s))
+        a, b, c = mk(2, 4, 7, 16), mk(2, 4, 1, 16), mk(2, 4, 3, 16)
+        for dim in (2, -2):
+            assert torch.equal(torch.cat([a.to(device), b.to(device), c.to(device)], dim).cpu(), torch.cat([a, b, c], dim))
+        assert torch.equal(torch.cat([a.to(device), a.to(device)], 0).cpu(), torch.cat([a, a], 0))
+        assert torch.equal(torch.cat([a.to(device), a.to(device)], -1).cpu(), torch.cat([a, a], -1))
+        assert torch.equal(torch.cat([a.to(device).transpose(1, 2), a.to(device).transpose(1, 2)], 1).cpu(),
+                           torch.cat([a.transpose(1, 2), a.transpose(1, 2)], 1))
+        t = mk(5, 6, 9)
+        idx = torch.tensor([4, 0, 0, 3, 1])
+        for dim in (0, 1, 2, -1):
+            n = t.size(dim)
+            ix = idx % n
+            assert torch.equal(torch.index_select(t.to(device), dim, ix.to(device)).cpu(), torch.index_select(t, dim, ix)), f"{dt} dim {dim}"
+        assert torch.equal(torch.index_select(t.to(device), 0, torch.tensor(2).to(device)).cpu(), torch.index_select(t, 0, torch.tensor(2)))
+    w = torch.randn(1000, 64).bfloat16()
+    tok = torch.randint(0, 1000, (3, 17))
+    assert torch.equal(F.embedding(tok.to(device), w.to(device)).cpu(), F.embedding(tok, w))
+    w33 = torch.randn(50, 33).half()                                       # rows that are not a multiple of 16 bytes
+    assert torch.equal(F.embedding(tok.to(device) % 50, w33.to(device)).cpu(), F.embedding(tok % 50, w33))
+    with pytest.raises(RuntimeError):
+        torch.cat([torch.zeros(2, 3).to(device), torch.zeros(2, 4).to(device)], 0)
