@@ -316,7 +316,7 @@ def main() -> int:
             "value": round((bytes_b + bytes_s + bytes_r) / (ms_b + ms_s + ms_r) / 1e6, 1), "unit": "GB/s",
             "ms_per_step": round(ms_b + ms_s + ms_r, 4),
             "rms_norm_bwd": {"ms": round(ms_b, 4), "algorithmic_bytes_per_launch": bytes_b,
-                             "kernel": "rms_norm_bwd_fused<bf16,2> + rms_norm_bwd_dw_final_wide",
+                             "kernel": "rms_norm_bwd_fused<bf16,1,512> + rms_norm_bwd_dw_final_wide",
                              "roofline": roofline("hbm", gb(bytes_b, ms_b), "rms_norm_bwd_fused")},
             "swiglu_bwd": {"ms": round(ms_s, 4), "algorithmic_bytes_per_launch": bytes_s, "kernel": "swiglu_bwd_vec<bf16>",
                            "roofline": roofline("hbm", gb(bytes_s, ms_s), "swiglu_bwd_vec")},

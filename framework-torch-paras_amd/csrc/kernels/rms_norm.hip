@@ -222,10 +222,11 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final(
 // column sums in ONE pass over grad_out and x.  A workgroup owns a slab of kDwSlabRows rows; each
 // thread keeps the same NV vectors of every row (and of w), so its 8*NV column sums live in
 // registers across the slab, and the next row's vectors are requested before the current row's
-// reduction.  Arithmetic in fp64 in the host's order of operations.  (NV = 2 needs 136 registers:
-// three workgroups per CU.  Re-reading w per row to fit four measured 20 % slower.)
+// reduction.  Arithmetic in fp64 in the host's order of operations.  One vector per thread needs
+// 96 registers (five waves per SIMD), two need 136-144 (three): rows are spread over 256, 512 or
+// 1024 threads with one vector each (4096-element rows: 98.7 us with 256 x 2, 93.3 us with 512 x 1).
 template <typename T, int NV, int BLOCK>
-__global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? 2 : (NV == 1 ? 4 : 3))) void rms_norm_bwd_fused(
+__global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? (BLOCK == 1024 ? 4 : 2) : 4)) void rms_norm_bwd_fused(
     const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
     const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
     using E = Elem<T>;
@@ -385,10 +386,10 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
             const dim3 grid(static_cast<unsigned>(slabs));
             if (nvec <= kBlock)
                 hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, kBlock>), grid, dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
-            else if (nvec <= kBlock * 2)
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 2, kBlock>), grid, dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
-            else   // rows of up to 8192 elements: the same two vectors per thread on 512 threads
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 2, 512>), grid, dim3(512), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            else if (nvec <= 512)
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, 512>), grid, dim3(512), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            else   // rows of up to 8192 elements
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, 1024>), grid, dim3(1024), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
             PARAS_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + 7) / 8)), dim3(kBlock), 0, s,
                                part, static_cast<S*>(gw), slabs, H);
