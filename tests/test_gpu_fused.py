@@ -156,6 +156,20 @@ def test_rms_norm_backward_one_pass_kernel(shape, dtype):
     assert_bit_exact(gw, wgw, "rms_norm grad_weight")
 
 
+def test_rms_norm_backward_many_rows_uses_taller_slabs():
+    """From 16384 rows on the one-pass kernel gives a workgroup 32 rows instead of 16 (half the
+    partial column sums); the last slab here is ragged, and a row count just below the switch runs
+    beside it."""
+    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520)):
+        torch.manual_seed(rows)
+        x, w, go = torch.randn(rows, H).bfloat16(), (1 + 0.1 * torch.randn(H)).bfloat16(), torch.randn(rows, H).bfloat16()
+        _, rstd = O.rms_norm(x, w, 1e-6)
+        gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(rstd))
+        wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
+        assert_bit_exact(gx, wgx, f"rms_norm grad_input {rows}x{H}")
+        assert_bit_exact(gw, wgw, f"rms_norm grad_weight {rows}x{H}")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_rotate_half_vector_path_and_fallbacks(dtype):
     for shape in [(3, 5, 128), (7, 64), (2, 16), (4, 48), (3, 24), (5, 130)]:
