@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final(
 // column sums in ONE pass over grad_out and x.  A workgroup owns a slab of kDwSlabRows rows; each
 // thread keeps the same NV vectors of every row (and of w), so its 8*NV column sums live in
 // registers across the slab, and the next row's vectors are requested before the current row's
-// reduction.  Arithmetic in fp64 in the host's order of operations.  One vector per thread needs
+// reduction (two rows ahead: no change).  Arithmetic in fp64 in the host's order of operations.  One vector per thread needs
 // 96 registers (five waves per SIMD), two need 136-144 (three): rows are spread over 256, 512 or
 // 1024 threads with one vector each (4096-element rows: 98.7 us with 256 x 2, 93.3 us with 512 x 1).
 template <typename T, int NV, int BLOCK>
@@ -267,6 +267,10 @@ __global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? (BLOCK == 1024 ? 4 : 2) : 4))
         }
         const double rr = static_cast<double>(rstd[r]);
         double dot = 0.0;
+        // g*w and x as doubles stay in registers for the second half of the row (the register
+        // budget of two 512-thread workgroups per CU has room for them; converting and
+        // multiplying again costs a fifth of the row's fp64 instructions).
+        double gwd[NV][V], xd[NV][V];
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i]) {
@@ -275,9 +279,11 @@ __global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? (BLOCK == 1024 ? 4 : 2) : 4))
                 const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
-                    const double g = E::to_f64(ge[j]), xj = E::to_f64(xe[j]);
-                    dot += g * E::to_f64(we[j]) * xj;
-                    dw[i][j] += g * xj * rr;
+                    const double g = E::to_f64(ge[j]);
+                    xd[i][j] = E::to_f64(xe[j]);
+                    gwd[i][j] = g * E::to_f64(we[j]);
+                    dot += gwd[i][j] * xd[i][j];
+                    dw[i][j] += g * xd[i][j] * rr;
                 }
             }
         {   // sum over the workgroup; two alternating slot sets, so one barrier per row
@@ -293,14 +299,11 @@ __global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? (BLOCK == 1024 ? 4 : 2) : 4))
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i]) {
-                const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv[i]);
-                const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv[i]);
-                const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
                 u32x4 o;
                 std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
 #pragma unroll
                 for (int j = 0; j < V; ++j)
-                    oe[j] = E::from_f64(E::to_f64(ge[j]) * E::to_f64(we[j]) * rr - coef * E::to_f64(xe[j]) * dot);
+                    oe[j] = E::from_f64(gwd[i][j] * rr - coef * xd[i][j] * dot);
                 store16_nt(gx + r * H + static_cast<long>(threadIdx.x + i * BLOCK) * V, o);
             }
     }
