@@ -100,7 +100,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=25)
+    ap.add_argument("--warmup", type=int, default=200)     # steady clocks: the first ~100 ms of launches after an idle gap run 1-2 % slower
     ap.add_argument("--workload", default="all",
                     choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe", "linear", "backward_ops", "copy"],
                     help="'copy' is the counter calibration: a plain 1 GiB device copy, not part of 'all'")
