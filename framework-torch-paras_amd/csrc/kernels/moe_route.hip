@@ -12,9 +12,17 @@
 //   argsort(stable) of the flattened expert ids (csrc/ops/sort_ops.cpp:129-166)
 //            == counting sort: histogram, exclusive scan, stable scatter
 //
-// Three launches over 256-token workgroups:
-//   route_topk     one lane per token (E <= 64 logits are one or two cache
-//                  lines); LDS histogram of the workgroup's expert ids
+// Up to 65536 tokens: ONE kernel over 256-token workgroups (route_fused_kernel), all of
+// them resident at once.  A lane owns a token: its row of logits arrives as one 16-byte
+// load (E = 8 of a 16-bit type) and stays in registers for the k selection scans; the
+// workgroup counts its tokens per expert with wavefront ballots, publishes the counts,
+// and meets the other workgroups at a counter in device memory (a bounded wait); then
+// every workgroup adds up the counts of all workgroups (expert offsets) and of the
+// workgroups before it (its own start positions) and scatters its (token, slot) pairs.
+// The counter is cleared by a one-workgroup fill kernel queued in front.
+//
+// More tokens than that: three launches over 256-token workgroups,
+//   route_topk     one lane per token; LDS histogram of the workgroup's expert ids
 //   route_scan     one 64-lane workgroup turns the per-workgroup histograms
 //                  into per-workgroup start positions, counts and offsets
 //   route_scatter  rank inside the workgroup from wavefront ballots (a token
@@ -157,6 +165,244 @@ __global__ __launch_bounds__(kBlock) void route_scatter_kernel(const long* __res
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// One-launch routing.  Scratch layout (bytes): [0] arrival counter (u32, zero at launch),
+// [4] set to 1 by a workgroup whose bounded wait ran out (outputs are undefined then),
+// [kScratchHeader ...] int counts[nblk][E].
+constexpr int  kScratchHeader   = 256;
+constexpr int  kFusedMaxBlocks  = 256;          // 256-thread workgroups: all resident on 256 CUs
+constexpr long kFusedMaxTokens  = static_cast<long>(kFusedMaxBlocks) * kBlock;
+constexpr int  kSpinLimit       = 1 << 22;      // polls of ~64 clocks each: seconds, then give up
+
+__global__ __launch_bounds__(64) void route_clear_kernel(unsigned* __restrict__ header) {
+    if (threadIdx.x < 2) header[threadIdx.x] = 0u;
+}
+
+// kSmall: E <= 8 and k <= 8, the row and the selection live in registers.
+template <typename T, bool kSmall>
+__global__ __launch_bounds__(kBlock) void route_fused_kernel(
+    const typename Elem<T>::store_t* __restrict__ logits, long T_, int E, int k, long* __restrict__ topi,
+    float* __restrict__ topw, long* __restrict__ order, long* __restrict__ inv_order, long* __restrict__ counts,
+    long* __restrict__ offsets, unsigned char* __restrict__ scratch, int spin_limit) {
+    using El = Elem<T>;
+    __shared__ int wave_cnt[kWavesPerBlock][kMaxExperts];
+    __shared__ long tot[kMaxExperts + 1];     // after the meeting: exclusive expert offsets
+    __shared__ int  pre[kMaxExperts];         // tokens of expert e in the workgroups before this one
+    __shared__ int  gave_up;
+    unsigned* header = reinterpret_cast<unsigned*>(scratch);
+    int* block_cnt = reinterpret_cast<int*>(scratch + kScratchHeader);
+    const int nblk = gridDim.x, bid = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const long t = static_cast<long>(bid) * kBlock + tid;
+    const bool live = t < T_;
+    if (tid == 0) gave_up = 0;
+
+    // ---- top-k and gate weights of this lane's token ---------------------------------
+    int sel[kSmall ? 8 : 1];                  // chosen expert per slot (small path)
+    if (live) {
+        const auto* row = logits + t * E;
+        double val[kSmall ? 8 : 1];
+        if constexpr (kSmall) {
+            if (sizeof(typename El::store_t) == 2 && E == 8) {     // the row is one aligned 16-byte load
+                const u32x4 w = load16(row);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    val[j] = El::to_f64(static_cast<typename El::store_t>(w[j >> 1] >> (16 * (j & 1))));
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) val[j] = j < E ? El::to_f64(row[j]) : 0.0;
+            }
+        }
+        double prev_val = 0.0, vmax = -INFINITY;
+        int prev_idx = -1;
+        bool has_prev = false;
+        double kept[kSmall ? 8 : 1];          // the kept values as fp32 (the softmax input is topv.float())
+        for (int s = 0; s < k; ++s) {
+            double best_val = 0.0;
+            int best_idx = -1;
+            bool has_best = false;
+            auto consider = [&](int j, double v) {
+                const bool within = !has_prev || (v < prev_val) || (v == prev_val && j > prev_idx);
+                const bool better = !has_best || (v > best_val) || (v == best_val && j < best_idx);
+                if (within && better) {
+                    best_val = v;
+                    best_idx = j;
+                    has_best = true;
+                }
+            };
+            if constexpr (kSmall) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (j < E) consider(j, val[j]);
+            } else {
+                for (int j = 0; j < E; ++j) consider(j, El::to_f64(row[j]));
+            }
+            topi[t * k + s] = best_idx;
+            prev_val = best_val;
+            prev_idx = best_idx;
+            has_prev = true;
+            const double vf = static_cast<double>(static_cast<float>(best_val));
+            if (vf > vmax) vmax = vf;
+            if constexpr (kSmall) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (i == s) {
+                        sel[i] = best_idx;
+                        kept[i] = vf;
+                    }
+            }
+        }
+        // gate weights: exp(v - max) / sum in fp64, narrowed to fp32
+        if constexpr (kSmall) {
+            double ex[8], sum = 0.0;
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+                if (s < k) {
+                    ex[s] = exp(kept[s] - vmax);
+                    sum += ex[s];
+                }
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+                if (s < k) topw[t * k + s] = static_cast<float>(ex[s] / sum);
+        } else {
+            double sum = 0.0;
+            for (int s = 0; s < k; ++s) {
+                const long idx = topi[t * k + s];
+                sum += exp(static_cast<double>(El::to_f32(row[idx >= 0 ? idx : 0])) - vmax);
+            }
+            for (int s = 0; s < k; ++s) {
+                const long idx = topi[t * k + s];
+                topw[t * k + s] = static_cast<float>(exp(static_cast<double>(El::to_f32(row[idx >= 0 ? idx : 0])) - vmax) / sum);
+            }
+        }
+    }
+    // slot in which this lane's token chose expert e, or -1 (a token chooses an expert at most once)
+    auto slot_of = [&](int e) -> int {
+        int mine = -1;
+        if (live) {
+            if constexpr (kSmall) {
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+                    if (s < k && sel[s] == e) mine = s;
+            } else {
+                for (int s = 0; s < k; ++s)
+                    if (topi[t * k + s] == e) mine = s;
+            }
+        }
+        return mine;
+    };
+
+    // ---- counts of this workgroup, published for the others ---------------------------
+    for (int e = 0; e < E; ++e) {
+        const unsigned long long mask = __ballot(slot_of(e) >= 0);
+        if (lane == 0) wave_cnt[wave][e] = __popcll(mask);
+    }
+    __syncthreads();
+    if (tid < E) {
+        int c = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) c += wave_cnt[w][tid];
+        __hip_atomic_store(&block_cnt[static_cast<long>(bid) * E + tid], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    }
+    __syncthreads();
+
+    // ---- meet: every workgroup of the grid has published ------------------------------
+    if (tid == 0) {
+        __hip_atomic_fetch_add(&header[0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        int polls = 0;
+        while (__hip_atomic_load(&header[0], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < static_cast<unsigned>(nblk)) {
+            if (++polls >= spin_limit) {
+                gave_up = 1;
+                __hip_atomic_store(&header[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    __syncthreads();
+    if (gave_up) return;                      // uniform: every wave of the workgroup leaves here
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+
+    // ---- totals (expert offsets) and the share of the workgroups before this one ---------
+    for (int e = wave; e < E; e += kWavesPerBlock) {
+        int all = 0, before = 0;
+        for (int j = lane; j < nblk; j += kWave) {
+            const int c = __hip_atomic_load(&block_cnt[static_cast<long>(j) * E + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            all += c;
+            before += j < bid ? c : 0;
+        }
+        all = wave_allreduce(all, [](int a, int b) { return a + b; });
+        before = wave_allreduce(before, [](int a, int b) { return a + b; });
+        if (lane == 0) {
+            tot[e] = all;
+            pre[e] = before;
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        long run = 0;
+        for (int e = 0; e < E; ++e) {
+            const long c = tot[e];
+            if (bid == 0) {
+                counts[e] = c;
+                offsets[e] = run;
+            }
+            tot[e] = run;
+            run += c;
+        }
+        if (bid == 0) offsets[E] = run;
+    }
+    __syncthreads();
+
+    // ---- stable scatter: expert offset + earlier workgroups + earlier waves + earlier lanes
+    const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (kWave - lane));
+    for (int e = 0; e < E; ++e) {
+        const int mine = slot_of(e);
+        const unsigned long long mask = __ballot(mine >= 0);
+        if (mine >= 0) {
+            long pos = tot[e] + pre[e] + __popcll(mask & below);
+            for (int w = 0; w < wave; ++w) pos += wave_cnt[w][e];
+            order[pos] = t * k + mine;
+            if (inv_order) inv_order[t * k + mine] = pos;
+        }
+    }
+}
+
+template <typename T>
+void launch_fused(const void* logits, long T_, int E, int k, long* topi, float* topw, long* order, long* inv_order,
+                  long* counts, long* offsets, unsigned char* scratch, hipStream_t s) {
+    using store_t = typename Elem<T>::store_t;
+    const dim3 grid(static_cast<unsigned>((T_ + kBlock - 1) / kBlock)), block(kBlock);
+    hipLaunchKernelGGL(route_clear_kernel, dim3(1), dim3(64), 0, s, reinterpret_cast<unsigned*>(scratch));
+    if (E <= 8 && k <= 8)
+        hipLaunchKernelGGL((route_fused_kernel<T, true>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
+                           topw, order, inv_order, counts, offsets, scratch, kSpinLimit);
+    else
+        hipLaunchKernelGGL((route_fused_kernel<T, false>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
+                           topw, order, inv_order, counts, offsets, scratch, kSpinLimit);
+}
+
+// Shared by the entry points: routes on `scratch` (device memory of route_scratch_bytes(T, E)).
+int route_on(const void* logits, long T_, int E, int k, int dtype, long* topi, float* topw, long* order, long* inv_order,
+             long* counts, long* offsets, unsigned char* scratch, hipStream_t s) {
+    switch (dtype) {
+        case PARAS_F32:  launch_fused<float>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
+        case PARAS_F64:  launch_fused<double>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
+        case PARAS_BF16: launch_fused<bf16_t>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
+        case PARAS_F16:  launch_fused<f16_t>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
+        default: return fail(PARAS_ERR_INVALID, "paras_moe_route: unknown dtype %d", dtype);
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+size_t route_scratch_bytes(long T_, long E) {
+    const long nblk = (T_ + kBlock - 1) / kBlock;
+    return static_cast<size_t>(kScratchHeader) + static_cast<size_t>(nblk * E) * sizeof(int);
+}
+
 }  // namespace
 }  // namespace paras
 
@@ -165,8 +411,7 @@ extern "C" {
 size_t paras_moe_route_workspace(int64_t T, int64_t E, int64_t k) {
     (void)k;
     if (T <= 0 || E <= 0) return 0;
-    const int64_t nblk = (T + paras::kBlock - 1) / paras::kBlock;
-    return static_cast<size_t>(nblk * E) * sizeof(int);
+    return paras::route_scratch_bytes(T, E);
 }
 
 int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dtype, int64_t* topi,
@@ -191,8 +436,11 @@ int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dty
     static_assert(sizeof(long) == sizeof(int64_t), "LP64 expected");
     const long nblk = (T + kBlock - 1) / kBlock;
     PARAS_REQUIRE(nblk <= 0x7fffffffL && T * k <= 0x7fffffffL, "paras_moe_route: too many routed rows");
-    int* hist = static_cast<int*>(workspace);
     long* ti = reinterpret_cast<long*>(topi);
+    if (T <= kFusedMaxTokens)
+        return route_on(logits, T, (int)E, (int)k, dtype, ti, topw, reinterpret_cast<long*>(order), reinterpret_cast<long*>(inv_order),
+                        reinterpret_cast<long*>(counts), reinterpret_cast<long*>(offsets), static_cast<unsigned char*>(workspace), s);
+    int* hist = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) + kScratchHeader);
     const dim3 grid(static_cast<unsigned>(nblk)), block(kBlock);
     switch (dtype) {
         case PARAS_F32:

@@ -38,6 +38,7 @@ void prepare(const Tensor& query, const Tensor& key, const Tensor& value, const 
     TORCH_CHECK(query.dim() >= 3 && key.dim() >= 3 && value.dim() >= 3,
                 "paras sdpa: query/key/value must be at least 3-D (..., seq, head_dim)");
     const bool has_mask = attn_mask.has_value() && attn_mask->defined();
+    require_same_device("paras sdpa", query, {{"key", &key}, {"value", &value}, {"attn_mask", has_mask ? &*attn_mask : nullptr}});
     TORCH_CHECK(!(is_causal && has_mask), "paras sdpa: is_causal and attn_mask are mutually exclusive");
     TORCH_CHECK(query.scalar_type() == key.scalar_type() && key.scalar_type() == value.scalar_type(),
                 "paras sdpa: query, key and value must have the same dtype");
@@ -214,8 +215,14 @@ OverrideableResult sdpa_overrideable(const Tensor& query, const Tensor& key, con
 int64_t fused_sdp_choice(const Tensor& query, const Tensor& key, const Tensor& value,
                          const c10::optional<Tensor>& attn_mask, double dropout_p, bool is_causal,
                          c10::optional<double> scale, bool enable_gqa) {
-    (void)key; (void)value; (void)attn_mask; (void)is_causal; (void)scale; (void)enable_gqa;
-    const bool fused = dropout_p == 0.0 && float_code(query.scalar_type()) >= 0 && query.dim() >= 3;
+    (void)attn_mask; (void)is_causal; (void)scale;
+    // The fused op maps query heads onto fewer key/value heads by itself; the reference only
+    // does so under enable_gqa (csrc/ops/attention_ops.cpp:83-92) and otherwise fails in its
+    // matmul.  Without the flag such shapes go to the math op, whose checks raise.  Inputs that
+    // need gradients also go there: the fused forward has no backward op behind it.
+    const bool heads_ok = query.dim() < 3 || key.dim() < 3 || enable_gqa || key.size(-3) == query.size(-3) || key.size(-3) == 1;
+    const bool needs_grad = at::GradMode::is_enabled() && (query.requires_grad() || key.requires_grad() || value.requires_grad());
+    const bool fused = dropout_p == 0.0 && float_code(query.scalar_type()) >= 0 && query.dim() >= 3 && heads_ok && !needs_grad;
     return static_cast<int64_t>(fused ? sdp::SDPBackend::overrideable : sdp::SDPBackend::math);
 }
 

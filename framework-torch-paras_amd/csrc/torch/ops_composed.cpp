@@ -22,6 +22,7 @@ Tensor rms_norm(const Tensor& input, c10::IntArrayRef normalized_shape, const c1
         H *= normalized_shape[i];
     }
     const bool has_w = weight.has_value() && weight->defined();
+    require_same_device("paras rms_norm", input, {{"weight", has_w ? &*weight : nullptr}});
     if (has_w)
         TORCH_CHECK(weight->sizes().equals(normalized_shape), "paras rms_norm: weight shape must equal normalized_shape");
     Tensor in = input.contiguous();
@@ -38,6 +39,7 @@ Tensor rms_norm(const Tensor& input, c10::IntArrayRef normalized_shape, const c1
 
 Tensor swiglu_device(const Tensor& x, const Tensor& gate) {
     TORCH_CHECK(x.scalar_type() == gate.scalar_type(), "paras swiglu: x and gate must have the same dtype");
+    require_same_device("paras swiglu", x, {{"gate", &gate}});
     auto shape = at::infer_size(x.sizes(), gate.sizes());
     Tensor xe = x.expand(shape).contiguous(), ge = gate.expand(shape).contiguous();
     Tensor out = at::empty_like(xe);

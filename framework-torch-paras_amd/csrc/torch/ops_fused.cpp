@@ -13,6 +13,7 @@ using at::Tensor;
 std::tuple<Tensor, Tensor> rms_norm(const Tensor& input, const Tensor& weight, double eps) {
     TORCH_CHECK(input.dim() <= 8, "paras rms_norm: rank exceeds kernel limit");
     TORCH_CHECK(input.dim() >= 1, "paras rms_norm: input must have rank >= 1");
+    require_same_device("paras rms_norm", input, {{"weight", &weight}});
     Tensor in = input.contiguous();
     Tensor w = weight.contiguous();
     const int64_t H = in.size(-1);
@@ -29,6 +30,8 @@ std::tuple<Tensor, Tensor> rms_norm(const Tensor& input, const Tensor& weight, d
 
 std::tuple<Tensor, Tensor> rms_norm_backward(const Tensor& grad_out, const Tensor& input, const Tensor& weight,
                                              const Tensor& rstd) {
+    require_same_device("paras rms_norm_backward", input, {{"grad_out", &grad_out}, {"weight", &weight}, {"rstd", &rstd}});
+    require_same_dtype("paras rms_norm_backward", input, {{"grad_out", &grad_out}, {"weight", &weight}});
     Tensor go = grad_out.contiguous(), in = input.contiguous(), w = weight.contiguous();
     Tensor rs = rstd.contiguous();
     const int64_t H = in.size(-1);
@@ -49,6 +52,7 @@ Tensor swiglu(const Tensor& gate, const Tensor& up) {
     TORCH_CHECK(gate.sizes() == up.sizes(), "paras swiglu: gate and up must have the same shape");
     TORCH_CHECK(gate.dim() <= 8, "paras swiglu: rank exceeds kernel limit");
     TORCH_CHECK(gate.scalar_type() == up.scalar_type(), "paras swiglu: gate and up must have the same dtype");
+    require_same_device("paras swiglu", gate, {{"up", &up}});
     Tensor g = gate.contiguous(), u = up.contiguous();
     Tensor out = at::empty_like(g);
     if (out.numel() == 0) return out;
@@ -58,6 +62,8 @@ Tensor swiglu(const Tensor& gate, const Tensor& up) {
 }
 
 std::tuple<Tensor, Tensor> swiglu_backward(const Tensor& grad_out, const Tensor& gate, const Tensor& up) {
+    require_same_device("paras swiglu_backward", grad_out, {{"gate", &gate}, {"up", &up}});
+    require_same_dtype("paras swiglu_backward", grad_out, {{"gate", &gate}, {"up", &up}});
     Tensor go = grad_out.contiguous(), g = gate.contiguous(), u = up.contiguous();
     TORCH_CHECK(go.numel() == g.numel() && g.numel() == u.numel(), "paras swiglu_backward: shape mismatch");
     Tensor grad_gate = at::empty_like(g), grad_up = at::empty_like(u);
@@ -69,6 +75,7 @@ std::tuple<Tensor, Tensor> swiglu_backward(const Tensor& grad_out, const Tensor&
 
 Tensor rotate_half_impl(const Tensor& x, bool backward, const char* name) {
     TORCH_CHECK(x.dim() >= 1, "paras ", name, ": input must have rank >= 1");
+    require_same_device(name, x, {});
     TORCH_CHECK(x.dim() <= 8, "paras ", name, ": rank exceeds kernel limit");
     const int64_t D = x.size(-1);
     TORCH_CHECK(D % 2 == 0, "paras ", name, ": last dimension must be even");
@@ -85,6 +92,7 @@ Tensor rotate_half_backward(const Tensor& g) { return rotate_half_impl(g, true, 
 // ---- MoE (no reference op; composition of reference primitives) -----------------
 std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor> moe_route(const Tensor& logits, int64_t k) {
     TORCH_CHECK(logits.dim() == 2, "paras moe_route: logits must be [tokens, experts]");
+    require_same_device("paras moe_route", logits, {});
     Tensor lg = logits.contiguous();
     const int64_t T = lg.size(0), E = lg.size(1);
     TORCH_CHECK(E >= 1 && E <= 64, "paras moe_route: expert count must be in [1, 64]");
@@ -112,6 +120,12 @@ Tensor moe_ffn(const Tensor& x, const Tensor& w_gate, const Tensor& w_up, const 
                 "paras moe_ffn: routing tensors do not match T*k / E");
     TORCH_CHECK(x.scalar_type() == c10::kBFloat16 || x.scalar_type() == c10::kHalf,
                 "paras moe_ffn: dtype must be bfloat16 or float16");
+    require_same_device("paras moe_ffn", x, {{"w_gate", &w_gate}, {"w_up", &w_up}, {"w_down", &w_down}, {"topw", &topw},
+                                             {"order", &order}, {"inv_order", &inv_order}, {"offsets", &offsets}});
+    require_same_dtype("paras moe_ffn", x, {{"w_gate", &w_gate}, {"w_up", &w_up}, {"w_down", &w_down}});
+    TORCH_CHECK(topw.scalar_type() == c10::kFloat, "paras moe_ffn: topw must be float32");
+    TORCH_CHECK(order.scalar_type() == c10::kLong && inv_order.scalar_type() == c10::kLong && offsets.scalar_type() == c10::kLong,
+                "paras moe_ffn: order, inv_order and offsets must be int64");
     Tensor xc = x.contiguous(), wg = w_gate.contiguous(), wu = w_up.contiguous(), wd = w_down.contiguous();
     Tensor tw = topw.contiguous(), od = order.contiguous(), iv = inv_order.contiguous(), of = offsets.contiguous();
     Tensor out = at::empty({T, H}, xc.options());

@@ -37,6 +37,7 @@ Tensor as_nt_operand(const Tensor& mat2, bool mfma) {
 }
 
 void check_dtypes(const Tensor& a, const Tensor& b, const char* what) {
+    require_same_device(what, a, {{"mat2", &b}});
     TORCH_CHECK(a.scalar_type() == b.scalar_type(), "paras ", what, ": operand dtypes differ");
     TORCH_CHECK(is_float(a), "paras ", what, ": only float dtypes (fp32, fp64, bf16, fp16) are supported on the device");
 }
@@ -96,6 +97,7 @@ Tensor addmm(const Tensor& self, const Tensor& mat1, const Tensor& mat2, const a
     TORCH_CHECK(mat1.size(1) == mat2.size(0), "paras addmm: shapes cannot be multiplied");
     check_dtypes(mat1, mat2, "addmm");
     TORCH_CHECK(self.scalar_type() == mat1.scalar_type(), "paras addmm: operand dtypes differ");
+    require_same_device("addmm", mat1, {{"self", &self}});
     return run_gemm(mat1, mat2, self, alpha.toDouble(), beta.toDouble(), 0);
 }
 

@@ -10,6 +10,9 @@
 #include <c10/util/Exception.h>
 #include <torch/library.h>
 
+#include <initializer_list>
+#include <utility>
+
 #include "paras_hip.h"
 
 namespace paras_torch {
@@ -23,6 +26,26 @@ inline void check(int rc) {
 }
 
 inline bool is_paras(const at::Tensor& t) { return t.device().type() == kParas; }
+
+// Every tensor argument of an op must live on the same `paras` device before any of its
+// pointers reaches a kernel: the dispatcher picks the PrivateUse1 kernel as soon as ONE
+// argument is on the device, and a host pointer handed to a HIP kernel is a GPU memory
+// fault rather than an error.  Raises (RuntimeError in Python) on the host, before any launch.
+inline void require_same_device(const char* op, const at::Tensor& ref, std::initializer_list<std::pair<const char*, const at::Tensor*>> others) {
+    TORCH_CHECK(is_paras(ref), op, ": expected a tensor on a paras device, got ", ref.device());
+    for (const auto& o : others) {
+        if (o.second == nullptr || !o.second->defined()) continue;
+        TORCH_CHECK(is_paras(*o.second) && o.second->device() == ref.device(), op, ": argument `", o.first, "` is on ",
+                    o.second->device(), " but the op runs on ", ref.device(), "; move it with .to('", ref.device(), "') first");
+    }
+}
+inline void require_same_dtype(const char* op, const at::Tensor& ref, std::initializer_list<std::pair<const char*, const at::Tensor*>> others) {
+    for (const auto& o : others) {
+        if (o.second == nullptr || !o.second->defined()) continue;
+        TORCH_CHECK(o.second->scalar_type() == ref.scalar_type(), op, ": argument `", o.first, "` has dtype ", o.second->scalar_type(),
+                    ", expected ", ref.scalar_type());
+    }
+}
 
 // paras_dtype code of a floating tensor type, or -1.
 inline int float_code(c10::ScalarType t) {

@@ -104,7 +104,10 @@ Tensor copy_from(const Tensor& self, const Tensor& dst, bool non_blocking) {
             staged = empty_paras(self.sizes(), convertible ? dst.scalar_type() : self.scalar_type(), self.device());
             device_copy(self, staged);
         }
-        if (staged.scalar_type() == dst.scalar_type() && dst.is_contiguous()) {
+        // copy_() reaches this function before any broadcasting: a source of fewer elements than
+        // the destination takes the second branch, which copies staged.numel() elements and lets
+        // the host copy expand them.
+        if (staged.scalar_type() == dst.scalar_type() && dst.is_contiguous() && staged.sizes().equals(dst.sizes())) {
             check(paras_memcpy(dev, dst.data_ptr(), staged.data_ptr(), nbytes_dst, 1));
         } else {
             Tensor host = at::empty(staged.sizes(), staged.options().device(c10::kCPU));

@@ -255,7 +255,9 @@ PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 /* inv_order: [T*k] int64 (position of flat slot in `order`; may be NULL);    */
 /* counts: [E] int64; offsets: [E+1] int64.  1 <= k <= E <= 64.               */
 /* `workspace`: paras_moe_route_workspace(T,E,k) bytes of device memory        */
-/* (per-workgroup histograms).                                                 */
+/* (an arrival counter and per-workgroup expert counts; contents on entry do   */
+/* not matter).  Up to 65536 tokens the whole routing is one kernel whose      */
+/* workgroups meet at that counter.                                            */
 /* ------------------------------------------------------------------------- */
 PARAS_API size_t paras_moe_route_workspace(int64_t T, int64_t E, int64_t k);
 PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k,

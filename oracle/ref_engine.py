@@ -197,6 +197,29 @@ def time_workload(name: str, sample: dict) -> dict:
         topi, topw, order, inv, counts, offsets = moe_route(logits, k)
         moe_ffn(x, wg, wu, wd, topw, order, inv, offsets, k)
         return {"seconds": time.perf_counter() - t0}
+    if name == "linear":
+        M, N, K = sample["M"], sample["N"], sample["K"]
+        a, w = torch.randn(M, K).to(bf), (0.02 * torch.randn(N, K)).to(bf)
+        da, dw = _dev(a), _dev(w)
+        t0 = time.perf_counter()
+        torch.mm(da, dw.t()).cpu()
+        return {"seconds": time.perf_counter() - t0}
+    if name == "backward_ops":
+        rows, H, I = sample["rows"], sample["H"], sample["I"]
+        x, go, w = torch.randn(rows, H).to(bf), torch.randn(rows, H).to(bf), (1 + 0.02 * torch.randn(H)).to(bf)
+        gate, up, g2 = torch.randn(rows, I).to(bf), torch.randn(rows, I).to(bf), torch.randn(rows, I).to(bf)
+        qh = torch.randn(32 * rows, 128).to(bf)
+        dx, dgo, dw = _dev(x), _dev(go), _dev(w)
+        rstd = torch.ops.paras.rms_norm(dx, dw, 1e-6)[1]
+        dgate, dup, dg2, dqh = _dev(gate), _dev(up), _dev(g2), _dev(qh)
+        t0 = time.perf_counter()
+        torch.ops.paras.rms_norm_backward(dgo, dx, dw, rstd)
+        t1 = time.perf_counter()
+        torch.ops.paras.swiglu_backward(dg2, dgate, dup)
+        t2 = time.perf_counter()
+        torch.ops.paras.rotate_half(dqh)
+        t3 = time.perf_counter()
+        return {"seconds": t3 - t0, "rms_norm_bwd_seconds": t1 - t0, "swiglu_bwd_seconds": t2 - t1, "rotate_half_seconds": t3 - t2}
     raise ValueError(name)
 
 

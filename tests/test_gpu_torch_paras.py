@@ -658,3 +658,62 @@ def test_cat_index_select_and_embedding_on_device(device):
     assert torch.equal(F.embedding(tok.to(device) % 50, w33.to(device)).cpu(), F.embedding(tok % 50, w33))
     with pytest.raises(RuntimeError):
         torch.cat([torch.zeros(2, 3).to(device), torch.zeros(2, 4).to(device)], 0)
+
+
+# ---- arguments on the wrong device raise on the host, before any launch ------------
+def test_host_tensor_mixed_into_a_device_op_raises(device):
+    """The dispatcher picks the device kernel as soon as one argument is on the device; a host
+    pointer must never reach a HIP kernel."""
+    import torch_paras  # noqa: F401
+    bf = torch.bfloat16
+    x, w = torch.randn(8, 64).to(bf), torch.randn(64).to(bf)
+    dx, dw = x.to(device), w.to(device)
+    cases = [
+        lambda: torch.mm(dx, torch.randn(64, 16).to(bf)),
+        lambda: torch.bmm(dx[None], torch.randn(1, 64, 16).to(bf)),
+        lambda: torch.addmm(torch.randn(16).to(bf), dx, torch.randn(64, 16).to(bf).to(device)),
+        lambda: torch.ops.paras.rms_norm(dx, w, 1e-6),
+        lambda: torch.ops.paras.rms_norm_backward(dx, dx, w, torch.ones(8).to(device)),
+        lambda: torch.ops.paras.rms_norm_backward(dx, dx, dw, torch.ones(8)),
+        lambda: torch.ops.paras.swiglu(dx, x),
+        lambda: torch.ops.paras.swiglu_backward(dx, x, dx),
+        lambda: torch.ops.aten.rms_norm(dx, [64], w, 1e-6),
+        lambda: torch.ops.torch_paras.swiglu(dx, x),
+        lambda: torch.ops.aten._scaled_dot_product_attention_math(dx.view(1, 1, 8, 64), x.view(1, 1, 8, 64), dx.view(1, 1, 8, 64)),
+        lambda: F.scaled_dot_product_attention(dx.view(1, 1, 8, 64), dx.view(1, 1, 8, 64), x.view(1, 1, 8, 64)),
+    ]
+    for i, fn in enumerate(cases):
+        with pytest.raises(RuntimeError):
+            fn()
+            pytest.fail(f"case {i} did not raise")
+    # MoE: weights on the host, and weights of another dtype than x
+    T, E, k, H, I = 16, 2, 1, 64, 64
+    xm = torch.randn(T, H).to(bf).to(device)
+    route = torch.ops.paras.moe_route(torch.randn(T, E).to(bf).to(device), k)
+    wg = torch.randn(E, I, H).to(bf)
+    wd = torch.randn(E, H, I).to(bf)
+    with pytest.raises(RuntimeError):
+        torch.ops.paras.moe_ffn(xm, wg, wg.to(device), wd.to(device), route[1], route[2], route[3], route[5], k)
+    with pytest.raises(RuntimeError, match="dtype"):
+        torch.ops.paras.moe_ffn(xm, wg.float().to(device), wg.to(device), wd.to(device), route[1], route[2], route[3], route[5], k)
+
+
+def test_sdpa_fused_path_honours_enable_gqa(device):
+    """Fewer key/value heads without enable_gqa fail as in the reference (its matmul cannot
+    broadcast 8 heads against 2); with the flag the fused op maps the heads."""
+    q, k = torch.randn(1, 8, 16, 64).bfloat16().to(device), torch.randn(1, 2, 16, 64).bfloat16().to(device)
+    with pytest.raises(RuntimeError):
+        F.scaled_dot_product_attention(q, k, k, enable_gqa=False)
+    out = F.scaled_dot_product_attention(q, k, k, enable_gqa=True)
+    ref = F.scaled_dot_product_attention(q.cpu().float(), k.cpu().float(), k.cpu().float(), enable_gqa=True)
+    assert (out.cpu().float() - ref).abs().max().item() <= 2e-2
+
+
+def test_device_to_host_copy_broadcasts(device):
+    src = torch.randn(5)
+    dst = torch.zeros(3, 5)
+    dst.copy_(src.to(device))
+    assert torch.equal(dst, src.expand(3, 5))
+    dst16 = torch.zeros(3, 5, dtype=torch.bfloat16)
+    dst16.copy_(src.to(device))
+    assert torch.equal(dst16, src.bfloat16().expand(3, 5))
