@@ -30,6 +30,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <mutex>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
@@ -403,6 +404,34 @@ size_t route_scratch_bytes(long T_, long E) {
     return static_cast<size_t>(kScratchHeader) + static_cast<size_t>(nblk * E) * sizeof(int);
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Scratch of the allocation-free entry point: one copy per GPU, held until the process ends.
+// Its name is a host-side stand-in, not a device address: host code only ever uses the
+// per-device address hipGetSymbolAddress returns (static_scratch_for below).
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(kScratchHeader) + static_cast<size_t>(kFusedMaxBlocks) * kMaxExperts * sizeof(int);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxGpus = 64;
+std::mutex g_scratch_mutex;
+unsigned char* g_scratch_ptr[kMaxGpus] = {};
+
+// Address of `scratch` on the calling thread's current device, resolved once per device.
+int static_scratch_for(unsigned char** out) {
+    int dev = -1;
+    PARAS_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxGpus) return fail(PARAS_ERR_UNSUPPORTED, "paras_moe_route_noalloc: device index %d beyond %d", dev, kMaxGpus);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        PARAS_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) return fail(PARAS_ERR_HIP, "paras_moe_route_noalloc: no device address for the scratch array");
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return PARAS_OK;
+}
+
 }  // namespace
 }  // namespace paras
 
@@ -465,6 +494,29 @@ int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dty
                        reinterpret_cast<long*>(order), reinterpret_cast<long*>(inv_order));
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
+}
+
+int paras_moe_route_noalloc(const void* logits, int64_t T, int64_t E, int64_t k, int dtype, int64_t* topi,
+                            float* topw, int64_t* order, int64_t* inv_order, int64_t* counts, int64_t* offsets,
+                            void* stream) {
+    using namespace paras;
+    PARAS_REQUIRE(T >= 1, "paras_moe_route_noalloc: at least one token is required");
+    PARAS_REQUIRE(T <= kFusedMaxTokens, "paras_moe_route_noalloc: %lld tokens exceed the static scratch (at most %ld tokens)",
+                  static_cast<long long>(T), kFusedMaxTokens);
+    PARAS_REQUIRE(E >= 1 && E <= kMaxExperts, "paras_moe_route_noalloc: expert count must be in [1, %d]", kMaxExperts);
+    PARAS_REQUIRE(k >= 1 && k <= E, "paras topk: k out of range");
+    PARAS_REQUIRE(T * k <= 0x7fffffffL, "paras_moe_route_noalloc: too many routed rows");
+    PARAS_REQUIRE(logits && topi && topw && order && counts && offsets, "paras_moe_route_noalloc: null pointer");
+    hipStream_t s = nullptr;
+    int rc = resolve_stream(stream, &s);
+    if (rc != PARAS_OK) return rc;
+    unsigned char* ptr = nullptr;
+    rc = static_scratch_for(&ptr);
+    if (rc != PARAS_OK) return rc;
+    // The counter in the scratch header is cleared by the fill kernel route_on queues first;
+    // the per-workgroup counts behind it are rewritten before they are read.
+    return route_on(logits, T, (int)E, (int)k, dtype, reinterpret_cast<long*>(topi), topw, reinterpret_cast<long*>(order),
+                    reinterpret_cast<long*>(inv_order), reinterpret_cast<long*>(counts), reinterpret_cast<long*>(offsets), ptr, s);
 }
 
 }  // extern "C"

@@ -265,6 +265,20 @@ PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t 
                               int64_t* inv_order, int64_t* counts, int64_t* offsets,
                               void* workspace, void* stream);
 
+/* paras_moe_route for callers that cannot allocate (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and same outputs, bit for bit,
+ * without the workspace: the per-workgroup counts and the arrival counter live
+ * in a fixed array in the library's device image (65,792 bytes per GPU, held
+ * until the process ends).  Limits: 1 <= T <= 65536 tokens, E <= 64; larger
+ * inputs are PARAS_ERR_INVALID.  The call allocates nothing and frees nothing.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU
+ * (two streams, two threads) race; calls queued on one stream do not. */
+PARAS_API int paras_moe_route_noalloc(const void* logits, int64_t T, int64_t E, int64_t k,
+                                      int dtype, int64_t* topi, float* topw, int64_t* order,
+                                      int64_t* inv_order, int64_t* counts, int64_t* offsets,
+                                      void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* MoE grouped expert FFN with SwiGLU.  Per routed row p (expert e):          */
 /*   xp = x[order[p] / k]                                   (index_select,    */

@@ -60,6 +60,7 @@ SIGNATURES = {
     "paras_sdpa_kernel_name": (C.c_char_p, [C.POINTER(SdpaArgs)]),
     "paras_moe_route_workspace": (sz, [i64, i64, i64]),
     "paras_moe_route": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp]),
+    "paras_moe_route_noalloc": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp]),
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
     "paras_index_select": (i32, [vp, vp, vp, i64, i64, i64, i64, vp]),
@@ -212,6 +213,21 @@ def moe_route(logits, k):
     check(lib().paras_moe_route(_ptr(logits), T, E, k, DT[logits.dtype], _ptr(topi), _ptr(topw), _ptr(order),
                                 _ptr(inv), _ptr(counts), _ptr(offsets), _ptr(ws), _stream()))
     return topi, topw, order, inv, counts, offsets
+
+
+def moe_route_noalloc(logits, k, out=None):
+    """paras_moe_route_noalloc: the outputs are allocated here, before the call, by the caller."""
+    logits = logits.contiguous()
+    T, E = logits.shape
+    dev = logits.device
+    if out is None:
+        out = (torch.empty(T, k, dtype=torch.int64, device=dev), torch.empty(T, k, dtype=torch.float32, device=dev),
+               torch.empty(T * k, dtype=torch.int64, device=dev), torch.empty(T * k, dtype=torch.int64, device=dev),
+               torch.empty(E, dtype=torch.int64, device=dev), torch.empty(E + 1, dtype=torch.int64, device=dev))
+    topi, topw, order, inv, counts, offsets = out
+    check(lib().paras_moe_route_noalloc(_ptr(logits), T, E, k, DT[logits.dtype], _ptr(topi), _ptr(topw), _ptr(order),
+                                        _ptr(inv), _ptr(counts), _ptr(offsets), _stream()))
+    return out
 
 
 def moe_ffn(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, k, workspace=None):
