@@ -134,6 +134,17 @@ __device__ __forceinline__ float wave_max(float v) {
     return wave_allreduce(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
+// ---- workgroup barrier for LDS traffic only -----------------------------------
+// __syncthreads() carries a release fence over every address space: the wave waits for all of
+// its global loads and stores in flight before it meets the others, which serialises a loop that
+// requested the next row from memory before reducing the current one.  This barrier orders LDS
+// accesses only (s_waitcnt lgkmcnt(0); s_barrier): use it where the data exchanged lives in LDS.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---- 16-byte global access ---------------------------------------------------
 __device__ __forceinline__ u32x4 load16(const void* p) {
     return *reinterpret_cast<const u32x4*>(p);

@@ -15,6 +15,8 @@
 // bit-identical to the host engine's.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
@@ -220,13 +222,24 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_final(
 
 // 16-bit tensors with 16-byte aligned rows of at most BLOCK*NV vectors: dx and the partial
 // column sums in ONE pass over grad_out and x.  A workgroup owns a slab of kDwSlabRows rows; each
-// thread keeps the same NV vectors of every row (and of w), so its 8*NV column sums live in
-// registers across the slab, and the next row's vectors are requested before the current row's
-// reduction (two rows ahead: no change).  Arithmetic in fp64 in the host's order of operations.  One vector per thread needs
-// 96 registers (five waves per SIMD), two need 136-144 (three): rows are spread over 256, 512 or
-// 1024 threads with one vector each (4096-element rows: 98.7 us with 256 x 2, 93.3 us with 512 x 1).
-template <typename T, int NV, int BLOCK>
-__global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? (BLOCK == 1024 ? 4 : 2) : 4)) void rms_norm_bwd_fused(
+// thread keeps the same NV vectors of every row (and of w, as doubles), so its 8*NV column sums
+// live in registers across the slab, and the next row's vectors are requested before the current
+// row's reduction.  Arithmetic in fp64, arranged so that every product that is exact on the host
+// is exact here and every rounding the host makes is made here:
+//   q = g*x (16-bit significands: exact), dot += q*w and dw += q*rstd (fma: the products are
+//   exact in fp64 -- at most 40 significant bits -- so only the additions round, as on the host);
+//   grad_x = fma(g*w, rstd, -(x * (coef*dot))): g*w*rstd is exact, so the one rounding of the
+//   fma is the host's rounding of the difference; x*(coef*dot) differs from the host's
+//   (coef*x)*dot in the last bit of a double at most, like the dot product's summation order.
+// The result is narrowed double -> float -> T with the conversion instructions (two roundings to
+// nearest even, as on the host); a vector in which a NaN turns up is narrowed again in software,
+// which canonicalises NaNs the way the host's types do.
+// One vector per thread needs ~100 registers: rows are spread over 256, 512 or 1024 threads.
+// kFull: every thread of the workgroup owns a vector (H == 8 * BLOCK * NV).  Then no memory
+// instruction sits under a lane mask and the compiler can count exactly which of them a wait has
+// to cover: with a mask it waits, before the next row, for the row's own store as well.
+template <typename T, int NV, int BLOCK, bool kFull>
+__global__ __launch_bounds__(BLOCK, 4) void rms_norm_bwd_fused(
     const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
     const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H,
     int slab_rows) {
@@ -238,75 +251,118 @@ __global__ __launch_bounds__(BLOCK, (BLOCK > 256 ? (BLOCK == 1024 ? 4 : 2) : 4))
     const long slab = blockIdx.x;
     const long r0 = slab * slab_rows;
     const long r1 = r0 + slab_rows < rows ? r0 + slab_rows : rows;
+    const double inv_h = 1.0 / static_cast<double>(H);   // only used where H is a power of two (exact)
+    const bool h_pow2 = __builtin_amdgcn_readfirstlane((H & (H - 1)) == 0) != 0;
     bool have[NV];
-    u32x4 wv[NV], gv[NV], xv[NV], gn[NV], xn[NV];
-    double dw[NV][V];
+    // One register set of row vectors: as soon as a row has been widened to doubles, the next row
+    // is requested into the same registers (no copies between rows, and the loads have the row's
+    // reduction, second half and store to arrive).
+    u32x4 gs[NV], xs[NV];
+    double w64[NV][V], dw[NV][V];
+    auto request = [&](long r) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (have[i]) {
+                const int c = threadIdx.x + i * BLOCK;
+                gs[i] = load16_nt(go + r * H + static_cast<long>(c) * V);
+                xs[i] = load16_nt(x + r * H + static_cast<long>(c) * V);
+            }
+    };
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int c = threadIdx.x + i * BLOCK;
-        have[i] = c < nvec;
-        if (have[i]) {
-            wv[i] = load16(w + static_cast<long>(c) * V);
-            gn[i] = load16_nt(go + r0 * H + static_cast<long>(c) * V);
-            xn[i] = load16_nt(x + r0 * H + static_cast<long>(c) * V);
-        }
+        have[i] = kFull || c < nvec;
+        u32x4 wv = {0u, 0u, 0u, 0u};
+        if (have[i]) wv = load16(w + static_cast<long>(c) * V);
+        const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv);
 #pragma unroll
-        for (int j = 0; j < V; ++j) dw[i][j] = 0.0;
+        for (int j = 0; j < V; ++j) {
+            w64[i][j] = E::to_f64(we[j]);
+            dw[i][j] = 0.0;
+        }
     }
+    request(r0);
     int sum_calls = 0;
-    for (long r = r0; r < r1; ++r) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            gv[i] = gn[i];
-            xv[i] = xn[i];
-            if (have[i] && r + 1 < r1) {
-                const int c = threadIdx.x + i * BLOCK;
-                gn[i] = load16_nt(go + (r + 1) * H + static_cast<long>(c) * V);
-                xn[i] = load16_nt(x + (r + 1) * H + static_cast<long>(c) * V);
-            }
-        }
-        const double rr = static_cast<double>(rstd[r]);
+    float rstd_next = rstd[r0];
+    auto do_row = [&](long r) __attribute__((always_inline)) {
+        const float rstd_now = rstd_next;
+        if (r + 1 < r1) rstd_next = rstd[r + 1];     // requested a row ahead
+        const double rr = static_cast<double>(rstd_now);
         double dot = 0.0;
-        // g*w and x as doubles stay in registers for the second half of the row (the register
-        // budget of two 512-thread workgroups per CU has room for them; converting and
-        // multiplying again costs a fifth of the row's fp64 instructions).
-        double gwd[NV][V], xd[NV][V];
+        double g64[NV][V], x64[NV][V];     // stay in registers for the second half of the row
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i]) {
-                const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gv[i]);
-                const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xv[i]);
-                const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
+                const std::uint16_t* ge = reinterpret_cast<const std::uint16_t*>(&gs[i]);
+                const std::uint16_t* xe = reinterpret_cast<const std::uint16_t*>(&xs[i]);
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
-                    const double g = E::to_f64(ge[j]);
-                    xd[i][j] = E::to_f64(xe[j]);
-                    gwd[i][j] = g * E::to_f64(we[j]);
-                    dot += gwd[i][j] * xd[i][j];
-                    dw[i][j] += g * xd[i][j] * rr;
+                    g64[i][j] = E::to_f64(ge[j]);
+                    x64[i][j] = E::to_f64(xe[j]);
+                    const double q = g64[i][j] * x64[i][j];
+                    dot = fma(q, w64[i][j], dot);
+                    dw[i][j] = fma(q, rr, dw[i][j]);
                 }
             }
+        if (r + 1 < r1) request(r + 1);
         {   // sum over the workgroup; two alternating slot sets, so one barrier per row
             dot = wave_sum(dot);
-            double* set = slots + (sum_calls++ & 1) * kWaves;
-            if ((threadIdx.x & (kWave - 1)) == 0) set[threadIdx.x / kWave] = dot;
-            __syncthreads();
+            double* slot = slots + (sum_calls++ & 1) * kWaves;
+            if ((threadIdx.x & (kWave - 1)) == 0) slot[threadIdx.x / kWave] = dot;
+            lds_barrier();   // not __syncthreads(): the loads requested above stay in flight across it
             dot = 0.0;
 #pragma unroll
-            for (int i = 0; i < kWaves; ++i) dot += set[i];
+            for (int i = 0; i < kWaves; ++i) dot += slot[i];
         }
-        const double coef = rr * rr * rr / static_cast<double>(H);
+        // (rstd^3 / H as the host forms it; the division is a multiplication when H is a power of two)
+        double coef = rr * rr * rr;
+        if (h_pow2) {
+            coef *= inv_h;
+        } else {
+            asm volatile("" ::: "memory");           // keeps the division out of the power-of-two path
+            coef = coef / static_cast<double>(H);
+        }
+        const double cd = coef * dot;
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i]) {
-                u32x4 o;
-                std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+                float y[V];
+                float nan_probe = 0.0f;
 #pragma unroll
-                for (int j = 0; j < V; ++j)
-                    oe[j] = E::from_f64(gwd[i][j] * rr - coef * xd[i][j] * dot);
+                for (int j = 0; j < V; ++j) {
+                    const double y64 = fma(g64[i][j] * w64[i][j], rr, -(x64[i][j] * cd));
+                    y[j] = static_cast<float>(y64);
+                    nan_probe += y[j];
+                }
+                u32x4 o;
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    if constexpr (__is_same(T, bf16_t)) {
+                        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                        o[p] = __builtin_bit_cast(std::uint32_t, __builtin_convertvector((f32x2){y[2 * p], y[2 * p + 1]}, bf16x2));
+                    } else {
+                        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+                        o[p] = __builtin_bit_cast(std::uint32_t, __builtin_convertvector((f32x2){y[2 * p], y[2 * p + 1]}, f16x2));
+                    }
+                }
+                // (a wave-uniform test, so that the software narrowing stays behind a branch instead of
+                // being evaluated for every vector and selected away)
+                if (__builtin_amdgcn_ballot_w64(nan_probe != nan_probe) != 0) {   // a NaN (or infinities of both signs) in some lane's vector
+                    asm volatile("" ::: "memory");           // not to be evaluated ahead of the branch
+                    std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) oe[j] = E::from_f32(y[j]);
+                }
                 store16_nt(gx + r * H + static_cast<long>(threadIdx.x + i * BLOCK) * V, o);
             }
-    }
+    };
+    // The first row is written out in front of the loop: entered straight from the prologue, the
+    // loop header would inherit "first loads pending" and the compiler's wait insertion would then
+    // make every trip wait for all memory traffic in flight, the previous row's store included;
+    // after a peeled row both ways into the header look alike (a row requested, a store in flight).
+    do_row(r0);
+    for (long r = r0 + 1; r < r1; ++r) do_row(r);
 #pragma unroll
     for (int i = 0; i < NV; ++i)
         if (have[i]) {
@@ -398,12 +454,15 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
                 slabs = (rows + slab_rows - 1) / slab_rows;
             }
             const dim3 grid(static_cast<unsigned>(slabs));
-            if (nvec <= kBlock)
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, kBlock>), grid, dim3(kBlock), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H, slab_rows);
-            else if (nvec <= 512)
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, 512>), grid, dim3(512), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H, slab_rows);
-            else   // rows of up to 8192 elements
-                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, 1024>), grid, dim3(1024), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H, slab_rows);
+#define PARAS_BWD_LAUNCH(BLOCK_, FULL_) \
+    hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, FULL_>), grid, dim3(BLOCK_), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H, slab_rows)
+            if (nvec == kBlock)      PARAS_BWD_LAUNCH(kBlock, true);
+            else if (nvec < kBlock)  PARAS_BWD_LAUNCH(kBlock, false);
+            else if (nvec == 512)    PARAS_BWD_LAUNCH(512, true);
+            else if (nvec < 512)     PARAS_BWD_LAUNCH(512, false);
+            else if (nvec == 1024)   PARAS_BWD_LAUNCH(1024, true);   // rows of up to 8192 elements
+            else                     PARAS_BWD_LAUNCH(1024, false);
+#undef PARAS_BWD_LAUNCH
             PARAS_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + kDwFinalCols - 1) / kDwFinalCols)), dim3(kDwFinalLanes * kDwFinalCols), 0, s,
                                part, static_cast<S*>(gw), slabs, H);

@@ -171,6 +171,35 @@ def test_rms_norm_backward_many_rows_uses_taller_slabs():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rms_norm_backward_adversarial_magnitudes(dtype):
+    """The one-pass backward on rows built to break a shortcut in its arithmetic: products g*w and
+    g*x far below / above the fp32 range (bf16), subnormal results, a huge rstd (eps = 0 on a tiny
+    row), rows of zeros and signed zeros, grad_x terms that cancel almost completely, and NaN / inf
+    entries.  Bit for bit against the oracle; NaNs compare as NaNs."""
+    torch.manual_seed(23)
+    rows, H = 48, 1024
+    big = 1e30 if dtype == torch.bfloat16 else 3e4
+    tiny = 1e-30 if dtype == torch.bfloat16 else 1e-6
+    x, go = torch.randn(rows, H), torch.randn(rows, H)
+    w = 1 + 0.1 * torch.randn(H)
+    go[0] *= tiny; x[1] *= tiny; go[2] *= tiny; x[2] *= tiny          # underflowing products
+    go[3] *= big; x[4] *= big                                         # overflowing products (fp32), finite in fp64
+    go[5] = 0.0; go[6] = -0.0; x[7] = 0.0; x[8, ::2] = 0.0; go[8, 1::2] = -0.0
+    go[9] = x[9] * 3.0                                                # grad_out parallel to x: the two terms cancel
+    go[10] = x[10]
+    go[11, 5] = float("nan"); x[12, 7] = float("inf"); go[13, 3] = float("-inf"); go[13, 4] = float("inf")
+    x[14] *= 1e-3; x[15] *= 250.0
+    w[17] = 0.0; w[18] = -0.0; w[19] = tiny; w[20] = 200.0
+    x, go, w = x.to(dtype), go.to(dtype), w.to(dtype)
+    for eps in (1e-6, 0.0):
+        _, rstd = O.rms_norm(x, w, eps)
+        gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(rstd))
+        wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
+        assert_bit_exact(gx, wgx, f"rms_norm grad_input eps={eps}")
+        assert_bit_exact(gw, wgw, f"rms_norm grad_weight eps={eps}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_rotate_half_vector_path_and_fallbacks(dtype):
     for shape in [(3, 5, 128), (7, 64), (2, 16), (4, 48), (3, 24), (5, 130)]:
         xr = torch.randn(*shape).to(dtype)
