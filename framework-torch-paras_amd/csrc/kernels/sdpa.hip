@@ -12,7 +12,7 @@
 namespace paras {
 namespace {
 
-enum class SdpaKernel { Flash, Decode, Generic };
+enum class SdpaKernel { Flash, Decode, Weights, Generic };
 
 int validate(const paras_sdpa_args* a) {
     PARAS_REQUIRE(a != nullptr, "paras sdpa: null argument block");
@@ -34,6 +34,7 @@ bool empty_output(const paras_sdpa_args& a) { return a.B == 0 || a.Hq == 0 || a.
 SdpaKernel choose(const paras_sdpa_args& a) {
     if (decode_supported(a)) return SdpaKernel::Decode;
     if (flash_supported(a)) return SdpaKernel::Flash;
+    if (weights_supported(a)) return SdpaKernel::Weights;
     return SdpaKernel::Generic;
 }
 
@@ -48,6 +49,7 @@ const char* paras_sdpa_kernel_name(const paras_sdpa_args* args) {
     switch (choose(*args)) {
         case SdpaKernel::Flash:  return "flash_mfma";
         case SdpaKernel::Decode: return "decode_split";
+        case SdpaKernel::Weights: return "math_mfma";
         default:                 return "generic";
     }
 }
@@ -81,6 +83,7 @@ int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream) {
     }
     switch (choose(a)) {
         case SdpaKernel::Flash: return launch_flash(a, s);
+        case SdpaKernel::Weights: return launch_weights(a, s);
         case SdpaKernel::Decode:
             PARAS_REQUIRE(workspace != nullptr || decode_workspace(a) == 0, "paras sdpa: workspace is null");
             return launch_decode(a, workspace, s);

@@ -1,4 +1,4 @@
-// Launchers of the three attention kernels; the C ABI entry point in sdpa.hip
+// Launchers of the attention kernels; the C ABI entry point in sdpa.hip
 // validates the request, picks one of them and calls it.
 #pragma once
 
@@ -19,7 +19,12 @@ bool   decode_supported(const paras_sdpa_args& a);
 size_t decode_workspace(const paras_sdpa_args& a);
 int    launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s);
 
-// Everything else (fp32/fp64, any head size, bool/additive masks, weights).
+// MFMA attention that also returns the softmax weights (the math op): bf16/f16,
+// D == Dv in {64, 128}, causal / bool / additive masks contiguous along the keys.
+bool weights_supported(const paras_sdpa_args& a);
+int  launch_weights(const paras_sdpa_args& a, hipStream_t s);
+
+// Everything else (fp32/fp64, any head size, other layouts).
 size_t generic_workspace(const paras_sdpa_args& a);
 int    launch_generic(const paras_sdpa_args& a, void* workspace, hipStream_t s);
 

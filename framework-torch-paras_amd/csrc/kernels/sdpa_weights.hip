@@ -1,0 +1,377 @@
+// Attention with returned weights on the matrix cores (bf16 / fp16): the math op
+// aten::_scaled_dot_product_attention_math must hand back softmax(q k^T * scale + mask)
+// as a tensor (csrc/ops/attention_ops.cpp:128-135), which a flash kernel never forms.
+//
+// This kernel forms it, narrowing exactly where the reference's composition narrows:
+//   s1 = T(q k^T)            fp32 accumulation on MFMA, one rounding     (bmm, vision_ops.cpp:398-406)
+//   s2 = T(s1 * scale)       evaluated in double like the host's mul_out  (pointwise_ops.cpp:280-284)
+//   s3 = masked_fill(-inf) / T(s2 + mask)                                (attention_ops.cpp:103-125)
+//   w  = T(exp(s3 - max) / sum)   row max and row sum over the NARROWED scores (softmax_out, :959-976)
+//   out = T(w v)             the narrowed weights are the operand of the second product (attention_ops.cpp:134)
+// so the weights differ from the reference's only where fp32 instead of fp64 softmax arithmetic
+// lands on the other side of a rounding boundary (one unit in the last place of T, for about one
+// weight in a thousand), and `out` differs by the accumulation order of the products.
+//
+// Two passes over the keys per block of 128 queries (4 wavefronts x 32 queries, a lane owns a
+// query as in the flash kernel: S^T = K Q^T on v_mfma_f32_32x32x16, O^T = V^T W^T):
+//   pass 1   scores tile by tile, running row max and row sum (each lane over its own half of the
+//            keys; the two halves of a query are merged once at the end)
+//   pass 2   scores again, weights written to `attn`, and the product with V accumulated
+// K / V tiles of 64 keys go global -> registers -> LDS (one buffer each, two barriers per tile:
+// this path feeds callers that ask for O(Lq Lk) output, its time is dominated by writing it).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+#include "kernels/sdpa_internal.h"
+
+namespace paras {
+namespace {
+
+constexpr int kBN = 64;    // keys per tile
+constexpr int kBM = 128;   // queries per workgroup: 4 waves x 32
+
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
+
+struct WeightsParams {
+    const std::uint16_t* q;
+    const std::uint16_t* k;
+    const std::uint16_t* v;
+    std::uint16_t*       out;
+    std::uint16_t*       attn;
+    float*               lse;
+    long qs_b, qs_h, qs_l;  // element strides
+    long ks_b, ks_h, ks_l;
+    long vs_b, vs_h, vs_l;
+    int  B, Hq, Hkv, Lq, Lk;
+    int  n_qblocks;
+    double scale;           // multiplies T(q k^T) in double, as the host engine's mul_out does
+    const unsigned char* mask;
+    long ms_b, ms_h, ms_q;  // element strides (0 = broadcast); the key stride is 1
+};
+
+template <typename T> struct Mma16;
+template <> struct Mma16<bf16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma16<f16_t> {
+    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+// v_permlane32_swap exchanges lanes 32..63 of its first register with lanes 0..31 of its second:
+// fed the same value twice, every lane ends up with the lower half's value in `lo` and the upper
+// half's in `hi`.  (Inline asm with the wait states spelled out: see the flash kernel.)
+__device__ __forceinline__ void halves(float x, float& lo, float& hi) {
+    float a = x, b = x;
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    lo = a;
+    hi = b;
+}
+
+// kMode: 0 no mask, 1 bool mask bytes (nonzero = attend), 2 additive mask of type T, 3 causal.
+template <typename T, int D, int kMode>
+__global__ __launch_bounds__(256, 2) void weights_fwd_kernel(const WeightsParams p) {
+    using El = Elem<T>;
+    constexpr int NW = 4;
+    constexpr int KSTEPS = D / 16;
+    constexpr int DBLK = D / 32;
+    constexpr int CHUNKS = D / 8;          // 16-byte chunks per row
+    constexpr int RPI = 64 / CHUNKS;       // rows one wave moves per instruction
+    constexpr int NI = kBN / (RPI * NW);
+    auto ksw = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto vsw = [](int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds[kBN * D];
+
+    const int nq = p.n_qblocks;
+    const int bh = blockIdx.x / nq, qblock = nq - 1 - blockIdx.x % nq;   // heaviest causal blocks first
+    const int b = bh / p.Hq, hq = bh % p.Hq;
+    const int hkv = hq / (p.Hq / p.Hkv);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lq = lane & 31, lh = lane >> 5;
+    const int q0 = qblock * kBM + wave * 32;
+    const int my_q = q0 + lq;
+    const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
+
+    i16x8 qreg[KSTEPS];
+    {
+        const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) qreg[ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
+    }
+    const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
+    const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
+
+    int n_tiles = (p.Lk + kBN - 1) / kBN;
+    if (kMode == 3) {   // keys beyond the workgroup's last query carry zero weight: written as zeros below, not computed
+        const int last_q = min(qblock * kBM + kBM, p.Lq) - 1;
+        n_tiles = (min(last_q + 1, p.Lk) + kBN - 1) / kBN;
+    }
+
+    // staging: 64 rows of K (and V), 16 bytes per thread and step, rows past Lk as zeros; the 16-byte
+    // chunks of a row are XOR-swizzled so that operand reads and transposed reads are conflict free
+    const int srow = wave * RPI + lane / CHUNKS, slot = lane % CHUNKS;
+    auto stage = [&](const std::uint16_t* base, long row_stride, int first, std::uint16_t* tile, bool is_v) {
+        u32x4 regs[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int row = first + i * RPI * NW + srow;
+            regs[i] = u32x4{0u, 0u, 0u, 0u};
+            if (row < p.Lk) regs[i] = load16(base + static_cast<long>(row) * row_stride + slot * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int r = i * RPI * NW + srow;
+            const int sw = is_v ? vsw(r) : ksw(r);
+            *reinterpret_cast<u32x4*>(tile + r * D + ((slot ^ sw) * 8)) = regs[i];
+        }
+    };
+
+    const int grp = lane >> 4, m16 = lane & 15;
+    int k_rd[KSTEPS], v_rd[DBLK];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) k_rd[ks] = lq * D + (((2 * ks + lh) ^ ksw(lq)) * 8);
+    {
+        const int vrow = 4 * lh + (m16 >> 2);
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+            v_rd[db] = vrow * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
+    }
+
+    const unsigned char* mrow = nullptr;
+    if constexpr (kMode == 1 || kMode == 2)
+        mrow = p.mask + (static_cast<long>(b) * p.ms_b + static_cast<long>(hq) * p.ms_h + static_cast<long>(qrow) * p.ms_q) * (kMode == 1 ? 1 : 2);
+
+    // Narrowed, scaled and masked scores of one 32-key block (block `jb` of the staged tile,
+    // first key `key0`): accumulator register r of lane (query lq, half lh) is key
+    // key0 + (r/4)*8 + 4*lh + r%4.
+    auto scores = [&](int jb, int key0, float16_t& sc) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks)
+            sc = Mma16<T>::run(*reinterpret_cast<const i16x8*>(&k_lds[jb * 32 * D + k_rd[ks]]), qreg[ks], sc);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
+            float s = El::to_f32(El::from_f32(sc[r]));                 // T(q k^T)
+            s = El::to_f32(El::from_f64(static_cast<double>(s) * p.scale));   // T(s1 * scale), evaluated in double
+            bool dead = key >= p.Lk;
+            if constexpr (kMode == 3) dead = dead || key > my_q;
+            if constexpr (kMode == 1) dead = dead || (key < p.Lk && mrow[key] == 0);
+            if constexpr (kMode == 2) {
+                if (key < p.Lk) {
+                    const float m = El::to_f32(*reinterpret_cast<const std::uint16_t*>(mrow + 2 * static_cast<long>(key)));
+                    s = El::to_f32(El::from_f32(s + m));               // T(s2 + mask)
+                }
+            }
+            sc[r] = dead ? -INFINITY : s;
+        }
+    };
+
+    // ---- pass 1: row max and row sum of exp over the narrowed scores
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int t = 0; t < n_tiles; ++t) {
+        stage(kbase, p.ks_l, t * kBN, k_lds, false);
+        __syncthreads();
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) {
+            const int key0 = t * kBN + jb * 32;
+            if (key0 >= p.Lk || (kMode == 3 && key0 > q0 + 31)) continue;   // wave-uniform
+            float16_t sc;
+            scores(jb, key0, sc);
+            float mx = sc[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+            const float m_new = fmaxf(m_run, mx);
+            if (m_new != -INFINITY) {
+                float add = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) add += __expf(sc[r] - m_new);
+                l_run = (m_run == -INFINITY ? 0.f : l_run * __expf(m_run - m_new)) + add;
+                m_run = m_new;
+            }
+        }
+        __syncthreads();
+    }
+    {   // merge the two halves of each query
+        float m_lo, m_hi, l_lo, l_hi;
+        halves(m_run, m_lo, m_hi);
+        halves(l_run, l_lo, l_hi);
+        const float m_all = fmaxf(m_lo, m_hi);
+        float l_all = 0.f;
+        if (m_all != -INFINITY) {
+            if (m_lo != -INFINITY) l_all += l_lo * __expf(m_lo - m_all);
+            if (m_hi != -INFINITY) l_all += l_hi * __expf(m_hi - m_all);
+        }
+        m_run = m_all;
+        l_run = l_all;
+    }
+    // A row without a visible key: max = -inf, every exp(-inf - -inf) is NaN, as in the reference's softmax.
+    const float inv_l = 1.0f / l_run;
+
+    // ---- pass 2: weights out, product with V
+    float16_t oacc[DBLK];
+#pragma unroll
+    for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    std::uint16_t* arow = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + qrow) * p.Lk;
+    const bool row_live = my_q < p.Lq;
+    const bool wide = (p.Lk % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.attn) & 7) == 0);   // 8-byte runs of four weights
+    for (int t = 0; t < n_tiles; ++t) {
+        stage(kbase, p.ks_l, t * kBN, k_lds, false);
+        stage(vbase, p.vs_l, t * kBN, v_lds, true);
+        __syncthreads();
+#pragma unroll
+        for (int jb = 0; jb < 2; ++jb) {
+            const int key0 = t * kBN + jb * 32;
+            if (key0 >= p.Lk) continue;
+            const bool skipped = kMode == 3 && key0 > q0 + 31;   // wave-uniform: this wave's queries see none of these keys
+            float16_t sc;
+            std::uint32_t pw[8];
+            if (!skipped) {
+                scores(jb, key0, sc);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float w0 = __expf(sc[2 * i] - m_run) * inv_l, w1 = __expf(sc[2 * i + 1] - m_run) * inv_l;
+                    pw[i] = static_cast<std::uint32_t>(El::from_f32(w0)) | (static_cast<std::uint32_t>(El::from_f32(w1)) << 16);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pw[i] = 0u;
+            }
+            if (row_live) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int key = key0 + g * 8 + 4 * lh;
+                    if (wide && key + 3 < p.Lk) {
+                        *reinterpret_cast<u32x2*>(arow + key) = u32x2{pw[2 * g], pw[2 * g + 1]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (key + e < p.Lk) arow[key + e] = static_cast<std::uint16_t>(pw[2 * g + (e >> 1)] >> (16 * (e & 1)));
+                    }
+                }
+            }
+            if (!skipped) {
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                    const u32x4 pv = {pw[4 * s2], pw[4 * s2 + 1], pw[4 * s2 + 2], pw[4 * s2 + 3]};
+#pragma unroll
+                    for (int db = 0; db < DBLK; ++db) {
+                        const std::uint16_t* vp = v_lds + jb * 32 * D + v_rd[db] + 16 * s2 * D;
+                        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+                        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
+                        const i16x8 vf = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        oacc[db] = Mma16<T>::run(vf, __builtin_bit_cast(i16x8, pv), oacc[db]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // causal: the keys past the workgroup's last query were never visited; their weights are zero.
+    // Each wave clears that part of its 32 rows, a row at a time with 16-byte stores where the
+    // row starts allow it.
+    if (kMode == 3 && n_tiles * kBN < p.Lk) {
+        const int first = n_tiles * kBN;
+        const bool rows16 = (p.Lk % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.attn) & 15) == 0);
+        for (int rr = 0; rr < 32; ++rr) {
+            const int row = q0 + rr;
+            if (row >= p.Lq) break;
+            std::uint16_t* zr = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + row) * p.Lk;
+            if (rows16) {
+                for (int key = first + lane * 8; key < p.Lk; key += 64 * 8) store16(zr + key, u32x4{0u, 0u, 0u, 0u});
+            } else {
+                for (int key = first + lane; key < p.Lk; key += 64) zr[key] = 0;
+            }
+        }
+    }
+
+    if (row_live) {
+        std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d = db * 32 + g * 8 + 4 * lh;
+                u32x2 w;
+                w[0] = static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 0])) | (static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 1])) << 16);
+                w[1] = static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 2])) | (static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 3])) << 16);
+                *reinterpret_cast<u32x2*>(op + d) = w;
+            }
+        if (p.lse != nullptr && lh == 0)
+            p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run + logf(l_run);
+    }
+}
+
+template <typename T, int D>
+int launch_t(WeightsParams p, int mode, hipStream_t s) {
+    p.n_qblocks = (p.Lq + kBM - 1) / kBM;
+    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
+    const dim3 grid(static_cast<unsigned>(blocks)), wg(256);
+    switch (mode) {
+        case 0: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 0>), grid, wg, 0, s, p); break;
+        case 1: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 1>), grid, wg, 0, s, p); break;
+        case 2: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 2>), grid, wg, 0, s, p); break;
+        default: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 3>), grid, wg, 0, s, p); break;
+    }
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+bool mult8(const int64_t* strides) { return strides[0] % 8 == 0 && strides[1] % 8 == 0 && strides[2] % 8 == 0; }
+
+}  // namespace
+
+bool weights_supported(const paras_sdpa_args& a) {
+    if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
+    if (a.attn == nullptr) return false;                            // without the weights the flash kernels are the path
+    if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
+    if (a.mask_kind != 0 && (a.mask == nullptr || a.is_causal)) return false;
+    if (a.mask_kind < 0 || a.mask_kind > 2) return false;
+    if (a.mask_kind != 0 && a.mask_strides[3] != 1 && a.Lk > 1) return false;
+    if (a.Lq < 1 || a.Lk < 1) return false;
+    if (!std::isfinite(a.scale)) return false;
+    if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || (reinterpret_cast<uintptr_t>(a.out) & 7) != 0) return false;
+    if (!mult8(a.q_strides) || !mult8(a.k_strides) || !mult8(a.v_strides)) return false;
+    const int64_t nq = (a.Lq + kBM - 1) / kBM;
+    if (a.B * a.Hq * nq > 0x7fffffffLL || a.Lq > 0x3fffffff || a.Lk > 0x3fffffff) return false;
+    return true;
+}
+
+int launch_weights(const paras_sdpa_args& a, hipStream_t s) {
+    WeightsParams p;
+    p.q = static_cast<const std::uint16_t*>(a.q);
+    p.k = static_cast<const std::uint16_t*>(a.k);
+    p.v = static_cast<const std::uint16_t*>(a.v);
+    p.out = static_cast<std::uint16_t*>(a.out);
+    p.attn = static_cast<std::uint16_t*>(a.attn);
+    p.lse = a.lse;
+    p.qs_b = a.q_strides[0]; p.qs_h = a.q_strides[1]; p.qs_l = a.q_strides[2];
+    p.ks_b = a.k_strides[0]; p.ks_h = a.k_strides[1]; p.ks_l = a.k_strides[2];
+    p.vs_b = a.v_strides[0]; p.vs_h = a.v_strides[1]; p.vs_l = a.v_strides[2];
+    p.B = static_cast<int>(a.B); p.Hq = static_cast<int>(a.Hq); p.Hkv = static_cast<int>(a.Hkv);
+    p.Lq = static_cast<int>(a.Lq); p.Lk = static_cast<int>(a.Lk);
+    p.n_qblocks = 0;
+    p.scale = a.scale;
+    p.mask = static_cast<const unsigned char*>(a.mask);
+    p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2];
+    const int mode = a.is_causal ? 3 : a.mask_kind;
+    if (a.dtype == PARAS_BF16)
+        return a.D == 128 ? launch_t<bf16_t, 128>(p, mode, s) : launch_t<bf16_t, 64>(p, mode, s);
+    return a.D == 128 ? launch_t<f16_t, 128>(p, mode, s) : launch_t<f16_t, 64>(p, mode, s);
+}
+
+}  // namespace paras

@@ -235,8 +235,8 @@ typedef struct paras_sdpa_args {
 PARAS_API size_t paras_sdpa_workspace(const paras_sdpa_args* args);
 /* `workspace` may be NULL when paras_sdpa_workspace() returned 0. */
 PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream);
-/* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma", "decode_split"
- * or "generic". */
+/* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma", "decode_split",
+ * "math_mfma" (bf16 / f16 with the weights returned) or "generic". */
 PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 
 /* ------------------------------------------------------------------------- */

@@ -276,6 +276,78 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
     assert float(err_oracle.max()) <= 2 * ABS_16BIT, f"{shape} {dtype} {kind}"
 
 
+def ulps_apart(a, b):
+    """Distance in units of the last place between two 16-bit float tensors of one sign pattern."""
+    ia, ib = a.cpu().contiguous().view(torch.int16).int(), b.cpu().contiguous().view(torch.int16).int()
+    return (ia - ib).abs()
+
+
+WEIGHT_SHAPES = [  # B, Hq, Hkv, Lq, Lk, D
+    (1, 2, 2, 128, 128, 128), (2, 4, 2, 200, 333, 64), (1, 8, 2, 70, 1, 128), (1, 2, 1, 257, 129, 64), (1, 3, 3, 33, 700, 128),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("variant", ["plain", "causal", "bool", "additive"])
+@pytest.mark.parametrize("shape", WEIGHT_SHAPES)
+def test_math_op_weights_on_the_mfma_kernel(dtype, variant, shape):
+    """The math op's 16-bit callers (weights returned) run on the MFMA kernel that narrows where the
+    reference's composition narrows: the weights are the host engine's up to one unit in the last
+    place for a small fraction of them (fp32 instead of fp64 softmax arithmetic next to a rounding
+    boundary), NaN rows included, and the output is within the 2e-2 bar."""
+    B, Hq, Hkv, Lq, Lk, D = shape
+    q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
+    kw = {}
+    dead_row = None
+    if variant == "causal":
+        kw = dict(is_causal=True)
+    elif variant in ("bool", "additive"):
+        keep = torch.rand(B, 1, Lq, Lk) > 0.3
+        keep[..., 0] = True
+        if Lq > 4:
+            dead_row = Lq // 2
+            keep[:, :, dead_row, :] = False                       # a query that sees nothing: NaN weights and output
+        kw = dict(mask=keep if variant == "bool" else (torch.randn(B, 1, Lq, Lk) * 0.5).masked_fill(~keep, -math.inf).to(dtype))
+    scale = O.round_to_dtype(1 / math.sqrt(D), dtype)      # the op layer narrows the scale to the tensor type (to_compute)
+    out, attn, lse, kern = run(q, k, v, want_attn=True, want_lse=True, scale=scale, **kw)
+    okw = {("attn_mask" if a == "mask" else a): b for a, b in kw.items()}
+    want, wattn = O.sdpa_math(q, k, v, enable_gqa=True, gemm="aten", scale=scale, **okw)
+    assert kern == "math_mfma"
+    assert torch.equal(attn.cpu().isnan(), wattn.isnan()) and torch.equal(out.cpu().isnan(), want.isnan())
+    if dead_row is not None:
+        assert bool(attn[:, :, dead_row].isnan().all())
+    ok = ~wattn.isnan()
+    # One unit in the last place, except where the fp32 sum of q k^T itself (accumulated in another
+    # order than ATen's) rounds to the neighbouring 16-bit score: that moves a weight by a few units
+    # (the last bit of a 16-bit GEMM result is not pinned by the reference).  Absolute bar 2e-2.
+    d = ulps_apart(attn, wattn)[ok]
+    # Measured at [1,4,4,512,512,128] causal and [1,2,2,1024,1024,128]: 3e-5 .. 3e-4 of the weights differ,
+    # 5e-7 .. 1.4e-5 by more than one unit (at most 4), the output by at most 2e-3.
+    assert float((d > 1).float().mean()) <= 5e-4, f"{float((d > 1).float().mean()):.2e} of the weights more than one unit apart"
+    assert float((d > 0).float().mean()) <= 5e-3, f"{float((d > 0).float().mean()):.2e} of the weights differ"
+    assert float((attn.cpu().double() - wattn.double()).abs()[ok].max()) <= ABS_16BIT
+    oko = ~want.isnan()
+    assert float((out.cpu().double() - want.double()).abs()[oko].max()) <= ABS_16BIT
+    # rows of weights sum to one; log-sum-exp of the narrowed scores
+    live = ~wattn.isnan().any(-1)
+    assert torch.allclose(attn.cpu().float().sum(-1)[live], torch.ones_like(attn.cpu().float().sum(-1)[live]), atol=2e-2)
+    assert bool(torch.isfinite(lse.cpu()[live]).all())
+
+
+def test_math_op_weights_kernel_strided_inputs_and_explicit_scale():
+    """Heads sliced out of a fused [B, L, 3, H, D] projection (strided q / k / v) and an explicit
+    scale (narrowed to the tensor type, as the op layer hands it over)."""
+    qkv = torch.randn(2, 150, 3, 4, 128).bfloat16()
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    dq = qkv.cuda()
+    scale = O.round_to_dtype(0.0737, torch.bfloat16)
+    out, attn, _, kern = capi.sdpa(*(dq[:, :, i].permute(0, 2, 1, 3) for i in range(3)), is_causal=True, scale=scale, want_attn=True)
+    want, wattn = O.sdpa_math(q, k, v, is_causal=True, scale=scale, gemm="aten")
+    assert kern == "math_mfma"
+    d = ulps_apart(attn, wattn)
+    assert float((d > 1).float().mean()) <= 5e-4 and max_abs(attn, wattn) <= ABS_16BIT and max_abs(out, want) <= ABS_16BIT
+
+
 def test_masks_the_flash_kernel_does_not_take_still_work():
     """A mask that is not contiguous along the keys goes to the generic kernel."""
     q, k, v = torch.randn(1, 2, 40, 64).bfloat16(), torch.randn(1, 2, 50, 64).bfloat16(), torch.randn(1, 2, 50, 64).bfloat16()
