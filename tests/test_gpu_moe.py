@@ -26,7 +26,9 @@ def assert_ffn_close(out, ref, dtype):
     whose fp32 summation order differs from ATen's flips the last bit of a few
     intermediate y values; weighted and re-rounded they reach the output as at
     most one ulp of the top binade of the outputs, for at most 1 element in
-    1000."""
+    1000.  Measured at BASELINE config 5 over all 8192 x 4096 outputs
+    (max |out| 11.25): worst 0.0625, 5472 elements (1.6e-4) beyond 2e-2, 3170
+    (9.4e-5) beyond max(2e-2, 1 ulp), mean error 7.8e-5."""
     err = (out.double().cpu() - ref.double()).abs()
     tol = torch.maximum(torch.full_like(err, 2e-2), ulp16(ref, dtype) * 1.001)
     frac = float((err > tol).double().mean())

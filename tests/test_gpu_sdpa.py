@@ -258,11 +258,12 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
         out, want = out[:, :, rows], want[:, :, rows]
     assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(want).all())
     # Two bars.  Against softmax(q k^T s + mask) v evaluated in fp64 from the same 16-bit inputs: 1e-2.
-    # Against the host-engine oracle: 4e-2.  The oracle rounds the scores to 16 bits before the softmax;
-    # with part of the keys masked out a row is often dominated by one or two keys, a 2^-9 relative
-    # step on a score of magnitude 4-8 is then several per cent on the leading weights, and the oracle
-    # is itself more than 1e-2 away from the exact value (the unmasked BASELINE shapes, where hundreds
-    # of keys share the weight, are held to 2e-2 in the tests above).
+    # Against the host-engine oracle: 2e-2 for all but 1e-4 of the elements, 3e-2 for those.  The oracle
+    # rounds the scores to 16 bits before the softmax; with part of the keys masked out a row is often
+    # dominated by one or two keys, a 2^-9 relative step on a score of magnitude 4-8 is then several per
+    # cent on the leading weights, and the oracle is itself more than 1e-2 away from the exact value.
+    # Measured over these 16 cases: worst 0.0234 (bf16, bool mask, [2,4,4,200,200,128]: 3 of 204800
+    # elements beyond 2e-2), every other case at most 0.0156, fp16 at most 0.002.
     rep = Hq // Hkv
     sc = (q.double() @ k.double().repeat_interleave(rep, 1).transpose(-1, -2)) / math.sqrt(D)
     full = mask if mask.dim() == 4 else mask.expand(1, 1, *mask.shape[-2:]) if mask.dim() == 2 else mask
@@ -273,7 +274,8 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
     err_exact = (out.double().cpu() - exact).abs()
     err_oracle = (out.double().cpu() - want.double()).abs()
     assert float(err_exact.max()) <= 1e-2, f"{shape} {dtype} {kind}"
-    assert float(err_oracle.max()) <= 2 * ABS_16BIT, f"{shape} {dtype} {kind}"
+    assert float((err_oracle > ABS_16BIT).double().mean()) <= 1e-4, f"{shape} {dtype} {kind}: {int((err_oracle > ABS_16BIT).sum())} elements beyond 2e-2"
+    assert float(err_oracle.max()) <= 1.5 * ABS_16BIT, f"{shape} {dtype} {kind}: worst {float(err_oracle.max()):.4f}"
 
 
 def ulps_apart(a, b):
@@ -393,7 +395,7 @@ def test_decode_with_masks_matches_oracle(dtype):
     bias = (2 * torch.randn(B, Hq, 1, Lk)).masked_fill(~keep, -math.inf).to(dtype)
     out, _, _, kern = run(q, k, v, mask=bias)
     want, _ = O.sdpa_math(q, k, v, attn_mask=bias, enable_gqa=True, gemm="aten")
-    assert kern == "decode_split" and max_abs(out, want) <= 2 * ABS_16BIT
+    assert kern == "decode_split" and max_abs(out, want) <= ABS_16BIT       # measured: 0.0156 (bf16), 0.002 (fp16)
     q2 = torch.randn(B, Hq, 2, 128).to(dtype)
     m2 = torch.rand(2, Lk) > 0.5
     m2[:, 0] = True
