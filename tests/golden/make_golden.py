@@ -87,6 +87,17 @@ def main():
     put("topk_ties_literal", x=t, vals=vals, idx=idx)
     put("argsort_literal", x=torch.tensor([3, 1, 2, 1, 3]), out=R.argsort_stable(torch.tensor([3, 1, 2, 1, 3])))
 
+    # the glue primitives (drawn after everything above, so that the cases above keep their values)
+    for name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16), ("f16", torch.float16)):
+        a, b, row = rn(6, 70).to(dt), (rn(6, 70) + 2.5).to(dt), rn(70).to(dt)
+        idx = torch.tensor([5, 0, 0, 3, 2, 5, 1])
+        put(f"glue_{name}", a=a, b=b, row=row, idx=idx,
+            add=R.binary(0, a, b, 1.0), add_alpha=R.binary(0, a, b, -0.75), sub=R.binary(3, a, b, 1.0),
+            sub_row_alpha=R.binary(3, a, row, 2.5), mul_row=R.binary(1, a, row), div=R.binary(2, a, b),
+            add_s=R.binary_scalar(0, a, 0.3, 1.0), sub_s_alpha=R.binary_scalar(3, a, 0.3, 2.0),
+            mul_s=R.binary_scalar(1, a, 1 / math.sqrt(128)), div_s=R.binary_scalar(2, a, 3.0),
+            rows=R.index_select_rows(a, idx))
+
     path = Path(__file__).resolve().parent / "hotpath.safetensors"
     save_file(out, str(path))
     print(f"wrote {path} ({path.stat().st_size / 1024:.0f} KiB, {len(out)} tensors)")

@@ -78,3 +78,21 @@ def test_moe_ffn_and_literals():
     assert torch.equal(vals, t["vals"]) and torch.equal(idx, t["idx"])
     a = case("argsort_literal")
     assert torch.equal(O.argsort_stable(a["x"]), a["out"])
+
+
+@pytest.mark.parametrize("tag", DTYPE_TAGS)
+def test_glue_primitives(tag):
+    """add / sub (alpha) / mul / div of tensors and of a tensor with a number, and the row gather."""
+    c = case(f"glue_{tag}")
+    a, b, row = c["a"], c["b"], c["row"]
+    assert_bit_exact(O.binary(O.OP_ADD, a, b, 1.0), c["add"], "add")
+    assert_bit_exact(O.binary(O.OP_ADD, a, b, -0.75), c["add_alpha"], "add alpha")
+    assert_bit_exact(O.binary(O.OP_SUB, a, b, 1.0), c["sub"], "sub")
+    assert_bit_exact(O.binary(O.OP_SUB, a, row, 2.5), c["sub_row_alpha"], "sub broadcast alpha")
+    assert_bit_exact(O.binary(O.OP_MUL, a, row), c["mul_row"], "mul broadcast")
+    assert_bit_exact(O.binary(O.OP_DIV, a, b), c["div"], "div")
+    assert_bit_exact(O.binary_scalar(O.OP_ADD, a, 0.3, 1.0), c["add_s"], "add number")
+    assert_bit_exact(O.binary_scalar(O.OP_SUB, a, 0.3, 2.0), c["sub_s_alpha"], "sub number alpha")
+    assert_bit_exact(O.binary_scalar(O.OP_MUL, a, 1 / math.sqrt(128)), c["mul_s"], "mul number")
+    assert_bit_exact(O.binary_scalar(O.OP_DIV, a, 3.0), c["div_s"], "div number")
+    assert_bit_exact(O.index_select_rows(a, c["idx"]), c["rows"], "index_select rows")

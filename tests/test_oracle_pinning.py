@@ -69,6 +69,17 @@ def test_oracle_equals_reference_engine_bitwise(dtype):
               ("rms_norm_composed", (x3, [4, 5]), {})]
     batch += [("sdpa_math", (q, k, v), kw) for kw in variants]
     batch += [("sdpa_math", (q, kg, vg), dict(enable_gqa=True))]
+    # the glue primitives: add / sub (with alpha) / mul / div of tensors (one broadcast) and of a
+    # tensor with a number, and the row gather of the MoE permutation
+    a2, b2, row = rn(6, 70).to(dtype), (rn(6, 70) + 2.5).to(dtype), rn(70).to(dtype)
+    idx = torch.tensor([5, 0, 0, 3, 2, 5, 1])
+    glue = [("binary", (O.OP_ADD, a2, b2, 1.0), {}), ("binary", (O.OP_ADD, a2, b2, -0.75), {}), ("binary", (O.OP_SUB, a2, b2, 1.0), {}),
+            ("binary", (O.OP_SUB, a2, row, 2.5), {}), ("binary", (O.OP_MUL, a2, row), {}), ("binary", (O.OP_DIV, a2, b2), {}),
+            ("binary_scalar", (O.OP_ADD, a2, 0.3, 1.0), {}), ("binary_scalar", (O.OP_SUB, a2, 0.3, 2.0), {}),
+            ("binary_scalar", (O.OP_MUL, a2, 1 / math.sqrt(128)), {}), ("binary_scalar", (O.OP_DIV, a2, 3.0), {}),
+            ("index_select_rows", (a2, idx), {})]
+    n_glue0 = len(batch)
+    batch += glue
     results = R.run_batch(batch)          # one child process: the engine owns PrivateUse1
 
     def same(got, want, what):
@@ -92,7 +103,9 @@ def test_oracle_equals_reference_engine_bitwise(dtype):
         alt = O.sdpa_math(q, k, v, gemm="c", **kw)
         tol = {torch.float32: 2e-6, torch.float64: 1e-14, torch.bfloat16: 1.6e-2, torch.float16: 2e-3}[dtype]
         assert (alt[0].double() - want[0].double()).abs().max() <= tol
-    same(O.sdpa_math(q, kg, vg, enable_gqa=True, gemm="aten"), results[-1], "sdpa gqa")
+    same(O.sdpa_math(q, kg, vg, enable_gqa=True, gemm="aten"), results[n_glue0 - 1], "sdpa gqa")
+    for (name, args, kw), want in zip(glue, results[n_glue0:]):
+        same(getattr(O, name)(*args, **kw), want, f"{name} op {args[0] if name != 'index_select_rows' else ''}")
 
 
 @needs_ref
