@@ -9,6 +9,8 @@
 #include <c10/core/impl/DeviceGuardImplInterface.h>
 #include <torch/version.h>
 
+#include <cstdlib>
+
 #include "paras_torch.h"
 
 #if TORCH_VERSION_MAJOR < 2 || (TORCH_VERSION_MAJOR == 2 && TORCH_VERSION_MINOR < 4)
@@ -18,7 +20,14 @@
 namespace paras_torch {
 namespace {
 
-thread_local c10::DeviceIndex tl_device = 0;
+int read_device_base() {
+    const char* v = std::getenv("PARAS_DEVICE_BASE");
+    return (v != nullptr && v[0] == '1' && v[1] == '\0') ? 1 : 0;
+}
+const int g_device_base = read_device_base();
+
+// The thread's current device: the first GPU under either numbering.
+thread_local c10::DeviceIndex tl_device = static_cast<c10::DeviceIndex>(g_device_base);
 
 struct GuardImpl final : public c10::impl::DeviceGuardImplInterface {
     c10::DeviceType type() const override { return kParas; }
@@ -33,10 +42,10 @@ struct GuardImpl final : public c10::impl::DeviceGuardImplInterface {
     c10::Stream getStream(c10::Device d) const noexcept override { return c10::Stream(c10::Stream::UNSAFE, d, 0); }
     c10::Stream getDefaultStream(c10::Device d) const override { return getStream(d); }
     c10::Stream exchangeStream(c10::Stream) const noexcept override { return getStream(c10::Device(kParas, tl_device)); }
-    c10::DeviceIndex deviceCount() const noexcept override { return static_cast<c10::DeviceIndex>(paras_device_count()); }
+    c10::DeviceIndex deviceCount() const noexcept override { return static_cast<c10::DeviceIndex>(paras_device_count() + g_device_base); }
     bool queryStream(const c10::Stream&) const override { return true; }
-    void synchronizeStream(const c10::Stream& s) const override { check(paras_synchronize(s.device().index())); }
-    void synchronizeDevice(const c10::DeviceIndex index) const override { check(paras_synchronize(index)); }
+    void synchronizeStream(const c10::Stream& s) const override { check(paras_synchronize(hip_device(s.device().index()))); }
+    void synchronizeDevice(const c10::DeviceIndex index) const override { check(paras_synchronize(hip_device(index))); }
 };
 
 GuardImpl g_guard;
@@ -44,7 +53,7 @@ c10::impl::DeviceGuardImplRegistrar g_guard_registrar(kParas, &g_guard);
 
 struct Hooks final : public at::PrivateUse1HooksInterface {
     bool hasPrimaryContext(c10::DeviceIndex index) const override {
-        return index >= 0 && index < paras_device_count();
+        return index >= g_device_base && index < paras_device_count() + g_device_base;
     }
     bool isAvailable() const override { return paras_device_count() > 0; }
 };
@@ -54,7 +63,7 @@ struct HooksRegistrar {
     HooksRegistrar() { at::RegisterPrivateUse1HooksInterface(&hooks); }
 } g_hooks_registrar;
 
-// DataPtr context: which pool the block goes back to.
+// DataPtr context: which pool (HIP device index) the block goes back to.
 struct Block {
     void* ptr;
     int   device;
@@ -71,18 +80,17 @@ void release_block(void* opaque) {
 
 struct Allocator final : public c10::Allocator {
     c10::DataPtr allocate(size_t nbytes) override {
-        const int dev = tl_device;
+        const c10::DeviceIndex index = tl_device;
+        const int dev = hip_device(index);
         void* p = nullptr;
         if (nbytes > 0) check(paras_alloc(dev, nbytes, &p));
-        else TORCH_CHECK(dev >= 0 && dev < paras_device_count(), "paras: invalid device index ", dev,
-                         " (device count: ", paras_device_count(), ")");
         auto* b = new Block{p, dev};
-        return c10::DataPtr(p, b, &release_block, c10::Device(kParas, static_cast<c10::DeviceIndex>(dev)));
+        return c10::DataPtr(p, b, &release_block, c10::Device(kParas, index));
     }
     c10::DeleterFnPtr raw_deleter() const override { return &release_block; }
     void copy_data(void* dest, const void* src, std::size_t count) const override {
-        check(paras_memcpy(tl_device, dest, src, count, 2));
-        check(paras_synchronize(tl_device));
+        check(paras_memcpy(hip_device(tl_device), dest, src, count, 2));
+        check(paras_synchronize(hip_device(tl_device)));
     }
 };
 
@@ -93,9 +101,22 @@ REGISTER_ALLOCATOR(kParas, &g_allocator);
 
 c10::DeviceIndex current_device() { return tl_device; }
 
+int device_base() { return g_device_base; }
+int device_count_torch() { return paras_device_count() + g_device_base; }
+
+int hip_device(c10::DeviceIndex index) {
+    TORCH_CHECK(!(g_device_base == 1 && index == 0),
+                "paras:0 is the host CPU engine in the reference's numbering (PARAS_DEVICE_BASE=1); this build has no host "
+                "engine: GPUs are paras:1 .. paras:", paras_device_count());
+    const int hip = static_cast<int>(index) - g_device_base;
+    TORCH_CHECK(hip >= 0 && hip < paras_device_count(), "paras: invalid device index ", static_cast<int>(index),
+                " (device count: ", device_count_torch(), ")");
+    return hip;
+}
+
 void* stream_for(c10::DeviceIndex index) {
     void* s = nullptr;
-    check(paras_stream(index, &s));
+    check(paras_stream(hip_device(index), &s));
     return s;
 }
 

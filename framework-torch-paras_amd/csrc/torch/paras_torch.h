@@ -64,6 +64,17 @@ inline int require_float_code(const at::Tensor& t, const char* op) {
     return c;
 }
 
+// Device numbering.  By default `paras:i` is HIP GPU i.  With PARAS_DEVICE_BASE=1 in the
+// environment the package numbers devices as the reference does (csrc/compat/paras_compat.cpp:
+// 87-97: device 0 is the host CPU engine, GPUs start at 1): `paras:i` is then HIP GPU i - 1 and
+// `paras:0` raises, because this build has no host engine.  device_base() is 0 or 1;
+// device_count_torch() is the number of `paras` indices (GPUs + base); hip_device() maps a
+// `paras` index to the library's HIP index or raises.
+int device_base();
+int device_count_torch();
+int hip_device(c10::DeviceIndex index);
+inline int hip_device(const at::Tensor& t) { return hip_device(t.device().index()); }
+
 // Makes `index` the calling thread's HIP device and returns the context
 // stream every `paras` op of that device is queued on.
 void* stream_for(c10::DeviceIndex index);

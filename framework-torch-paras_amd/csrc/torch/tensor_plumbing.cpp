@@ -27,7 +27,8 @@ c10::Device resolve(c10::optional<c10::Device> device) {
     c10::Device d = device.value_or(c10::Device(kParas, current_device()));
     TORCH_CHECK(d.type() == kParas, "paras: expected a paras device, got ", d);
     if (!d.has_index()) d = c10::Device(kParas, current_device());
-    const int n = paras_device_count();
+    (void)hip_device(d.index());       // raises for paras:0 under the reference's numbering and for indices out of range
+    const int n = device_count_torch();
     TORCH_CHECK(d.index() >= 0 && d.index() < n, "paras: invalid device index ", static_cast<int>(d.index()),
                 " (device count: ", n, ")");
     return d;
@@ -96,7 +97,7 @@ Tensor copy_from(const Tensor& self, const Tensor& dst, bool non_blocking) {
     const size_t nbytes_dst = static_cast<size_t>(dst.numel()) * dst.element_size();
 
     if (src_dev && dst.device().is_cpu()) {
-        const int dev = self.device().index();
+        const int dev = hip_device(self);
         Tensor staged = self;
         if (!self.is_contiguous() || self.scalar_type() != dst.scalar_type()) {
             const bool convertible = self.scalar_type() == dst.scalar_type() ||
@@ -118,7 +119,7 @@ Tensor copy_from(const Tensor& self, const Tensor& dst, bool non_blocking) {
         return dst;
     }
     if (self.device().is_cpu() && dst_dev) {
-        const int dev = dst.device().index();
+        const int dev = hip_device(dst);
         Tensor src_c = self.expand_as(dst);
         if (src_c.scalar_type() != dst.scalar_type()) src_c = src_c.to(dst.scalar_type());
         src_c = src_c.contiguous();
@@ -139,7 +140,7 @@ Tensor copy_from(const Tensor& self, const Tensor& dst, bool non_blocking) {
             return dst;
         }
         if (dense_same_layout(self, dst) && self.scalar_type() == dst.scalar_type())
-            check(paras_memcpy(dst.device().index(), dst.data_ptr(), self.data_ptr(), nbytes_dst, 2));
+            check(paras_memcpy(hip_device(dst), dst.data_ptr(), self.data_ptr(), nbytes_dst, 2));
         else
             device_copy(self, dst);
         return dst;
@@ -169,7 +170,7 @@ Tensor& zero_(Tensor& self) { return fill_scalar(self, 0); }
 c10::Scalar local_scalar_dense(const Tensor& self) {
     TORCH_CHECK(self.numel() == 1, "paras: a tensor with ", self.numel(), " elements cannot be converted to a scalar");
     Tensor host = at::empty({}, self.options().device(c10::kCPU));
-    check(paras_memcpy(self.device().index(), host.data_ptr(), self.data_ptr(), self.element_size(), 1));
+    check(paras_memcpy(hip_device(self), host.data_ptr(), self.data_ptr(), self.element_size(), 1));
     return at::_local_scalar_dense(host);
 }
 
@@ -201,8 +202,8 @@ const Tensor& resize_(const Tensor& self, c10::IntArrayRef size, c10::optional<c
         c10::DataPtr fresh = c10::GetAllocator(kParas)->allocate(need);
         const size_t keep = self.storage().nbytes();
         if (keep > 0)
-            check(paras_memcpy(self.device().index(), fresh.get(), self.storage().data(), keep, 2));
-        check(paras_synchronize(self.device().index()));
+            check(paras_memcpy(hip_device(self), fresh.get(), self.storage().data(), keep, 2));
+        check(paras_synchronize(hip_device(self)));
         self.storage().set_data_ptr_noswap(std::move(fresh));
         self.storage().set_nbytes(need);
     }

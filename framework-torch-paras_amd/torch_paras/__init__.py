@@ -12,9 +12,12 @@ device_count, is_available, synchronize, manual_seed(_all), empty_cache,
 device_name, backend_name, is_gpu_device, memory_allocated, memory_cached,
 get_amp_supported_dtype, and the ``nn`` submodule.  One difference in device
 numbering, on purpose: this build is HIP-only, so ``paras:i`` is HIP GPU ``i``;
-there is no host-CPU engine behind ``paras:0``.  With no GPU visible the
-package still imports, ``device_count()`` is 0 and every op on a ``paras``
-tensor raises.
+there is no host-CPU engine behind ``paras:0``.  Scripts written for the
+reference's numbering (``paras:0`` = host engine, GPUs from ``paras:1``) run
+unchanged with ``PARAS_DEVICE_BASE=1`` in the environment before the import:
+``paras:i`` is then HIP GPU ``i - 1``, ``device_count()`` counts the host slot
+as the reference does, and any use of ``paras:0`` raises.  With no GPU visible
+the package still imports and every op on a ``paras`` tensor raises.
 """
 from __future__ import annotations
 
@@ -33,12 +36,13 @@ __all__ = [
 
 
 def device_count() -> int:
-    """Number of paras devices (= visible HIP GPUs)."""
+    """Number of paras device indices: the visible HIP GPUs, plus the (unusable) host
+    slot ``paras:0`` under PARAS_DEVICE_BASE=1."""
     return _C.device_count()
 
 
 def is_available() -> bool:
-    return device_count() > 0
+    return device_count() - _C.device_base() > 0
 
 
 def backend_name() -> str:
@@ -55,7 +59,7 @@ def is_gpu_device(device: int) -> bool:
 
 
 def current_device() -> int:
-    return 0
+    return _C.current_device()
 
 
 def synchronize(device: int | None = None) -> None:

@@ -717,3 +717,9 @@ def test_device_to_host_copy_broadcasts(device):
     dst16 = torch.zeros(3, 5, dtype=torch.bfloat16)
     dst16.copy_(src.to(device))
     assert torch.equal(dst16, src.bfloat16().expand(3, 5))
+
+
+def test_reference_device_numbering_on_the_gpu():
+    """PARAS_DEVICE_BASE=1 with a GPU present: ops run on `paras:1`, `paras:0` raises."""
+    from test_package_cpu import test_reference_device_numbering_is_an_opt_in
+    test_reference_device_numbering_is_an_opt_in()
