@@ -172,7 +172,94 @@ __global__ __launch_bounds__(kThreads) void moe_combine_kernel(const std::uint16
     }
 }
 
+// ---- sizes the MFMA tiles do not take (hidden or intermediate size not a multiple of 64) -------
+// One thread per output element: the routed row's expert is looked up in `offsets`, the dot
+// products over the contraction dim accumulate in fp32 (one rounding to T, like the tile kernels),
+// the SwiGLU of GEMM 1 is applied to the narrowed gate and up values.  No alignment or size
+// requirement; two orders of magnitude slower than the tiles, so it only serves odd shapes.
+template <typename T, bool kSwiglu>
+__global__ __launch_bounds__(kThreads) void grouped_any_kernel(const FfnGemmParams p) {
+    using El = Elem<T>;
+    const long prow = blockIdx.y;
+    const long col = static_cast<long>(blockIdx.x) * kThreads + threadIdx.x;
+    if (col >= p.N) return;
+    int e = 0;
+    while (e + 1 < p.E && prow >= p.offsets[e + 1]) ++e;
+    const long src = p.order ? p.order[prow] / p.k : prow;
+    const std::uint16_t* a = p.a + src * p.K;
+    const std::uint16_t* w0 = p.b + (static_cast<long>(e) * p.Nw + col) * p.K;
+    float acc0 = 0.f, acc1 = 0.f;
+    if (kSwiglu) {
+        const std::uint16_t* w1 = p.b2 + (static_cast<long>(e) * p.Nw + col) * p.K;
+        for (long kk = 0; kk < p.K; ++kk) {
+            const float av = El::to_f32(a[kk]);
+            acc0 = fmaf(av, El::to_f32(w0[kk]), acc0);
+            acc1 = fmaf(av, El::to_f32(w1[kk]), acc1);
+        }
+        p.c[prow * p.N + col] = swiglu_one<T>(El::from_f32(acc0), El::from_f32(acc1));
+    } else {
+        for (long kk = 0; kk < p.K; ++kk) acc0 = fmaf(El::to_f32(a[kk]), El::to_f32(w0[kk]), acc0);
+        p.c[prow * p.N + col] = El::from_f32(acc0);
+    }
+}
+
+// The combine for any H: one element per thread.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void moe_combine_any_kernel(const std::uint16_t* __restrict__ y, const float* __restrict__ topw,
+                                                                  const long* __restrict__ inv_order, std::uint16_t* __restrict__ out,
+                                                                  long T_, int k, long H) {
+    using El = Elem<T>;
+    const long total = T_ * H;
+    for (long i = static_cast<long>(blockIdx.x) * kThreads + threadIdx.x; i < total; i += static_cast<long>(gridDim.x) * kThreads) {
+        const long t = i / H, c = i % H;
+        double acc = 0.0;
+        for (int s = 0; s < k; ++s) {
+            const double w = El::to_f64(El::from_f32(topw[t * k + s]));
+            acc += El::to_f64(El::from_f64(El::to_f64(y[inv_order[t * k + s] * H + c]) * w));
+        }
+        out[t * H + c] = El::from_f64(acc);
+    }
+}
+
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+template <typename T>
+int run_ffn_any(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw, const long* order,
+                const long* inv_order, const long* offsets, void* out, void* workspace, long T_, int E, int k, long H, long I,
+                hipStream_t s) {
+    const long R = T_ * k;
+    auto* h = static_cast<std::uint16_t*>(workspace);
+    auto* y = reinterpret_cast<std::uint16_t*>(static_cast<char*>(workspace) + align_up(static_cast<size_t>(R) * I * 2, 256));
+    PARAS_REQUIRE(R <= 65535, "paras_moe_ffn: at most 65535 routed rows when the hidden or intermediate size is not a multiple of %d", kBK);
+    FfnGemmParams g1{};
+    g1.a = static_cast<const std::uint16_t*>(x);
+    g1.b = static_cast<const std::uint16_t*>(w_gate);
+    g1.b2 = static_cast<const std::uint16_t*>(w_up);
+    g1.c = h;
+    g1.order = order;
+    g1.offsets = offsets;
+    g1.K = H; g1.N = I; g1.Nw = I; g1.R = R; g1.E = E; g1.k = k;
+    hipLaunchKernelGGL((grouped_any_kernel<T, true>), dim3(static_cast<unsigned>((I + kThreads - 1) / kThreads), static_cast<unsigned>(R)),
+                       dim3(kThreads), 0, s, g1);
+    PARAS_HIP_TRY(hipGetLastError());
+    FfnGemmParams g2{};
+    g2.a = h;
+    g2.b = static_cast<const std::uint16_t*>(w_down);
+    g2.b2 = g2.b;
+    g2.c = y;
+    g2.order = nullptr;
+    g2.offsets = offsets;
+    g2.K = I; g2.N = H; g2.Nw = H; g2.R = R; g2.E = E; g2.k = k;
+    hipLaunchKernelGGL((grouped_any_kernel<T, false>), dim3(static_cast<unsigned>((H + kThreads - 1) / kThreads), static_cast<unsigned>(R)),
+                       dim3(kThreads), 0, s, g2);
+    PARAS_HIP_TRY(hipGetLastError());
+    long blocks = (T_ * H + kThreads - 1) / kThreads;
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    hipLaunchKernelGGL((moe_combine_any_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, y, topw, inv_order,
+                       static_cast<std::uint16_t*>(out), T_, k, H);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
 
 template <typename T, typename S>
 int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
@@ -264,13 +351,11 @@ int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up, const voi
     PARAS_REQUIRE(T >= 0 && E >= 1 && k >= 1 && H >= 1 && I >= 1, "paras_moe_ffn: bad shape");
     if (T == 0) return PARAS_OK;
     PARAS_REQUIRE(dtype == PARAS_BF16 || dtype == PARAS_F16, "paras_moe_ffn: dtype must be bf16 or f16");
-    if (H % kBK != 0 || I % kBK != 0)
-        return fail(PARAS_ERR_UNSUPPORTED, "paras_moe_ffn: hidden (%lld) and intermediate (%lld) sizes must be multiples of %d",
-                    (long long)H, (long long)I, kBK);
+    const bool tiles = H % kBK == 0 && I % kBK == 0;     // else: the general kernels (any size, any alignment)
     PARAS_REQUIRE(x && w_gate && w_up && w_down && topw && order && inv_order && offsets && out && workspace,
                   "paras_moe_ffn: null pointer");
-    PARAS_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_gate) | reinterpret_cast<uintptr_t>(w_up) |
-                    reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0,
+    PARAS_REQUIRE(!tiles || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_gate) | reinterpret_cast<uintptr_t>(w_up) |
+                              reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0,
                   "paras_moe_ffn: tensors must be 16-byte aligned");
     PARAS_REQUIRE(T * k <= 0x3fffffffLL, "paras_moe_ffn: too many routed rows");
     if (T * H >= (1LL << 32) || T * k * I >= (1LL << 32) || I * H >= (1LL << 32))
@@ -281,6 +366,11 @@ int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up, const voi
     const long* ord = reinterpret_cast<const long*>(order);
     const long* inv = reinterpret_cast<const long*>(inv_order);
     const long* off = reinterpret_cast<const long*>(offsets);
+    if (!tiles) {
+        if (dtype == PARAS_BF16)
+            return run_ffn_any<bf16_t>(x, w_gate, w_up, w_down, topw, ord, inv, off, out, workspace, T, (int)E, (int)k, H, I, s);
+        return run_ffn_any<f16_t>(x, w_gate, w_up, w_down, topw, ord, inv, off, out, workspace, T, (int)E, (int)k, H, I, s);
+    }
     if (dtype == PARAS_BF16)
         return run_ffn<bf16_t>(x, w_gate, w_up, w_down, topw, ord, inv, off, out, workspace, T, (int)E, (int)k, H, I, s);
     return run_ffn<f16_t>(x, w_gate, w_up, w_down, topw, ord, inv, off, out, workspace, T, (int)E, (int)k, H, I, s);

@@ -197,8 +197,9 @@ __global__ __launch_bounds__(kBlock) void rms_norm_bwd_dw_partial(
     const typename Elem<T>::store_t* __restrict__ go, const typename Elem<T>::store_t* __restrict__ x,
     const float* __restrict__ rstd, double* __restrict__ partial, long rows, long H) {
     using E = Elem<T>;
-    const long j = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
-    const long slab = blockIdx.y;
+    // slabs along grid x (up to 2^31 - 1 of them), columns along grid y
+    const long j = static_cast<long>(blockIdx.y) * kBlock + threadIdx.x;
+    const long slab = blockIdx.x;
     if (j >= H) return;
     const long r0 = slab * kDwSlabRows;
     const long r1 = r0 + kDwSlabRows < rows ? r0 + kDwSlabRows : rows;
@@ -470,13 +471,13 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
             return PARAS_OK;
         }
     }
+    const unsigned gx_blocks = static_cast<unsigned>((H + kBlock - 1) / kBlock);
+    PARAS_REQUIRE(gx_blocks <= 65535, "paras_rms_norm_bwd: rows of more than %d elements are not supported", 65535 * kBlock);   // before any launch
     hipLaunchKernelGGL((rms_norm_bwd_dx<T>), dim3(grid_for_rows(rows)), dim3(kBlock), 0, s,
                        static_cast<const S*>(go), static_cast<const S*>(x), static_cast<const S*>(w),
                        rstd, static_cast<S*>(gx), rows, H);
     PARAS_HIP_TRY(hipGetLastError());
-    const unsigned gx_blocks = static_cast<unsigned>((H + kBlock - 1) / kBlock);
-    PARAS_REQUIRE(slabs <= 65535, "paras_rms_norm_bwd: too many rows for this dtype / row size");
-    hipLaunchKernelGGL((rms_norm_bwd_dw_partial<T>), dim3(gx_blocks, static_cast<unsigned>(slabs)),
+    hipLaunchKernelGGL((rms_norm_bwd_dw_partial<T>), dim3(static_cast<unsigned>(slabs), gx_blocks),
                        dim3(kBlock), 0, s, static_cast<const S*>(go), static_cast<const S*>(x), rstd,
                        static_cast<double*>(workspace), rows, H);
     PARAS_HIP_TRY(hipGetLastError());

@@ -1,5 +1,5 @@
 // Split-KV decode attention for gfx950: few query rows per KV head (query
-// length x GQA group <= 16), long K/V, bf16 / fp16, head dim 128.  The job is
+// length x GQA group <= 16), long K/V, bf16 / fp16, head dim 64 or 128.  The job is
 // HBM-bound -- every K and V byte is read exactly once, K/V heads are never
 // replicated for GQA (the reference copies them Hq/Hkv times:
 // csrc/ops/tensor_ops.cpp:687-729) -- so the design is about keeping many
@@ -30,9 +30,9 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves   = 4;
-constexpr int kD       = 128;
 constexpr int kTile    = 32;        // keys per wave per step
-constexpr int kVS      = kD + 16;   // V row stride in LDS: 8 consecutive rows x 32 B hit 64 distinct banks
+// V row stride in LDS is D + 16 elements: 8 consecutive rows x 32 B then hit 64 distinct banks
+// (288-byte rows at D = 128, 160-byte rows at D = 64).
 constexpr int kMaxRows = 16;        // query rows per KV head (MFMA N)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -44,7 +44,7 @@ struct DecodeParams {
     const std::uint16_t* v;
     std::uint16_t* out;
     float* lse;
-    float* part_o;   // [pairs, splits, 16, 128]
+    float* part_o;   // [pairs, splits, 16, D]
     float* part_ml;  // [pairs, splits, 2, 16]
     long qs_b, qs_h, qs_l, ks_b, ks_h, ks_l, vs_b, vs_h, vs_l;
     int B, Hq, Hkv, Lq, Lk, G, R;
@@ -91,10 +91,14 @@ __device__ __forceinline__ float group_sum(float x) {
 }
 
 // kMask: 0 = none, 1 = bool (true = attend), 2 = additive values of dtype T
-template <typename T, int kMask>
+template <typename T, int D, int kMask>
 __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeParams p) {
+    constexpr int kD = D, kVS = D + 16;
+    constexpr int KS = D / 32;           // 32-wide contraction steps of q k^T
+    constexpr int DB = D / 16;           // 16-wide output blocks of O^T
+    constexpr int VCH = kTile * D / 8 / 64;   // 16-byte chunks of a V tile per lane
     // Per-wave V tiles (double buffered); reused as fp32 merge space at the end.
-    __shared__ __attribute__((aligned(16))) std::uint16_t v_lds[kWaves][2][kTile * kVS];
+    __shared__ __attribute__((aligned(16))) std::uint16_t v_lds[kWaves][2][kTile * (D + 16)];
     __shared__ float m_lds[kWaves][kMaxRows], l_lds[kWaves][kMaxRows];
 
     const int split = blockIdx.x, pair = blockIdx.y;
@@ -103,13 +107,13 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
     const int lq = lane & 15, lg = lane >> 4;
 
     // ---- the query rows of this KV head: row r = gi*Lq + i  (head hkv*G+gi, position i)
-    i16x8 qreg[4];
+    i16x8 qreg[KS];
     {
         const bool live = lq < p.R;
         const int gi = live ? lq / p.Lq : 0, qi = live ? lq % p.Lq : 0;
         const std::uint16_t* qp = p.q + b * p.qs_b + static_cast<long>(hkv * p.G + gi) * p.qs_h + static_cast<long>(qi) * p.qs_l;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             i16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
             qreg[ks] = live ? *reinterpret_cast<const i16x8*>(qp + 32 * ks + 8 * lg) : z;
         }
@@ -134,39 +138,39 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
     const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
     const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
 
-    i16x8 kcur[2][4], knext[2][4];
-    u32x4 vst[8];
-    auto load_k = [&](int t, i16x8 (&dst)[2][4]) {
+    i16x8 kcur[2][KS], knext[2][KS];
+    u32x4 vst[VCH];
+    auto load_k = [&](int t, i16x8 (&dst)[2][KS]) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             int key = k_begin + t * kTile + kb * 16 + lq;
             key = key < p.Lk ? key : p.Lk - 1;  // masked later; keep the load in bounds
             const std::uint16_t* kp = kbase + static_cast<long>(key) * p.ks_l + 8 * lg;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) dst[kb][ks] = __builtin_bit_cast(i16x8, load16_nt(kp + 32 * ks));  // read once: keep it out of the caches
+            for (int ks = 0; ks < KS; ++ks) dst[kb][ks] = __builtin_bit_cast(i16x8, load16_nt(kp + 32 * ks));  // read once: keep it out of the caches
         }
     };
     auto load_v = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int c = lane + i * 64;  // 16-byte chunk of the 32 x 128 tile
-            const int row = c >> 4, col = (c & 15) * 8;
+        for (int i = 0; i < VCH; ++i) {
+            const int c = lane + i * 64;  // 16-byte chunk of the 32 x D tile
+            const int row = c / (D / 8), col = (c % (D / 8)) * 8;
             const int key = k_begin + t * kTile + row;
             vst[i] = key < k_end ? load16_nt(vbase + static_cast<long>(key) * p.vs_l + col) : u32x4{0, 0, 0, 0};
         }
     };
     auto store_v = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < VCH; ++i) {
             const int c = lane + i * 64;
-            const int row = c >> 4, col = (c & 15) * 8;
+            const int row = c / (D / 8), col = (c % (D / 8)) * 8;
             *reinterpret_cast<u32x4*>(&v_lds[wave][buf][row * kVS + col]) = vst[i];
         }
     };
 
-    float4_t oacc[8];
+    float4_t oacc[DB];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < DB; ++i) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
     if (n_tiles > 0) {
@@ -189,7 +193,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
         for (int kb = 0; kb < 2; ++kb) {
             sacc[kb] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) sacc[kb] = Mma16<T>::run(kcur[kb][ks], qreg[ks], sacc[kb]);
+            for (int ks = 0; ks < KS; ++ks) sacc[kb] = Mma16<T>::run(kcur[kb][ks], qreg[ks], sacc[kb]);
         }
         const int key0 = k_begin + t * kTile;
         if constexpr (kMask != 0) {
@@ -234,7 +238,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
             }
         l_run = l_run * alpha + lsum;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
+        for (int i = 0; i < DB; ++i) oacc[i] *= alpha;
         // P^T operand: contraction order e<4 -> key 4*lg+e, e>=4 -> key 16+4*lg+(e-4)
         u32x4 w;
         w[0] = Mma16<T>::pack2(sacc[0][0], sacc[0][1]);
@@ -248,7 +252,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int db = 0; db < 8; ++db) {
+        for (int db = 0; db < DB; ++db) {
             const std::uint16_t* vp = &v_lds[wave][buf][v_off + db * 16];
             const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
             const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 16 * kVS));
@@ -260,17 +264,18 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) kcur[kb][ks] = knext[kb][ks];
+                for (int ks = 0; ks < KS; ++ks) kcur[kb][ks] = knext[kb][ks];
         }
     }
 
     // ---- merge the 4 waves: O^T lane (query lq, group lg) holds d = 16*db + 4*lg + r
     const float l_wave = group_sum(l_run);
     __syncthreads();  // everyone is done with the V tiles
-    float* o_lds = reinterpret_cast<float*>(&v_lds[0][0][0]);  // [wave][16][128] floats = 32 KB
+    float* o_lds = reinterpret_cast<float*>(&v_lds[0][0][0]);  // [wave][16][D] floats: 32 KB / 16 KB, inside the V tiles' space
+    static_assert(sizeof(float) * kWaves * kMaxRows * D <= sizeof(std::uint16_t) * kWaves * 2 * kTile * kVS, "merge space");
     if (lq < p.R) {
 #pragma unroll
-        for (int db = 0; db < 8; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int r = 0; r < 4; ++r) o_lds[(wave * kMaxRows + lq) * kD + 16 * db + 4 * lg + r] = oacc[db][r];
         if (lg == 0) {
@@ -309,9 +314,10 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
     }
 }
 
-// One workgroup of 128 threads (one per d) per (pair, query row).
-template <typename T>
-__global__ __launch_bounds__(kD) void decode_combine_kernel(const DecodeParams p) {
+// One workgroup of D threads (one per d) per (pair, query row).
+template <typename T, int D>
+__global__ __launch_bounds__(D) void decode_combine_kernel(const DecodeParams p) {
+    constexpr int kD = D;
     const int pair = blockIdx.x, r = blockIdx.y, d = threadIdx.x;
     const int b = pair / p.Hkv, hkv = pair % p.Hkv;
     float M = -INFINITY;
@@ -356,7 +362,7 @@ void plan(const paras_sdpa_args& a, int* splits, int* chunk) {
 
 bool decode_supported(const paras_sdpa_args& a) {
     if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
-    if (a.D != kD || a.Dv != kD) return false;
+    if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
     if (a.attn != nullptr || a.is_causal) return false;
     if (a.mask_kind != 0 && (a.mask == nullptr || a.mask_kind > 2)) return false;
     if (a.Hkv < 1 || a.Hq % a.Hkv != 0) return false;
@@ -374,7 +380,7 @@ size_t decode_workspace(const paras_sdpa_args& a) {
     plan(a, &splits, &chunk);
     if (splits == 1) return 0;
     const size_t slots = static_cast<size_t>(a.B * a.Hkv) * splits;
-    return slots * (kMaxRows * kD + 2 * kMaxRows) * sizeof(float);
+    return slots * (kMaxRows * a.D + 2 * kMaxRows) * sizeof(float);
 }
 
 int launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s) {
@@ -395,30 +401,33 @@ int launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s) {
     p.scale_log2 = static_cast<float>(a.scale * 1.4426950408889634);
     const size_t slots = static_cast<size_t>(a.B * a.Hkv) * p.splits;
     p.part_o = static_cast<float*>(workspace);
-    p.part_ml = p.part_o ? p.part_o + slots * kMaxRows * kD : nullptr;
+    p.part_ml = p.part_o ? p.part_o + slots * kMaxRows * a.D : nullptr;
     const dim3 grid(p.splits, static_cast<unsigned>(a.B * a.Hkv));
     p.mask = static_cast<const unsigned char*>(a.mask);
     p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2]; p.ms_k = a.mask_strides[3];
     p.inv_scale = static_cast<float>(1.0 / a.scale);
     const bool bf = a.dtype == PARAS_BF16;
     const dim3 block(kThreads);
-    if (a.mask_kind == 0) {
-        if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t, 0>), grid, block, 0, s, p);
-        else    hipLaunchKernelGGL((decode_split_kernel<f16_t, 0>), grid, block, 0, s, p);
-    } else if (a.mask_kind == 1) {
-        if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t, 1>), grid, block, 0, s, p);
-        else    hipLaunchKernelGGL((decode_split_kernel<f16_t, 1>), grid, block, 0, s, p);
+    const dim3 g2(static_cast<unsigned>(a.B * a.Hkv), p.R);
+#define PARAS_DECODE_LAUNCH(T_, D_)                                                                        \
+    do {                                                                                                   \
+        if (a.mask_kind == 0)      hipLaunchKernelGGL((decode_split_kernel<T_, D_, 0>), grid, block, 0, s, p); \
+        else if (a.mask_kind == 1) hipLaunchKernelGGL((decode_split_kernel<T_, D_, 1>), grid, block, 0, s, p); \
+        else                       hipLaunchKernelGGL((decode_split_kernel<T_, D_, 2>), grid, block, 0, s, p); \
+        PARAS_HIP_TRY(hipGetLastError());                                                                  \
+        if (p.splits > 1) {                                                                                \
+            hipLaunchKernelGGL((decode_combine_kernel<T_, D_>), g2, dim3(D_), 0, s, p);                    \
+            PARAS_HIP_TRY(hipGetLastError());                                                              \
+        }                                                                                                  \
+    } while (0)
+    if (a.D == 128) {
+        if (bf) PARAS_DECODE_LAUNCH(bf16_t, 128);
+        else    PARAS_DECODE_LAUNCH(f16_t, 128);
     } else {
-        if (bf) hipLaunchKernelGGL((decode_split_kernel<bf16_t, 2>), grid, block, 0, s, p);
-        else    hipLaunchKernelGGL((decode_split_kernel<f16_t, 2>), grid, block, 0, s, p);
+        if (bf) PARAS_DECODE_LAUNCH(bf16_t, 64);
+        else    PARAS_DECODE_LAUNCH(f16_t, 64);
     }
-    PARAS_HIP_TRY(hipGetLastError());
-    if (p.splits > 1) {
-        const dim3 g2(static_cast<unsigned>(a.B * a.Hkv), p.R);
-        if (bf) hipLaunchKernelGGL((decode_combine_kernel<bf16_t>), g2, dim3(kD), 0, s, p);
-        else    hipLaunchKernelGGL((decode_combine_kernel<f16_t>), g2, dim3(kD), 0, s, p);
-        PARAS_HIP_TRY(hipGetLastError());
-    }
+#undef PARAS_DECODE_LAUNCH
     return PARAS_OK;
 }
 

@@ -14,7 +14,7 @@ bool flash_supported(const paras_sdpa_args& a);
 int  launch_flash(const paras_sdpa_args& a, hipStream_t s);
 
 // Split-KV decode: short query (Lq * Hq/Hkv <= 16), long K/V, bf16/f16,
-// D == Dv == 128, no explicit mask, not causal.
+// D == Dv in {64, 128}, optional bool / additive mask, not causal.
 bool   decode_supported(const paras_sdpa_args& a);
 size_t decode_workspace(const paras_sdpa_args& a);
 int    launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s);

@@ -170,6 +170,18 @@ def test_rms_norm_backward_many_rows_uses_taller_slabs():
         assert_bit_exact(gw, wgw, f"rms_norm grad_weight {rows}x{H}")
 
 
+def test_rms_norm_backward_general_path_with_more_than_a_million_rows():
+    """fp32 takes the three-kernel path, whose partial column sums are laid out one slab of 16 rows
+    per workgroup along grid x: more than 65535 slabs (1,048,560 rows) must work."""
+    rows, H = 16 * 65535 + 40, 8
+    x, w, go = torch.randn(rows, H), 1 + 0.1 * torch.randn(H), torch.randn(rows, H)
+    _, rstd = O.rms_norm(x, w, 1e-6)
+    gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(rstd))
+    wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
+    assert_bit_exact(gx, wgx, "rms_norm grad_input")
+    assert torch.allclose(gw.cpu(), wgw, rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_rms_norm_backward_adversarial_magnitudes(dtype):
     """The one-pass backward on rows built to break a shortcut in its arithmetic: products g*w and

@@ -103,12 +103,19 @@ def test_ffn_matches_oracle(shape, dtype):
     assert err.mean().item() < 1e-3
 
 
-def test_ffn_rejects_unsupported_sizes():
-    T, E, k = 16, 2, 1
-    with pytest.raises(capi.ParasError, match="multiples of 64"):
-        z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device="cuda")
-        route = capi.moe_route(torch.randn(T, E, device="cuda").bfloat16(), k)
-        capi.moe_ffn(z(T, 72), z(E, 64, 72), z(E, 64, 72), z(E, 72, 64), route[1], route[2], route[3], route[5], k)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(50, 3, 2, 72, 100), (33, 4, 1, 64, 40), (20, 2, 2, 7, 64)])
+def test_ffn_sizes_the_tiles_do_not_take(shape, dtype):
+    """Hidden or intermediate sizes that are not multiples of 64 run on the general kernels."""
+    T, E, k, H, I = shape
+    x, logits = torch.randn(T, H).to(dtype), torch.randn(T, E).to(dtype)
+    wg, wu = (0.1 * torch.randn(E, I, H)).to(dtype), (0.1 * torch.randn(E, I, H)).to(dtype)
+    wd = (0.1 * torch.randn(E, H, I)).to(dtype)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    r = O.moe_route(logits, k)
+    want = O.moe_ffn(x, wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
+    assert_ffn_close(out, want, dtype)
 
 
 def test_config5_routing_exact_and_sampled_tokens():

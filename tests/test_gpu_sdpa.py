@@ -377,6 +377,25 @@ def test_decode_matches_oracle(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 8, 2, 1, 1000), (1, 16, 1, 1, 4099), (3, 4, 4, 3, 300), (1, 2, 2, 1, 31)])
+def test_decode_head_size_64(dtype, shape):
+    """The split-KV decode kernel at head size 64 (half as many contraction steps and output blocks
+    per tile), with and without a key-padding mask."""
+    B, Hq, Hkv, Lq, Lk = shape
+    q, k, v = torch.randn(B, Hq, Lq, 64).to(dtype), torch.randn(B, Hkv, Lk, 64).to(dtype), torch.randn(B, Hkv, Lk, 64).to(dtype)
+    out, _, lse, kern = run(q, k, v, want_lse=True)
+    want, _ = O.sdpa_math(q, k, v, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split" and max_abs(out, want) <= ABS_16BIT
+    s = (q.float() @ k.float().repeat_interleave(Hq // Hkv, 1).transpose(-1, -2)) / 8.0
+    assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=1e-3, atol=1e-3)
+    keep = torch.ones(B, 1, 1, Lk, dtype=torch.bool)
+    keep[0, ..., Lk // 2:] = False
+    out, _, _, kern = run(q, k, v, mask=keep)
+    want, _ = O.sdpa_math(q, k, v, attn_mask=keep, enable_gqa=True, gemm="aten")
+    assert kern == "decode_split" and max_abs(out, want) <= ABS_16BIT
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_decode_with_masks_matches_oracle(dtype):
     """Ragged batches: decode with a key-padding mask [B,1,1,Lk], a per-head additive bias
     [B,Hq,1,Lk], a [Lq,Lk] mask for two query positions, a sequence whose first 3000 keys are all
