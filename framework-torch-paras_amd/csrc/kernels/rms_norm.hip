@@ -304,22 +304,28 @@ __device__ __forceinline__ double bwd_coef(double rr, int H, bool h_pow2, double
 // kFull: every thread of the workgroup owns a vector (H == 8 * BLOCK * NV).  Then no memory
 // instruction sits under a lane mask and the compiler can count exactly which of them a wait has
 // to cover: with a mask it waits, before the next row, for the row's own store as well.
-template <typename T, int NV, int BLOCK, bool kFull>
-__global__ __launch_bounds__(BLOCK, 4) void rms_norm_bwd_fused(
+template <typename T, int NV, int BLOCK, bool kFull, int kTeams = 1>
+__global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
     const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
     const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
     using E = Elem<T>;
     constexpr int V = 8;
     constexpr int kWaves = BLOCK / kWave;
-    __shared__ double slots[2 * kWaves];
+    __shared__ double slots[2 * kTeams * kWaves];
+    __shared__ double team_dw[kTeams > 1 ? BLOCK * NV * V : 1];
     const int nvec = H / V;
+    const int team = kTeams > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / BLOCK) : 0;
+    const int tid = kTeams > 1 ? static_cast<int>(threadIdx.x) - team * BLOCK : static_cast<int>(threadIdx.x);
     const long slab = blockIdx.x;
     // Rows are dealt out round-robin: workgroup b takes rows b, b + G, b + 2G, ... (G workgroups),
     // so the rows in flight at any moment are neighbours in memory and spread over every memory
     // channel.  (A contiguous slab per workgroup puts the workgroups, which advance in step, a
     // constant 2^k bytes apart: 82 us instead of 76 for 16384 x 4096.)
-    const long rstep = gridDim.x;
-    const long r0 = slab;
+    // With kTeams = 2 a workgroup is two teams of BLOCK threads, each with rows of its own (the
+    // launcher sees to it that all teams have equally many): one partial sum for both, so half as
+    // many to write and to add up.
+    const long rstep = static_cast<long>(gridDim.x) * kTeams;
+    const long r0 = slab * kTeams + team;
     const long r1 = rows;
     const double inv_h = 1.0 / static_cast<double>(H);   // only used where H is a power of two (exact)
     const bool h_pow2 = __builtin_amdgcn_readfirstlane((H & (H - 1)) == 0) != 0;
@@ -333,14 +339,14 @@ __global__ __launch_bounds__(BLOCK, 4) void rms_norm_bwd_fused(
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i]) {
-                const int c = threadIdx.x + i * BLOCK;
+                const int c = tid + i * BLOCK;
                 gs[i] = load16_nt(go + r * H + static_cast<long>(c) * V);
                 xs[i] = load16_nt(x + r * H + static_cast<long>(c) * V);
             }
     };
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int c = threadIdx.x + i * BLOCK;
+        const int c = tid + i * BLOCK;
         have[i] = kFull || c < nvec;
         u32x4 wv = {0u, 0u, 0u, 0u};
         if (have[i]) wv = load16(w + static_cast<long>(c) * V);
@@ -366,8 +372,8 @@ __global__ __launch_bounds__(BLOCK, 4) void rms_norm_bwd_fused(
         if (r + rstep < r1) request(r + rstep);
         {   // sum over the workgroup; two alternating slot sets, so one barrier per row
             dot = wave_sum(dot);
-            double* slot = slots + (sum_calls++ & 1) * kWaves;
-            if ((threadIdx.x & (kWave - 1)) == 0) slot[threadIdx.x / kWave] = dot;
+            double* slot = slots + ((sum_calls++ & 1) * kTeams + team) * kWaves;
+            if ((tid & (kWave - 1)) == 0) slot[tid / kWave] = dot;
             lds_barrier();   // not __syncthreads(): the loads requested above stay in flight across it
             dot = 0.0;
 #pragma unroll
@@ -377,7 +383,7 @@ __global__ __launch_bounds__(BLOCK, 4) void rms_norm_bwd_fused(
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i])
-                store16_nt(gx + r * H + static_cast<long>(threadIdx.x + i * BLOCK) * V, bwd_vec_second<T>(g64[i], x64[i], w64[i], rr, cd));
+                store16_nt(gx + r * H + static_cast<long>(tid + i * BLOCK) * V, bwd_vec_second<T>(g64[i], x64[i], w64[i], rr, cd));
     };
     // The first row is written out in front of the loop: entered straight from the prologue, the
     // loop header would inherit "first loads pending" and the compiler's wait insertion would then
@@ -385,10 +391,25 @@ __global__ __launch_bounds__(BLOCK, 4) void rms_norm_bwd_fused(
     // after a peeled row both ways into the header look alike (a row requested, a store in flight).
     do_row(r0);
     for (long r = r0 + rstep; r < r1; r += rstep) do_row(r);
+    if constexpr (kTeams > 1) {
+        // team 1 hands its column sums to team 0 through LDS
+        if (team == 1) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int j = 0; j < V; ++j) team_dw[(i * V + j) * BLOCK + tid] = dw[i][j];
+        }
+        __syncthreads();
+        if (team == 1) return;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int j = 0; j < V; ++j) dw[i][j] += team_dw[(i * V + j) * BLOCK + tid];
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i)
         if (have[i]) {
-            double* dst = partial + slab * H + static_cast<long>(threadIdx.x + i * BLOCK) * V;
+            double* dst = partial + slab * H + static_cast<long>(tid + i * BLOCK) * V;
 #pragma unroll
             for (int j = 0; j < V; ++j) dst[j] = dw[i][j];
         }
@@ -407,8 +428,18 @@ __global__ __launch_bounds__(kDwFinalLanes * kDwFinalCols) void rms_norm_bwd_dw_
     const int c = threadIdx.x % kDwFinalCols, l = threadIdx.x / kDwFinalCols;
     const long j = static_cast<long>(blockIdx.x) * kDwFinalCols + c;
     double acc = 0.0;
-    if (j < H)
-        for (long sl = l; sl < slabs; sl += kDwFinalLanes) acc += partial[sl * H + j];
+    if (j < H) {
+        // eight loads in flight at a time, added in slab order
+        long sl = l;
+        for (; sl + 7 * kDwFinalLanes < slabs; sl += 8 * kDwFinalLanes) {
+            double v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(sl + u * kDwFinalLanes) * H + j];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; sl < slabs; sl += kDwFinalLanes) acc += partial[sl * H + j];
+    }
     part[l][c] = acc;
     __syncthreads();
     if (l == 0 && j < H) {
@@ -474,17 +505,25 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
             int dev = 0;
             (void)hipGetDevice(&dev);
             auto* dst = DeviceContext::instance().device(dev);
-            const long resident = 2 * (dst ? dst->compute_units : 256);
-            if (slabs > resident) slabs = resident;
+            const long cus = dst ? dst->compute_units : 256;
+            if (slabs > 2 * cus) slabs = 2 * cus;
+            // Rows of 4096 elements, plenty of them: workgroups of two teams of 512 threads, one
+            // workgroup per compute unit, when the rows divide evenly among the teams.
+            const bool teams = nvec == 512 && slabs == 2 * cus && rows % (2 * cus) == 0;
+            if (teams) slabs = cus;
             const dim3 grid(static_cast<unsigned>(slabs));
 #define PARAS_BWD_LAUNCH(BLOCK_, FULL_) \
     hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, FULL_>), grid, dim3(BLOCK_), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
-            if (nvec == kBlock)      PARAS_BWD_LAUNCH(kBlock, true);
+#define PARAS_BWD_LAUNCH_TEAMS(BLOCK_) \
+    hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, true, 2>), grid, dim3(2 * BLOCK_), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
+            if (teams)               PARAS_BWD_LAUNCH_TEAMS(512);
+            else if (nvec == kBlock) PARAS_BWD_LAUNCH(kBlock, true);
             else if (nvec < kBlock)  PARAS_BWD_LAUNCH(kBlock, false);
             else if (nvec == 512)    PARAS_BWD_LAUNCH(512, true);
             else if (nvec < 512)     PARAS_BWD_LAUNCH(512, false);
             else if (nvec == 1024)   PARAS_BWD_LAUNCH(1024, true);   // rows of up to 8192 elements
             else                     PARAS_BWD_LAUNCH(1024, false);
+#undef PARAS_BWD_LAUNCH_TEAMS
 #undef PARAS_BWD_LAUNCH
             PARAS_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + kDwFinalCols - 1) / kDwFinalCols)), dim3(kDwFinalLanes * kDwFinalCols), 0, s,

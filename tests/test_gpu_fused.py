@@ -156,11 +156,11 @@ def test_rms_norm_backward_one_pass_kernel(shape, dtype):
     assert_bit_exact(gw, wgw, "rms_norm grad_weight")
 
 
-def test_rms_norm_backward_many_rows_uses_taller_slabs():
-    """From 16384 rows on the one-pass kernel gives a workgroup 32 rows instead of 16 (half the
-    partial column sums); the last slab here is ragged, and a row count just below the switch runs
-    beside it."""
-    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520)):
+def test_rms_norm_backward_many_rows_are_dealt_round_robin():
+    """The one-pass kernel runs at most two workgroups per compute unit; with more rows than that
+    times 16 every workgroup takes rows b, b + G, b + 2G, ...: row counts around the switch, with
+    workgroups that get one row more than others."""
+    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520), (8192 + 7, 264)):
         torch.manual_seed(rows)
         x, w, go = torch.randn(rows, H).bfloat16(), (1 + 0.1 * torch.randn(H)).bfloat16(), torch.randn(rows, H).bfloat16()
         _, rstd = O.rms_norm(x, w, 1e-6)
@@ -168,6 +168,22 @@ def test_rms_norm_backward_many_rows_uses_taller_slabs():
         wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
         assert_bit_exact(gx, wgx, f"rms_norm grad_input {rows}x{H}")
         assert_bit_exact(gw, wgw, f"rms_norm grad_weight {rows}x{H}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows", [8192, 8192 + 512, 8192 + 100])
+def test_rms_norm_backward_rows_of_4096_in_two_team_workgroups(rows, dtype):
+    """Rows of 4096 elements whose count is a multiple of twice the compute units (512) run in
+    workgroups of two teams of 512 threads that share one partial column sum; 8192 + 100 rows do
+    not divide evenly and take the one-team workgroups."""
+    H = 4096
+    torch.manual_seed(rows)
+    x, w, go = torch.randn(rows, H).to(dtype), (1 + 0.1 * torch.randn(H)).to(dtype), torch.randn(rows, H).to(dtype)
+    _, rstd = O.rms_norm(x, w, 1e-6)
+    gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(rstd))
+    wgx, wgw = O.rms_norm_backward(go, x, w, rstd)
+    assert_bit_exact(gx, wgx, f"rms_norm grad_input {rows}x{H}")
+    assert_bit_exact(gw, wgw, f"rms_norm grad_weight {rows}x{H}")
 
 
 def test_rms_norm_backward_general_path_with_more_than_a_million_rows():
