@@ -271,6 +271,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
                                                      lane_off + (first + r0) * row_bytes, 0, 0, 0);
         }
     };
+    auto stage_one = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile, int i) {
+        const int r0 = i * RPI * NW;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)(tile + (r0 + wave * RPI) * D), 16,
+                                                 lane_off + (first + r0) * row_bytes, 0, 0, 0);
+    };
     // Requests the pair tile t's blocks need beyond K tile t: K tile t+1 and V tile t (`par` = parity of t).
     auto stage_pair = [&](int t, auto par) {
         stage_rows(k_rsrc, k_lane, k_row_bytes, (t + 1) * kBN - 32, kbuf(par, true));
@@ -443,8 +448,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         fetch(j, s0, par);
         fetch(j, s0 + 1, par);
     };
-    auto block = [&](int j, float16_t (&cur)[QB], float16_t (&nxt)[QB], auto next_tag, auto tail, auto par) {
+    auto block = [&](int j, float16_t (&cur)[QB], float16_t (&nxt)[QB], auto next_tag, auto tail, auto par, auto stage_tag) {
         constexpr bool kNext = decltype(next_tag)::value;
+        constexpr bool kStage = decltype(stage_tag)::value;
         constexpr bool kTail = !std::is_same<decltype(tail), NoTail>::value;
         constexpr int S0 = kNext ? 0 : KSTEPS;           // first slot that exists
         static_assert(QB == 1, "the max tree below is written for one query block per wave");
@@ -499,6 +505,17 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
                 for (int qb = 0; qb < QB; ++qb)
                     oacc[qb][db] = Mma<T>::run(frag[c % 4], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
             }
+            if constexpr (kStage) {
+                // The next tile pair (K tile t+2, V tile t+1), one request every other slot: all of
+                // them at the start of the tile, from every wave at once right after the barrier,
+                // cost 1.5 % (they queue up in front of the waves' first MFMAs).
+                static_assert(2 * (2 * NI - 1) < NS, "the requests fit the block's slots");
+                if (c % 2 == 0 && c / 2 < 2 * NI) {
+                    const int i = c / 2, t = j >> 1;
+                    if (i < NI) stage_one(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN - 32, kbuf(par, false), i);
+                    else        stage_one(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true), i - NI);
+                }
+            }
             if (c + 2 < NS) fetch(j, c + 2, par);
             else if constexpr (kTail)    // only ever the second block of the same tile: same parity
                 fetch(j + 1, (std::is_same<decltype(tail), KFirst>::value ? 0 : KSTEPS) + (c + 2 - NS), par);
@@ -543,14 +560,12 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         finish_scores(0, s_a, mx, m0);
     }
     // One tile of the main loop (`par` = parity of t, a compile-time name for the buffers; two
-    // tiles per trip).  The first fragment reads are in flight while the next pair is requested.
+    // tiles per trip).  The tile's first block also requests the next tile pair (= stage_pair(t + 1)).
     auto tile = [&](int t, auto par) {
         first_fetches(2 * t, KFirst{}, par);
         __builtin_amdgcn_sched_barrier(0);                // keep the reads ahead of the requests
-        stage_rows(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN - 32, kbuf(par, false));   // = stage_pair(t + 1)
-        stage_rows(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true));
-        block(2 * t, s_a, s_b, Yes{}, KFirst{}, par);
-        block(2 * t + 1, s_b, s_a, Yes{}, NoTail{}, par); // its successor's K rows arrive with the barrier below
+        block(2 * t, s_a, s_b, Yes{}, KFirst{}, par, Yes{});
+        block(2 * t + 1, s_b, s_a, Yes{}, NoTail{}, par, No{}); // its successor's K rows arrive with the barrier below
         publish();
     };
     int t_main = 0;
@@ -571,11 +586,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
         const int second0 = (2 * t + 1) * 32;
         if (second0 >= p.Lk || (kCausal && second0 > q0 + WQ - 1)) {
             first_fetches(2 * t, VFirst{}, par);
-            block(2 * t, s_a, s_b, No{}, NoTail{}, par);
+            block(2 * t, s_a, s_b, No{}, NoTail{}, par, No{});
         } else {
             first_fetches(2 * t, KFirst{}, par);
-            block(2 * t, s_a, s_b, Yes{}, VFirst{}, par);
-            block(2 * t + 1, s_b, s_a, No{}, NoTail{}, par);
+            block(2 * t, s_a, s_b, Yes{}, VFirst{}, par, No{});
+            block(2 * t + 1, s_b, s_a, No{}, NoTail{}, par, No{});
         }
         publish();
     }
