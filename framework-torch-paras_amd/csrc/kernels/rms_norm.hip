@@ -312,7 +312,7 @@ __global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
     constexpr int V = 8;
     constexpr int kWaves = BLOCK / kWave;
     __shared__ double slots[2 * kTeams * kWaves];
-    __shared__ double team_dw[kTeams > 1 ? BLOCK * NV * V : 1];
+    __shared__ double team_dw[kTeams > 1 ? (kTeams - 1) * BLOCK * NV * V : 1];
     const int nvec = H / V;
     const int team = kTeams > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / BLOCK) : 0;
     const int tid = kTeams > 1 ? static_cast<int>(threadIdx.x) - team * BLOCK : static_cast<int>(threadIdx.x);
@@ -321,9 +321,9 @@ __global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
     // so the rows in flight at any moment are neighbours in memory and spread over every memory
     // channel.  (A contiguous slab per workgroup puts the workgroups, which advance in step, a
     // constant 2^k bytes apart: 82 us instead of 76 for 16384 x 4096.)
-    // With kTeams = 2 a workgroup is two teams of BLOCK threads, each with rows of its own (the
-    // launcher sees to it that all teams have equally many): one partial sum for both, so half as
-    // many to write and to add up.
+    // With kTeams > 1 a workgroup is several teams of BLOCK threads, each with rows of its own (the
+    // launcher sees to it that all teams have equally many): one partial sum for all of them, so
+    // fewer to write and to add up.
     const long rstep = static_cast<long>(gridDim.x) * kTeams;
     const long r0 = slab * kTeams + team;
     const long r1 = rows;
@@ -392,19 +392,21 @@ __global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
     do_row(r0);
     for (long r = r0 + rstep; r < r1; r += rstep) do_row(r);
     if constexpr (kTeams > 1) {
-        // team 1 hands its column sums to team 0 through LDS
-        if (team == 1) {
+        // the other teams hand their column sums to team 0 through LDS; added in team order
+        if (team > 0) {
 #pragma unroll
             for (int i = 0; i < NV; ++i)
 #pragma unroll
-                for (int j = 0; j < V; ++j) team_dw[(i * V + j) * BLOCK + tid] = dw[i][j];
+                for (int j = 0; j < V; ++j) team_dw[((team - 1) * NV * V + i * V + j) * BLOCK + tid] = dw[i][j];
         }
         __syncthreads();
-        if (team == 1) return;
+        if (team > 0) return;
 #pragma unroll
-        for (int i = 0; i < NV; ++i)
+        for (int tm = 1; tm < kTeams; ++tm)
 #pragma unroll
-            for (int j = 0; j < V; ++j) dw[i][j] += team_dw[(i * V + j) * BLOCK + tid];
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int j = 0; j < V; ++j) dw[i][j] += team_dw[((tm - 1) * NV * V + i * V + j) * BLOCK + tid];
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i)
@@ -500,23 +502,28 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
             auto* gx16 = static_cast<std::uint16_t*>(gx);
             auto* part = static_cast<double*>(workspace);
             // One workgroup per kDwSlabRows rows (the workspace is sized for that many partial sums)
-            // up to two per compute unit -- what is resident at once: beyond that a workgroup takes
-            // more rows instead, so the partial sums to write and to add up stop growing.
+            // up to what is resident at once (four waves per SIMD: 4, 2 or 1 workgroups per compute
+            // unit): beyond that a workgroup takes more rows instead, so the partial sums to write and
+            // to add up stop growing.
             int dev = 0;
             (void)hipGetDevice(&dev);
             auto* dst = DeviceContext::instance().device(dev);
             const long cus = dst ? dst->compute_units : 256;
-            if (slabs > 2 * cus) slabs = 2 * cus;
-            // Rows of 4096 elements, plenty of them: workgroups of two teams of 512 threads, one
-            // workgroup per compute unit, when the rows divide evenly among the teams.
-            const bool teams = nvec == 512 && slabs == 2 * cus && rows % (2 * cus) == 0;
+            const long resident = (nvec <= kBlock ? 4 : nvec <= 512 ? 2 : 1) * cus;
+            const bool plenty = slabs >= resident;
+            if (plenty) slabs = resident;
+            // Rows of 2048 or 4096 elements, plenty of them: workgroups of 1024 threads in teams of
+            // one row's width (4 x 256 or 2 x 512), one workgroup per compute unit, when the rows
+            // divide evenly among the teams.
+            const bool teams = (nvec == 512 || nvec == kBlock) && plenty && rows % resident == 0;
             if (teams) slabs = cus;
             const dim3 grid(static_cast<unsigned>(slabs));
 #define PARAS_BWD_LAUNCH(BLOCK_, FULL_) \
     hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, FULL_>), grid, dim3(BLOCK_), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
 #define PARAS_BWD_LAUNCH_TEAMS(BLOCK_) \
-    hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, true, 2>), grid, dim3(2 * BLOCK_), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
-            if (teams)               PARAS_BWD_LAUNCH_TEAMS(512);
+    hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, true, 1024 / BLOCK_>), grid, dim3(1024), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
+            if (teams && nvec == 512) PARAS_BWD_LAUNCH_TEAMS(512);
+            else if (teams)          PARAS_BWD_LAUNCH_TEAMS(kBlock);
             else if (nvec == kBlock) PARAS_BWD_LAUNCH(kBlock, true);
             else if (nvec < kBlock)  PARAS_BWD_LAUNCH(kBlock, false);
             else if (nvec == 512)    PARAS_BWD_LAUNCH(512, true);

@@ -171,12 +171,13 @@ def test_rms_norm_backward_many_rows_are_dealt_round_robin():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("rows", [8192, 8192 + 512, 8192 + 100])
-def test_rms_norm_backward_rows_of_4096_in_two_team_workgroups(rows, dtype):
-    """Rows of 4096 elements whose count is a multiple of twice the compute units (512) run in
-    workgroups of two teams of 512 threads that share one partial column sum; 8192 + 100 rows do
-    not divide evenly and take the one-team workgroups."""
-    H = 4096
+@pytest.mark.parametrize("shape", [(8192, 4096), (8192 + 512, 4096), (8192 + 100, 4096), (16384, 2048), (16384 + 1024, 2048),
+                                   (16384 + 24, 2048)])
+def test_rms_norm_backward_team_workgroups(shape, dtype):
+    """Rows of 4096 (2048) elements whose count is a multiple of 2 (4) per compute unit run in
+    workgroups of 2 (4) teams that share one partial column sum; the row counts that do not divide
+    evenly take the one-team workgroups."""
+    rows, H = shape
     torch.manual_seed(rows)
     x, w, go = torch.randn(rows, H).to(dtype), (1 + 0.1 * torch.randn(H)).to(dtype), torch.randn(rows, H).to(dtype)
     _, rstd = O.rms_norm(x, w, 1e-6)
