@@ -173,9 +173,16 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
     for (int i = 0; i < DB; ++i) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
+    // Every wave starts at a tile of its own within its range and wraps around: the workgroups and
+    // waves, which advance in step, would otherwise always be the same power of two apart in memory.
+    const int rot = n_tiles > 1 ? (pair * 5 + split * 3 + wave * 7) % n_tiles : 0;
+    auto tile_of = [&](int t) {
+        const int tt = t + rot;
+        return tt >= n_tiles ? tt - n_tiles : tt;
+    };
     if (n_tiles > 0) {
-        load_k(0, kcur);
-        load_v(0);
+        load_k(tile_of(0), kcur);
+        load_v(tile_of(0));
         store_v(0);
     }
     // ds_read_tr lane offsets: group lg reads keys 4*lg + (m/4) (+16), 4 d's at 4*(m%4)
@@ -184,8 +191,8 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
         if (t + 1 < n_tiles) {
-            load_k(t + 1, knext);
-            load_v(t + 1);
+            load_k(tile_of(t + 1), knext);
+            load_v(tile_of(t + 1));
         }
         // S^T for two 16-key blocks
         float4_t sacc[2];
@@ -195,7 +202,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) sacc[kb] = Mma16<T>::run(kcur[kb][ks], qreg[ks], sacc[kb]);
         }
-        const int key0 = k_begin + t * kTile;
+        const int key0 = k_begin + tile_of(t) * kTile;
         if constexpr (kMask != 0) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
