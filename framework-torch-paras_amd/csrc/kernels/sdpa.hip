@@ -12,7 +12,7 @@
 namespace paras {
 namespace {
 
-enum class SdpaKernel { Flash, Decode, Weights, Generic };
+enum class SdpaKernel { Flash, Decode, Weights, Padded, Generic };
 
 int validate(const paras_sdpa_args* a) {
     PARAS_REQUIRE(a != nullptr, "paras sdpa: null argument block");
@@ -31,11 +31,82 @@ int validate(const paras_sdpa_args* a) {
 
 bool empty_output(const paras_sdpa_args& a) { return a.B == 0 || a.Hq == 0 || a.Lq == 0 || a.Dv == 0; }
 
+// 16-bit head sizes below 128 other than 64: the MFMA kernels exist for 64 and 128, so q, k and v
+// are copied into the workspace with zero columns appended (q.k and the first D output columns do
+// not change; the scale is the caller's, i.e. that of the real head size) and the first D columns
+// of the padded result are copied out -- instead of the general fp64 kernel, three orders of
+// magnitude slower.
+struct PaddedPlan {
+    paras_sdpa_args inner;      // the padded problem; its pointers are offsets into the workspace until bound
+    size_t q_off, k_off, v_off, out_off, inner_off, total;
+};
+size_t up256(size_t n) { return (n + 255) / 256 * 256; }
+
+bool plan_padded(const paras_sdpa_args& a, PaddedPlan* plan) {
+    if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
+    if (a.attn != nullptr || a.D != a.Dv || a.D < 1 || a.D >= 128 || a.D == 64) return false;
+    if (a.Lq < 1 || a.Lk < 1) return false;
+    const int64_t Dp = a.D < 64 ? 64 : 128;
+    PaddedPlan pl{};
+    pl.inner = a;
+    pl.inner.D = pl.inner.Dv = Dp;
+    const int64_t qs[3] = {a.Hq * a.Lq * Dp, a.Lq * Dp, Dp}, ks[3] = {a.Hkv * a.Lk * Dp, a.Lk * Dp, Dp};
+    for (int i = 0; i < 3; ++i) {
+        pl.inner.q_strides[i] = qs[i];
+        pl.inner.k_strides[i] = ks[i];
+        pl.inner.v_strides[i] = ks[i];
+    }
+    size_t off = 0;
+    pl.q_off = off;   off += up256(static_cast<size_t>(a.B * a.Hq * a.Lq * Dp) * 2);
+    pl.k_off = off;   off += up256(static_cast<size_t>(a.B * a.Hkv * a.Lk * Dp) * 2);
+    pl.v_off = off;   off += up256(static_cast<size_t>(a.B * a.Hkv * a.Lk * Dp) * 2);
+    pl.out_off = off; off += up256(static_cast<size_t>(a.B * a.Hq * a.Lq * Dp) * 2);
+    pl.inner_off = off;
+    // the support checks look at pointer alignment: stand-ins with the alignment the bound ones will have
+    char* const fake = reinterpret_cast<char*>(static_cast<uintptr_t>(256));
+    pl.inner.q = fake; pl.inner.k = fake; pl.inner.v = fake; pl.inner.out = fake;
+    size_t inner_ws = 0;
+    if (decode_supported(pl.inner)) inner_ws = decode_workspace(pl.inner);
+    else if (!flash_supported(pl.inner)) return false;
+    pl.total = off + up256(inner_ws);
+    if (plan) *plan = pl;
+    return true;
+}
+
 SdpaKernel choose(const paras_sdpa_args& a) {
     if (decode_supported(a)) return SdpaKernel::Decode;
     if (flash_supported(a)) return SdpaKernel::Flash;
     if (weights_supported(a)) return SdpaKernel::Weights;
+    if (plan_padded(a, nullptr)) return SdpaKernel::Padded;
     return SdpaKernel::Generic;
+}
+
+int launch_padded(const paras_sdpa_args& a, void* workspace, void* stream, hipStream_t s) {
+    PaddedPlan pl;
+    PARAS_REQUIRE(plan_padded(a, &pl), "paras sdpa: not a shape for the padded route");
+    PARAS_REQUIRE(workspace != nullptr, "paras sdpa: workspace is null");
+    PARAS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "paras sdpa: the workspace must be 256-byte aligned");
+    char* ws = static_cast<char*>(workspace);
+    paras_sdpa_args in = pl.inner;
+    in.q = ws + pl.q_off; in.k = ws + pl.k_off; in.v = ws + pl.v_off; in.out = ws + pl.out_off;
+    const int64_t Dp = in.D, one = 1;
+    // zeros (a fill kernel: the caller may be capturing this stream), then the real columns
+    const int64_t zero_elems = static_cast<int64_t>(pl.out_off / 2);      // q, k, v regions
+    int rc = paras_fill_strided(ws, 1, &zero_elems, &one, 2, 0, stream);
+    if (rc != PARAS_OK) return rc;
+    auto copy_in = [&](const void* src, const int64_t (&st)[3], void* dst, int64_t H, int64_t L) {
+        const int64_t sizes[4] = {a.B, H, L, a.D}, ss[4] = {st[0], st[1], st[2], 1}, ds[4] = {H * L * Dp, L * Dp, Dp, 1};
+        return paras_copy_strided(src, dst, 4, sizes, ss, ds, 2, a.dtype, a.dtype, stream);
+    };
+    if ((rc = copy_in(a.q, a.q_strides, const_cast<void*>(in.q), a.Hq, a.Lq)) != PARAS_OK) return rc;
+    if ((rc = copy_in(a.k, a.k_strides, const_cast<void*>(in.k), a.Hkv, a.Lk)) != PARAS_OK) return rc;
+    if ((rc = copy_in(a.v, a.v_strides, const_cast<void*>(in.v), a.Hkv, a.Lk)) != PARAS_OK) return rc;
+    if (decode_supported(in)) rc = launch_decode(in, ws + pl.inner_off, s);
+    else                      rc = launch_flash(in, s);
+    if (rc != PARAS_OK) return rc;
+    const int64_t sizes[4] = {a.B, a.Hq, a.Lq, a.D}, ss[4] = {a.Hq * a.Lq * Dp, a.Lq * Dp, Dp, 1},
+                  ds[4] = {a.Hq * a.Lq * a.D, a.Lq * a.D, a.D, 1};
+    return paras_copy_strided(in.out, a.out, 4, sizes, ss, ds, 2, a.dtype, a.dtype, stream);
 }
 
 }  // namespace
@@ -50,6 +121,7 @@ const char* paras_sdpa_kernel_name(const paras_sdpa_args* args) {
         case SdpaKernel::Flash:  return "flash_mfma";
         case SdpaKernel::Decode: return "decode_split";
         case SdpaKernel::Weights: return "math_mfma";
+        case SdpaKernel::Padded: return "padded_mfma";
         default:                 return "generic";
     }
 }
@@ -60,6 +132,10 @@ size_t paras_sdpa_workspace(const paras_sdpa_args* args) {
     switch (choose(*args)) {
         case SdpaKernel::Decode:  return decode_workspace(*args);
         case SdpaKernel::Generic: return generic_workspace(*args);
+        case SdpaKernel::Padded: {
+            PaddedPlan pl;
+            return plan_padded(*args, &pl) ? pl.total : 0;
+        }
         default:                  return 0;
     }
 }
@@ -84,6 +160,7 @@ int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream) {
     switch (choose(a)) {
         case SdpaKernel::Flash: return launch_flash(a, s);
         case SdpaKernel::Weights: return launch_weights(a, s);
+        case SdpaKernel::Padded: return launch_padded(a, workspace, stream, s);
         case SdpaKernel::Decode:
             PARAS_REQUIRE(workspace != nullptr || decode_workspace(a) == 0, "paras sdpa: workspace is null");
             return launch_decode(a, workspace, s);

@@ -174,33 +174,8 @@ OverrideableResult sdpa_overrideable(const Tensor& query, const Tensor& key, con
     (void)return_debug_mask;
     Prepared p;
     prepare(query, key, value, attn_bias, is_causal, scale, /*enable_gqa=*/true, &p);
-    // The MFMA kernels exist for head sizes 64 and 128.  Other 16-bit head sizes up to 128 are run
-    // on them with zero columns appended to q, k and v (q.k and the first D output columns do not
-    // change; the scale stays that of the real head size) rather than on the generic fp64 kernel,
-    // which is three orders of magnitude slower.
-    const int64_t D = p.a.D;
-    const bool sixteen_bit = query.scalar_type() == c10::kBFloat16 || query.scalar_type() == c10::kHalf;
-    if (sixteen_bit && D == p.a.Dv && D != 64 && D != 128 && D >= 1 && D < 128 && p.a.Lq > 0 && p.a.Lk > 0) {
-        const int64_t Dp = D < 64 ? 64 : 128;
-        auto padded = [&](const Tensor& t) {
-            Tensor z = empty_paras({t.size(0), t.size(1), t.size(2), Dp}, t.scalar_type(), t.device());
-            z.zero_();
-            z.narrow(3, 0, D).copy_(t);
-            return z;
-        };
-        const Tensor q2 = padded(p.q), k2 = padded(p.k), v2 = padded(p.v);
-        const double s = scale.has_value() ? *scale : 1.0 / std::sqrt(static_cast<double>(D));
-        Prepared pp;
-        prepare(q2, k2, v2, attn_bias, is_causal, s, /*enable_gqa=*/true, &pp);
-        Tensor out2, lse2;
-        run(&pp, &out2, nullptr, &lse2);
-        std::vector<int64_t> lse_shape(p.out_shape.begin(), p.out_shape.end() - 1);
-        const auto opts = query.options();
-        Tensor none = at::empty({0}, opts.dtype(c10::kLong));
-        return {out2.narrow(3, 0, D).contiguous().reshape(p.out_shape), lse2.reshape(lse_shape), none, none,
-                c10::SymInt(p.a.Lq), c10::SymInt(p.a.Lk), at::empty({0}, opts.dtype(c10::kLong)),
-                at::empty({0}, opts.dtype(c10::kLong)), at::empty({0}, opts)};
-    }
+    // (16-bit head sizes below 128 other than 64 run on the MFMA kernels too: the library pads q, k
+    // and v with zero columns inside its workspace.)
     Tensor out, lse;
     run(&p, &out, nullptr, &lse);
     std::vector<int64_t> lse_shape(p.out_shape.begin(), p.out_shape.end() - 1);

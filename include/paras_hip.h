@@ -236,7 +236,10 @@ PARAS_API size_t paras_sdpa_workspace(const paras_sdpa_args* args);
 /* `workspace` may be NULL when paras_sdpa_workspace() returned 0. */
 PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream);
 /* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma", "decode_split",
- * "math_mfma" (bf16 / f16 with the weights returned) or "generic". */
+ * "math_mfma" (bf16 / f16 with the weights returned), "padded_mfma" (bf16 / f16
+ * head sizes below 128 other than 64: q, k, v copied into the workspace with
+ * zero columns up to 64 or 128, then flash_mfma / decode_split; the workspace
+ * must be 256-byte aligned) or "generic". */
 PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 
 /* ------------------------------------------------------------------------- */

@@ -64,11 +64,12 @@ def test_golden_vectors_generic_kernel(tag):
         else:
             assert_bit_exact(attn, c[f"attn_{name}"], f"{tag} {name} weights")
             one_ulp_of_the_gemm(out, c[f"out_{name}"])
-    out, _, _, _ = run(q, c["kg"], c["vg"])
+    out, _, _, kern = run(q, c["kg"], c["vg"])
     if tag == "f32":
-        assert rel_err(out, c["out_gqa"]) <= REL_F32
+        assert kern == "generic" and rel_err(out, c["out_gqa"]) <= REL_F32
     else:
-        one_ulp_of_the_gemm(out, c["out_gqa"])
+        # no weights asked for and 16 bits: the head size is padded to 64 and the flash kernel runs
+        assert kern == "padded_mfma" and max_abs(out, c["out_gqa"]) <= ABS_16BIT
 
 
 @pytest.mark.parametrize("tag", ("bf16", "f16"))
@@ -502,3 +503,31 @@ def test_config4_shape_slice_and_gqa_equivalence():
     assert max_abs(out[:8], rep.cpu()) <= 4e-3
     ones, _, _, _ = capi.sdpa(qd, kd, torch.ones_like(vd))
     assert (ones.float() - 1).abs().max().item() <= 2 ** -7
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case_", [
+    # B, Hq, Hkv, Lq, Lk, D, causal, mask
+    (2, 4, 4, 200, 200, 80, True, None), (1, 8, 2, 130, 130, 96, False, None), (2, 2, 1, 77, 300, 40, False, "bool"),
+    (1, 4, 4, 64, 64, 100, True, None), (2, 8, 2, 1, 900, 96, False, None), (1, 4, 1, 2, 700, 48, False, "add"),
+    (1, 2, 2, 50, 50, 1, False, None), (1, 2, 2, 33, 65, 127, True, None)])
+def test_head_sizes_between_the_mfma_kernels_are_padded_inside_the_library(case_, dtype):
+    """16-bit head sizes below 128 other than 64, through the C ABI: the library copies q, k, v into
+    its workspace with zero columns appended and runs the flash / decode kernels (prefill and decode
+    shapes, GQA, causal, bool and additive masks, strided inputs)."""
+    B, Hq, Hkv, Lq, Lk, D, causal, mk = case_
+    torch.manual_seed(Lk + D)
+    q = torch.randn(B, Lq, Hq, D).to(dtype).transpose(1, 2)            # heads and rows swapped in memory
+    k, v = torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
+    mask = None
+    if mk == "bool":
+        mask = torch.rand(B, 1, Lq, Lk) > 0.3
+        mask[..., 0] = True
+    elif mk == "add":
+        mask = torch.randn(1, Hq, Lq, Lk).to(dtype)
+    scale = O.round_to_dtype(1.0 / math.sqrt(D), dtype)
+    out, _, lse, name = run(q, k, v, is_causal=causal, mask=mask, scale=scale, want_lse=True)
+    want, _ = O.sdpa_math(q, k, v, is_causal=causal, attn_mask=mask, scale=scale, enable_gqa=True, gemm="aten")
+    assert name == "padded_mfma" and out.shape == (B, Hq, Lq, D)
+    assert max_abs(out, want) <= ABS_16BIT
+    assert bool(torch.isfinite(lse).all())
