@@ -19,6 +19,8 @@
 // and meets the other workgroups at a counter in device memory (a bounded wait); then
 // every workgroup adds up the counts of all workgroups (expert offsets) and of the
 // workgroups before it (its own start positions) and scatters its (token, slot) pairs.
+// A workgroup whose wait runs out (the others kept off the chip by unrelated work) does
+// not depend on them any more: it counts every token's choices itself, from the logits.
 // The counter is cleared by a one-workgroup fill kernel queued in front.
 //
 // More tokens than that: three launches over 256-token workgroups,
@@ -30,6 +32,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 
 #include "core/device_context.h"
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(kBlock) void route_scatter_kernel(const long* __res
 constexpr int  kScratchHeader   = 256;
 constexpr int  kFusedMaxBlocks  = 256;          // 256-thread workgroups: all resident on 256 CUs
 constexpr long kFusedMaxTokens  = static_cast<long>(kFusedMaxBlocks) * kBlock;
-constexpr int  kSpinLimit       = 1 << 22;      // polls of ~64 clocks each: seconds, then give up
+constexpr int  kSpinLimit       = 1 << 20;      // polls of ~64 clocks each: tens of milliseconds, then the workgroup counts for itself
 
 __global__ __launch_bounds__(64) void route_clear_kernel(unsigned* __restrict__ header) {
     if (threadIdx.x < 2) header[threadIdx.x] = 0u;
@@ -191,6 +194,7 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     __shared__ long tot[kMaxExperts + 1];     // after the meeting: exclusive expert offsets
     __shared__ int  pre[kMaxExperts];         // tokens of expert e in the workgroups before this one
     __shared__ int  gave_up;
+    __shared__ int  recount[2][kMaxExperts];  // only used by a workgroup whose wait ran out
     unsigned* header = reinterpret_cast<unsigned*>(scratch);
     int* block_cnt = reinterpret_cast<int*>(scratch + kScratchHeader);
     const int nblk = gridDim.x, bid = blockIdx.x;
@@ -323,10 +327,54 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
         }
     }
     __syncthreads();
-    if (gave_up) return;                      // uniform: every wave of the workgroup leaves here
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
     // ---- totals (expert offsets) and the share of the workgroups before this one ---------
+    if (gave_up) {
+        // The others did not all arrive in time (workgroups of this grid kept off the chip by other
+        // work): this workgroup counts every token's choices itself, from the logits, with the same
+        // selection rule.  Slow, and independent of anybody else, so the result never depends on
+        // which workgroups were resident together.
+        for (int e = tid; e < E; e += kBlock) {
+            recount[0][e] = 0;
+            recount[1][e] = 0;
+        }
+        __syncthreads();
+        for (long j = tid; j < T_; j += kBlock) {
+            const auto* rowj = logits + j * E;
+            const bool earlier = j / kBlock < bid;
+            double prev_val = 0.0;
+            int prev_idx = -1;
+            bool has_prev = false;
+            for (int s = 0; s < k; ++s) {
+                double best_val = 0.0;
+                int best_idx = -1;
+                bool has_best = false;
+                for (int i = 0; i < E; ++i) {
+                    const double v = El::to_f64(rowj[i]);
+                    const bool within = !has_prev || (v < prev_val) || (v == prev_val && i > prev_idx);
+                    const bool better = !has_best || (v > best_val) || (v == best_val && i < best_idx);
+                    if (within && better) {
+                        best_val = v;
+                        best_idx = i;
+                        has_best = true;
+                    }
+                }
+                if (best_idx >= 0) {
+                    atomicAdd(&recount[0][best_idx], 1);
+                    if (earlier) atomicAdd(&recount[1][best_idx], 1);
+                }
+                prev_val = best_val;
+                prev_idx = best_idx;
+                has_prev = true;
+            }
+        }
+        __syncthreads();
+        for (int e = tid; e < E; e += kBlock) {
+            tot[e] = recount[0][e];
+            pre[e] = recount[1][e];
+        }
+    } else
     for (int e = wave; e < E; e += kWavesPerBlock) {
         int all = 0, before = 0;
         for (int j = lane; j < nblk; j += kWave) {
@@ -376,13 +424,17 @@ void launch_fused(const void* logits, long T_, int E, int k, long* topi, float* 
                   long* counts, long* offsets, unsigned char* scratch, hipStream_t s) {
     using store_t = typename Elem<T>::store_t;
     const dim3 grid(static_cast<unsigned>((T_ + kBlock - 1) / kBlock)), block(kBlock);
+    // PARAS_ROUTE_SPIN_LIMIT: polls before a workgroup stops waiting for the others (tests set 1 to
+    // drive the workgroups through the path that counts for itself)
+    const char* env = std::getenv("PARAS_ROUTE_SPIN_LIMIT");
+    const int spin = env != nullptr && std::atoi(env) > 0 ? std::atoi(env) : kSpinLimit;
     hipLaunchKernelGGL(route_clear_kernel, dim3(1), dim3(64), 0, s, reinterpret_cast<unsigned*>(scratch));
     if (E <= 8 && k <= 8)
         hipLaunchKernelGGL((route_fused_kernel<T, true>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, kSpinLimit);
+                           topw, order, inv_order, counts, offsets, scratch, spin);
     else
         hipLaunchKernelGGL((route_fused_kernel<T, false>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, kSpinLimit);
+                           topw, order, inv_order, counts, offsets, scratch, spin);
 }
 
 // Shared by the entry points: routes on `scratch` (device memory of route_scratch_bytes(T, E)).

@@ -163,3 +163,23 @@ def test_ffn_256_row_tiles_with_ragged_tiny_and_empty_experts():
     r = O.moe_route(logits[sel], k)
     ref = O.moe_ffn(x[sel], wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
     assert_ffn_close(out.cpu()[sel], ref, dt)
+
+
+@pytest.mark.parametrize("shape", [(8192, 8, 2, torch.bfloat16), (5000, 64, 6, torch.float32), (700, 16, 4, torch.float16)])
+def test_route_when_the_workgroups_do_not_wait_for_each_other(shape, monkeypatch):
+    """With a wait of one poll most workgroups of the one-kernel routing stop waiting for the others
+    and count every token's choices themselves (the path for a chip kept busy by unrelated work);
+    the few that arrive last take the usual path.  Same outputs either way, bit for bit."""
+    T, E, k, dtype = shape
+    torch.manual_seed(T)
+    logits = torch.randn(T, E).to(dtype)
+    logits[5] = logits[5, 0]
+    want = O.moe_route(logits, k)
+    monkeypatch.setenv("PARAS_ROUTE_SPIN_LIMIT", "1")
+    for _ in range(3):
+        got = capi.moe_route(logits.cuda(), k)
+        for name, g, w in zip(NAMES, got, want):
+            assert_bit_exact(g, w, f"moe_route {name} without waiting")
+    got = capi.moe_route_noalloc(logits.cuda(), k)
+    for name, g, w in zip(NAMES, got, want):
+        assert_bit_exact(g, w, f"moe_route_noalloc {name} without waiting")
