@@ -34,9 +34,19 @@ __device__ __forceinline__ std::uint16_t f32_to_bf16_bits(float f) {
 __device__ __forceinline__ float bf16_bits_to_f32(std::uint16_t b) {
     return __builtin_bit_cast(float, static_cast<std::uint32_t>(b) << 16);
 }
+// float -> half as v_cvt_f16_f32 rounds (to nearest even).  The value is made opaque first: left
+// to itself the compiler fuses a preceding fp32 multiply into v_fma_mixlo_f16 with a +0 addend,
+// which turns a product of -0 into +0.  A NaN keeps its payload here; the host's c10::Half writes
+// sign | 0x7E00 (f32_to_f16_bits_host below).
 __device__ __forceinline__ std::uint16_t f32_to_f16_bits(float f) {
-    const _Float16 h = static_cast<_Float16>(f);  // v_cvt_f16_f32, RNE
+    asm("" : "+v"(f));
+    const _Float16 h = static_cast<_Float16>(f);
     return __builtin_bit_cast(std::uint16_t, h);
+}
+__device__ __forceinline__ std::uint16_t f32_to_f16_bits_host(float f) {
+    const std::uint16_t h = f32_to_f16_bits(f);
+    const std::uint32_t u = __builtin_bit_cast(std::uint32_t, f);
+    return f != f ? static_cast<std::uint16_t>(((u >> 16) & 0x8000u) | 0x7E00u) : h;
 }
 __device__ __forceinline__ float f16_bits_to_f32(std::uint16_t b) {
     return static_cast<float>(__builtin_bit_cast(_Float16, b));
@@ -81,15 +91,12 @@ template <> struct Elem<f16_t> {
     static constexpr int kVec = 8;
     __device__ static __forceinline__ float  to_f32(std::uint16_t v) { return f16_bits_to_f32(v); }
     __device__ static __forceinline__ double to_f64(std::uint16_t v) { return static_cast<double>(f16_bits_to_f32(v)); }
-    __device__ static __forceinline__ std::uint16_t from_f32(float v) { return f32_to_f16_bits(v); }
+    __device__ static __forceinline__ std::uint16_t from_f32(float v) { return f32_to_f16_bits_host(v); }
+    // for values known not to be NaN
     __device__ static __forceinline__ std::uint16_t from_f32_finite(float v) { return f32_to_f16_bits(v); }
-    // Two roundings as on the host (double -> float -> half).  The empty asm
-    // keeps the compiler from merging them into one double -> half rounding.
-    __device__ static __forceinline__ std::uint16_t from_f64(double v) {
-        float f = static_cast<float>(v);
-        asm volatile("" : "+v"(f));
-        return f32_to_f16_bits(f);
-    }
+    // Two roundings as on the host (double -> float -> half); the conversion to half keeps its
+    // input opaque, so the compiler cannot merge them into one double -> half rounding.
+    __device__ static __forceinline__ std::uint16_t from_f64(double v) { return f32_to_f16_bits_host(static_cast<float>(v)); }
 };
 
 // ---- wavefront reductions ----------------------------------------------------

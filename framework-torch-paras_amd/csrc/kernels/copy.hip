@@ -157,7 +157,8 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_composed_v
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float v = E::to_f32(e[j]);
-                    acc += static_cast<double>(E::to_f32(E::from_f32(v * v)));
+                    // (the conversion instruction: a NaN's payload does not matter in a sum)
+                    acc += static_cast<double>(E::to_f32(E::from_f32_finite(v * v)));
                 }
             }
         }
@@ -180,11 +181,30 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_composed_v
                 const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv[i]);
                 u32x4 o;
                 std::uint16_t* oe = reinterpret_cast<std::uint16_t*>(&o);
+                // Narrowing by the conversion instructions; they keep a NaN's payload where the host's
+                // types canonicalise it, so a vector with a NaN in it (the probe below; inf - inf also
+                // sets it off, harmlessly) is narrowed again in software, behind a wave-uniform branch.
+                float probe = 0.f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    std::uint16_t y = E::from_f32(E::to_f32(e[j]) * inv);
-                    if (w != nullptr) y = E::from_f32(E::to_f32(y) * E::to_f32(we[j]));
+                    const float y1 = E::to_f32(e[j]) * inv;
+                    std::uint16_t y = E::from_f32_finite(y1);
+                    probe += y1;
+                    if (w != nullptr) {
+                        const float y2 = E::to_f32(y) * E::to_f32(we[j]);
+                        y = E::from_f32_finite(y2);
+                        probe += y2;
+                    }
                     oe[j] = y;
+                }
+                if (__builtin_amdgcn_ballot_w64(probe != probe) != 0) {
+                    asm volatile("" ::: "memory");           // not to be evaluated ahead of the branch
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        std::uint16_t y = E::from_f32(E::to_f32(e[j]) * inv);
+                        if (w != nullptr) y = E::from_f32(E::to_f32(y) * E::to_f32(we[j]));
+                        oe[j] = y;
+                    }
                 }
                 store16_nt(out + r * H + static_cast<long>(c) * 8, o);
             }

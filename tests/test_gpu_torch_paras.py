@@ -224,6 +224,17 @@ def test_composed_ops_streaming_kernels_are_exact(device):
         x = (scale * torch.randn(5, 512)).to(dt)
         got = torch.ops.aten.rms_norm(x.to(device), [512], None, 1e-6)
         assert_bit_exact(got.cpu(), O.rms_norm_composed(x, [512], None, 1e-6), f"aten::rms_norm tiny {dt}")
+        # rows with NaN, infinities of both signs, zeros and huge values: NaNs must come out as the
+        # host's types write them (the conversion instructions alone would keep their payloads)
+        x = torch.randn(8, 4096)
+        x[0, 5] = float("nan"); x[1, 7] = float("inf"); x[2, 9] = float("-inf"); x[2, 10] = float("inf")
+        x[3] = 0.0; x[4] *= 1e4 if dt == torch.float16 else 1e30; x[5, ::2] = -0.0
+        x = x.to(dt)
+        x[6].view(torch.int16)[3] = 0x7FA5 if dt == torch.bfloat16 else 0x7DA5          # a NaN with a payload
+        w4 = (1 + 0.1 * torch.randn(4096)).to(dt)
+        for wt in (w4, None):
+            got = torch.ops.aten.rms_norm(x.to(device), [4096], None if wt is None else wt.to(device), 1e-6)
+            assert_bit_exact(got.cpu(), O.rms_norm_composed(x, [4096], wt, 1e-6), f"aten::rms_norm special values {dt}")
         g = (4 * torch.randn(5, 1031)).to(dt)
         u = (torch.randn(5, 1031) * torch.tensor([1e-30, 1.0, 1e3, 1e-3, 30.0]).view(5, 1)).to(dt)
         got = torch.ops.torch_paras.swiglu(u.to(device), g.to(device))
@@ -581,6 +592,13 @@ def test_elementwise_binary_ops_on_device_match_the_host_engine(device):
         d += b.to(device)
         d *= row.to(device)
         assert_bit_exact(d.cpu(), O.binary(O.OP_MUL, O.binary(O.OP_ADD, a, b), row), f"in-place {dt}")
+        # signed zeros, infinities and NaNs (with payloads) keep the host's bits: -0 * x = -0, and a NaN
+        # comes out as the host's 16-bit types write it
+        z = torch.tensor([0.0, -0.0, 1.5, -2.0, float("inf"), float("-inf"), float("nan"), 1e-30]).to(dt)
+        zz, tt = z.view(8, 1).expand(8, 8).contiguous(), z.view(1, 8).expand(8, 8).contiguous()
+        for fn, code in ops:
+            got, want = fn(zz.to(device), tt.to(device)).cpu(), O.binary(code, zz, tt)
+            assert_bit_exact(got, want, f"{fn.__name__} {dt} special values")
     # integer tensors and promoting mixes are not part of the device surface: host route, same values as the CPU
     i = torch.arange(12).view(3, 4)
     assert torch.equal((i.to(device) + i.to(device)).cpu(), i + i)
