@@ -77,6 +77,25 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
         const int c = threadIdx.x + i * kBlock;
         if (c < nvec) wv[i] = load16(w + static_cast<long>(c) * V);  // shared by every row: an L2 hit
     }
+    // A NaN result must come out as the host's 16-bit types write it, which the fast tier's
+    // conversion instructions do not do, and its range test does not see a NaN (min / max skip
+    // them).  NaNs can only come from a weight that is not finite or from a row whose rstd is
+    // not an ordinary positive number (a NaN or an infinity in the row, or a row of zeros with
+    // eps = 0): both are known without looking at the elements.
+    bool w_odd[NV];
+    if constexpr (sizeof(S) == 2) {
+        constexpr std::uint32_t kExp = __is_same(T, bf16_t) ? 0x7F80u : 0x7C00u;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            w_odd[i] = false;
+            const int c = threadIdx.x + i * kBlock;
+            if (c < nvec) {
+#pragma unroll
+                for (int p = 0; p < 4; ++p)
+                    w_odd[i] = w_odd[i] || ((wv[i][p] & kExp) == kExp) || (((wv[i][p] >> 16) & kExp) == kExp);
+            }
+        }
+    }
     int sum_calls = 0;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         const S* xr = x + r * H;
@@ -107,12 +126,14 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
         const float rs32 = static_cast<float>(rs);
         if (threadIdx.x == 0) rstd[r] = rs32;
         if constexpr (sizeof(S) == 2) {
+            const bool row_odd = !(rs32 > 0.0f && rs32 <= 3.4028234663852886e38f);
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int c = threadIdx.x + i * kBlock;
                 if (c < nvec) {
                     bool fix;
                     u32x4 o = scale_vec16_fast<T>(xv[i], wv[i], rs32, fix);
+                    fix = fix || row_odd || w_odd[i];
                     if (__builtin_expect(fix, 0)) o = scale_vec16_fix<T>(xv[i], wv[i], o, rs32, rs);
                     store16_nt(outr + static_cast<long>(c) * V, o);
                 }

@@ -139,9 +139,16 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_vec(const std::uint16_t* __
 // (negated for backward).  Negation flips the sign bit, which is what
 // -(double)v rounded back gives for every finite value and infinity; a NaN
 // stays a NaN.
+// A 16-bit NaN as the host writes it after its trip through double: bf16 0x7FC0, half sign | 0x7E00
+// (kind 1 / 2; anything else passes through).
+__device__ __forceinline__ std::uint32_t host_nan16(std::uint32_t h, int kind) {
+    if (kind == 1) return (h & 0x7FFFu) > 0x7F80u ? 0x7FC0u : h;
+    if (kind == 2) return (h & 0x7FFFu) > 0x7C00u ? ((h & 0x8000u) | 0x7E00u) : h;
+    return h;
+}
 template <typename S>
 __global__ __launch_bounds__(kBlock) void rotate_half_any(const S* __restrict__ x, S* __restrict__ out,
-                                                          long n, long D, int backward) {
+                                                          long n, long D, int backward, int nan_kind) {
     const long half = D / 2;
     const long stride = static_cast<long>(gridDim.x) * kBlock;
     constexpr S kSign = static_cast<S>(S{1} << (sizeof(S) * 8 - 1));
@@ -150,7 +157,11 @@ __global__ __launch_bounds__(kBlock) void rotate_half_any(const S* __restrict__ 
         const bool first = col < half;
         const S v = x[first ? i + half : i - half];
         const bool negate = backward ? !first : first;
-        out[i] = negate ? static_cast<S>(v ^ kSign) : v;
+        S r = negate ? static_cast<S>(v ^ kSign) : v;
+        // the negated half goes through double on the host and comes back as its 16-bit types
+        // write a NaN; the other half is copied as it is
+        if constexpr (sizeof(S) == 2) r = negate ? static_cast<S>(host_nan16(r, nan_kind)) : r;
+        out[i] = r;
     }
 }
 
@@ -158,16 +169,33 @@ __global__ __launch_bounds__(kBlock) void rotate_half_any(const S* __restrict__ 
 // partner vector sits half a row away, the sign flips are one XOR per register.
 __global__ __launch_bounds__(kBlock) void rotate_half_vec16(const std::uint16_t* __restrict__ x,
                                                             std::uint16_t* __restrict__ out, long nvec,
-                                                            int vec_per_row, int backward) {
+                                                            int vec_per_row, int backward, int nan_kind) {
     const int half = vec_per_row / 2;
     const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
     if (i >= nvec) return;
     const int col = static_cast<int>(i % vec_per_row);
     const bool first = col < half;
     u32x4 v = load16_nt(x + (first ? i + half : i - half) * 8);
-    if (backward ? !first : first) {
+    const bool negate = backward ? !first : first;
+    if (negate) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) v[k] ^= 0x80008000u;
+    }
+    // The negated half goes through double on the host and comes back as its 16-bit types write
+    // a NaN (the other half is copied as it is).  Rare, so behind a wave-uniform test: an exponent
+    // field of all ones in any of the eight elements, i.e. a NaN or an infinity.
+    const std::uint32_t exp_mask = nan_kind == 1 ? 0x7F807F80u : 0x7C007C00u;
+    bool special = false;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const std::uint32_t e = v[k] & exp_mask;
+        special = special || (e & 0xFFFFu) == (exp_mask & 0xFFFFu) || (e >> 16) == (exp_mask >> 16);
+    }
+    if (__builtin_amdgcn_ballot_w64(special && negate) != 0) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (negate) v[k] = host_nan16(v[k] & 0xFFFFu, nan_kind) | (host_nan16(v[k] >> 16, nan_kind) << 16);
     }
     store16_nt(out + i * 8, v);
 }
@@ -294,11 +322,11 @@ int paras_rotate_half(const void* x, void* out, int64_t rows, int64_t D, int bac
     switch (dtype) {
         case PARAS_F32:
             hipLaunchKernelGGL((rotate_half_any<uint32_t>), grid, block, 0, s, static_cast<const uint32_t*>(x),
-                               static_cast<uint32_t*>(out), n, (long)D, backward);
+                               static_cast<uint32_t*>(out), n, (long)D, backward, 0);
             break;
         case PARAS_F64:
             hipLaunchKernelGGL((rotate_half_any<uint64_t>), grid, block, 0, s, static_cast<const uint64_t*>(x),
-                               static_cast<uint64_t*>(out), n, (long)D, backward);
+                               static_cast<uint64_t*>(out), n, (long)D, backward, 0);
             break;
         case PARAS_BF16:
         case PARAS_F16:
@@ -307,10 +335,10 @@ int paras_rotate_half(const void* x, void* out, int64_t rows, int64_t D, int bac
                 const long nvec = n / 8;
                 hipLaunchKernelGGL(rotate_half_vec16, dim3(static_cast<unsigned>((nvec + kBlock - 1) / kBlock)), block, 0, s,
                                    static_cast<const uint16_t*>(x), static_cast<uint16_t*>(out), nvec,
-                                   static_cast<int>(D / 8), backward);
+                                   static_cast<int>(D / 8), backward, dtype == PARAS_BF16 ? 1 : 2);
             } else {
                 hipLaunchKernelGGL((rotate_half_any<uint16_t>), grid, block, 0, s, static_cast<const uint16_t*>(x),
-                                   static_cast<uint16_t*>(out), n, (long)D, backward);
+                                   static_cast<uint16_t*>(out), n, (long)D, backward, dtype == PARAS_BF16 ? 1 : 2);
             }
             break;
         default: return fail(PARAS_ERR_INVALID, "paras_rotate_half: unknown dtype %d", dtype);

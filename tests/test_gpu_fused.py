@@ -275,3 +275,73 @@ def test_swiglu_backward_random_and_ragged(dtype):
     wgg, wgu = O.swiglu_backward(d2.contiguous(), g2.contiguous(), u2.contiguous())
     assert_bit_exact(gg, wgg, "grad_gate unaligned")
     assert_bit_exact(gu, wgu, "grad_up unaligned")
+
+
+def assert_same_bits_nan_aware(got, want, what):
+    """Bit for bit; a NaN must be a NaN at the same place.  bf16 NaNs also have the host's bits (its
+    type writes every NaN as 0x7FC0); for the other types the sign of a NaN that an invalid operation
+    produced is the host FPU's business (x86 makes it negative, the GPU positive) and is not compared."""
+    got = got.cpu()
+    assert got.shape == want.shape and got.dtype == want.dtype, what
+    if want.dtype == torch.bfloat16:
+        assert_bit_exact(got, want, what)
+        return
+    gn, wn = got.isnan(), want.isnan()
+    assert torch.equal(gn, wn), f"{what}: NaNs at different places"
+    it = {2: torch.int16, 4: torch.int32, 8: torch.int64}[want.element_size()]
+    assert torch.equal(got.view(it)[~wn], want.view(it)[~wn]), f"{what}: bits differ"
+
+
+SPECIALS = [0.0, -0.0, 1.5, -2.0, float("inf"), float("-inf"), float("nan"), 1e-30, -1e-30, 3e4, -3e4, 1e-7, 65504.0, 6e-8, -6e-8, 0.3]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_signed_zeros_infinities_and_nans_come_out_as_on_the_host(dtype):
+    """RMSNorm forward and backward, SwiGLU forward and backward and rotate_half on rows that hold
+    signed zeros, infinities, NaNs (also negative ones and ones with payloads), subnormal and huge
+    values, weights that are zero or negative, eps = 0 on rows of zeros."""
+    torch.manual_seed(3)
+    H = 512
+    x = torch.randn(16, H).to(dtype)
+    for r, v in enumerate(SPECIALS):
+        x[r, (r * 7) % H] = v
+    x[1, ::2] = -0.0
+    x[2] = 0.0
+    x[3] = -0.0
+    if dtype != torch.float32:
+        x[9].view(torch.int16)[11] = 0x7FA5 if dtype == torch.bfloat16 else 0x7DA5
+        x[10].view(torch.int16)[12] = -0x005B if dtype == torch.bfloat16 else -0x025B      # negative, with a payload
+    w = (1 + 0.1 * torch.randn(H)).to(dtype)
+    w[5], w[6], w[7] = -0.0, 0.0, -1.0
+    for eps in (1e-6, 0.0):
+        out, rstd = capi.rms_norm(dev(x), dev(w), eps)
+        wo, wr = O.rms_norm(x, w, eps)
+        assert_same_bits_nan_aware(out, wo, f"rms_norm {dtype} eps={eps}")
+        assert_same_bits_nan_aware(rstd, wr, f"rstd {dtype} eps={eps}")
+        if dtype != torch.float32:          # (fp32 column sums are compared with a tolerance elsewhere)
+            go = torch.randn(16, H).to(dtype)
+            go[0, 3], go[4, 9] = -0.0, float("nan")
+            go[2] = -0.0
+            gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(wr))
+            wgx, wgw = O.rms_norm_backward(go, x, w, wr)
+            assert_same_bits_nan_aware(gx, wgx, f"rms_norm grad_x {dtype} eps={eps}")
+            assert_same_bits_nan_aware(gw, wgw, f"rms_norm grad_w {dtype} eps={eps}")
+    g = torch.tensor(SPECIALS).repeat(16, 1).to(dtype)
+    u = torch.tensor(SPECIALS).view(16, 1).repeat(1, 16).to(dtype)
+    assert_same_bits_nan_aware(capi.swiglu(dev(g), dev(u)), O.swiglu(g, u), f"swiglu {dtype}")
+    go = torch.randn(16, 16).to(dtype)
+    go[0], go[1], go[2, 3], go[3, 4] = -0.0, 0.0, float("nan"), float("inf")
+    a, b = capi.swiglu_backward(dev(go), dev(g), dev(u))
+    wa, wb = O.swiglu_backward(go, g, u)
+    assert_same_bits_nan_aware(a, wa, f"swiglu grad_gate {dtype}")
+    assert_same_bits_nan_aware(b, wb, f"swiglu grad_up {dtype}")
+    xr = torch.tensor(SPECIALS).repeat(8, 8).to(dtype)
+    if dtype != torch.float32:
+        xr[0].view(torch.int16)[70] = 0x7FA5 if dtype == torch.bfloat16 else 0x7DA5        # a payload in each half
+        xr[1].view(torch.int16)[5] = 0x7FA5 if dtype == torch.bfloat16 else 0x7DA5
+    for backward in (False, True):
+        got, want = capi.rotate_half(dev(xr), backward), O.rotate_half(xr, backward)
+        if dtype == torch.bfloat16:
+            assert_bit_exact(got, want, f"rotate_half {dtype} backward={backward}")
+        else:
+            assert_same_bits_nan_aware(got, want, f"rotate_half {dtype} backward={backward}")
