@@ -131,6 +131,13 @@ __global__ __launch_bounds__(kBlock) void topk_rows_kernel(const typename Elem<T
     const auto* xr = x + static_cast<long>(blockIdx.x) * n;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
 
+    // NaNs.  The host scans a row from the left and an element replaces the running best only if
+    // it compares greater (or equal with a lower index): a NaN therefore never replaces anything and
+    // is never "after" the previous slot -- it can only be chosen by being the scan's first element,
+    // x[0] in slot 0.  The slot after that finds no element "after" a NaN (index -1, value 0), and
+    // the one after it goes on from (0, -1) like from any other previous slot.  In a parallel
+    // search that is: NaNs take no part, except that a NaN x[0] is slot 0.
+    const bool first_is_nan = n > 0 && E::to_f64(xr[0]) != E::to_f64(xr[0]);
     double prev_v = 0.0;
     long prev_i = -1;
     for (long s = 0; s < k; ++s) {
@@ -138,6 +145,7 @@ __global__ __launch_bounds__(kBlock) void topk_rows_kernel(const typename Elem<T
         long best_i = -1;
         for (long j = threadIdx.x; j < n; j += kBlock) {
             const double v = E::to_f64(xr[j]);
+            if (v != v) continue;
             // strictly after the previous slot in (value, index) order
             if (s > 0 && !comes_before(prev_v, prev_i, v, j, largest)) continue;
             if (best_i < 0 || comes_before(v, j, best_v, best_i, largest)) {
@@ -170,12 +178,16 @@ __global__ __launch_bounds__(kBlock) void topk_rows_kernel(const typename Elem<T
             }
         }
         __syncthreads();
+        if (first_is_nan && s == 0) {
+            best_i = 0;
+            best_v = E::to_f64(xr[0]);
+        }
         if (threadIdx.x == 0) {
-            // a row of NaNs has no element that "comes before" another: the host engine then
-            // reports index -1 for later slots; keep that
-            values[static_cast<long>(blockIdx.x) * k + s] = best_i >= 0 ? xr[best_i] : E::from_f64(0.0);
+            // no eligible element: the host engine reports index -1 and value 0
+            values[static_cast<long>(blockIdx.x) * k + s] = E::from_f64(best_i >= 0 ? best_v : 0.0);   // (a NaN as the host narrows it)
             indices[static_cast<long>(blockIdx.x) * k + s] = best_i;
         }
+        if (best_i < 0) best_v = 0.0;
         prev_v = best_v;
         prev_i = best_i;
     }
@@ -234,6 +246,9 @@ __global__ __launch_bounds__(kBlock) void topk_rows_wave_kernel(const typename E
         const int j = lane + i * kWave;
         v[i] = j < n ? E::to_f64(xr[j]) : 0.0;
     }
+    // (NaNs take no part in the search, except that a NaN x[0] is slot 0: see topk_rows_kernel)
+    const double x0 = __shfl(v[0], 0, kWave);
+    const bool first_is_nan = x0 != x0;
     double prev_v = 0.0;
     long prev_i = -1;
     for (int s = 0; s < k; ++s) {
@@ -242,7 +257,7 @@ __global__ __launch_bounds__(kBlock) void topk_rows_wave_kernel(const typename E
 #pragma unroll
         for (int i = 0; i < EPL; ++i) {
             const long j = lane + i * kWave;
-            if (j >= n) continue;
+            if (j >= n || v[i] != v[i]) continue;
             if (s > 0 && !comes_before(prev_v, prev_i, v[i], j, largest)) continue;   // strictly after the previous slot
             if (best_i < 0 || comes_before(v[i], j, best_v, best_i, largest)) {
                 best_v = v[i];
@@ -258,11 +273,16 @@ __global__ __launch_bounds__(kBlock) void topk_rows_wave_kernel(const typename E
                 best_i = oi;
             }
         }
+        if (first_is_nan && s == 0) {
+            best_i = 0;
+            best_v = x0;
+        }
         if (lane == 0) {
-            // a row of NaNs has no element that "comes before" another: index -1, value 0, as the host engine
-            values[row * k + s] = best_i >= 0 ? xr[best_i] : E::from_f64(0.0);
+            // no eligible element: index -1, value 0, as the host engine
+            values[row * k + s] = E::from_f64(best_i >= 0 ? best_v : 0.0);   // (a NaN as the host narrows it)
             indices[row * k + s] = best_i;
         }
+        if (best_i < 0) best_v = 0.0;
         prev_v = best_v;
         prev_i = best_i;
     }

@@ -79,3 +79,35 @@ def test_short_rows_with_nan_and_infinities():
     wv, wi = O.topk_last(x, 3)
     assert_bit_exact(gi, wi, "topk indices with NaN rows")
     assert torch.equal(gv.cpu().isnan(), wv.isnan()) and torch.equal(gv.cpu().nan_to_num(7.0), wv.nan_to_num(7.0))
+
+
+@pytest.mark.parametrize("dtype", FLOATS)
+@pytest.mark.parametrize("n", [40, 200, 700])
+def test_topk_rows_with_nans_follow_the_host_scan(dtype, n):
+    """The host picks each slot by a scan from the left in which a NaN never replaces the running
+    best and is never 'after' the previous slot: a NaN is chosen only as x[0] in slot 0, the slot
+    after that has no candidate (index -1, value 0), and the one after that goes on from (0, -1).
+    NaNs first, last, in runs and next to infinities, on the one-wave and the workgroup kernels,
+    largest and smallest."""
+    torch.manual_seed(n)
+    x = torch.randn(12, n).to(dtype)
+    nan, inf = float("nan"), float("inf")
+    x[0, 5] = nan
+    x[1, 0] = nan
+    x[2, 0], x[2, 9] = nan, nan
+    x[3, n - 1] = nan
+    x[4, 1:5] = nan
+    x[5, 0], x[5, 1] = nan, inf
+    x[6, 0], x[6, 3] = inf, nan
+    x[7, 0], x[7, 2], x[7, 3] = nan, 0.0, -0.0
+    x[8, ::2] = nan
+    x[9, 0], x[9, 1:] = 1.0, nan
+    for k in (1, 3, min(n, 40)):
+        for largest in (True, False):
+            gv, gi = capi.topk_rows(x.cuda(), k, largest)
+            wv, wi = O.topk_last(x, k, largest)
+            assert_bit_exact(gi, wi, f"topk indices {dtype} n={n} k={k} largest={largest}")
+            if dtype == torch.bfloat16 or not bool(wv.isnan().any()):
+                assert_bit_exact(gv, wv, f"topk values {dtype} n={n} k={k} largest={largest}")
+            else:
+                assert torch.equal(gv.cpu().isnan(), wv.isnan()) and torch.equal(gv.cpu().nan_to_num(7.0), wv.nan_to_num(7.0))
