@@ -146,7 +146,8 @@ int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream) {
     if (rc != PARAS_OK) return rc;
     const paras_sdpa_args& a = *args;
     if (empty_output(a)) return PARAS_OK;
-    PARAS_REQUIRE(a.q && a.k && a.v && a.out, "paras sdpa: null tensor pointer");
+    PARAS_REQUIRE(a.out != nullptr, "paras sdpa: null output pointer");
+    PARAS_REQUIRE(a.Lk == 0 || (a.q && a.k && a.v), "paras sdpa: null tensor pointer");   // (empty k / v have no storage)
     hipStream_t s = nullptr;
     rc = resolve_stream(stream, &s);
     if (rc != PARAS_OK) return rc;

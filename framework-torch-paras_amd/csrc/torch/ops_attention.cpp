@@ -55,7 +55,9 @@ void prepare(const Tensor& query, const Tensor& key, const Tensor& value, const 
         std::vector<int64_t> full(lead.begin(), lead.end());
         full.insert(full.end(), t.sizes().end() - 3, t.sizes().end());
         Tensor e = t.expand(full);
-        return e.reshape({-1, t.size(-3), t.size(-2), t.size(-1)});
+        int64_t batch = 1;                       // (spelled out: -1 cannot be inferred for an empty tensor)
+        for (int64_t d : lead) batch *= d;
+        return e.reshape({batch, t.size(-3), t.size(-2), t.size(-1)});
     };
     std::vector<int64_t> lead(query.sizes().begin(), query.sizes().end() - 3);
     {

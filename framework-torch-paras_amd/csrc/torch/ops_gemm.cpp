@@ -42,13 +42,13 @@ void check_dtypes(const Tensor& a, const Tensor& b, const char* what) {
     TORCH_CHECK(is_float(a), "paras ", what, ": only float dtypes (fp32, fp64, bf16, fp16) are supported on the device");
 }
 
-// out[b] = alpha * a[b] @ mat2[b] + beta * addend
+// out[b] = alpha * a[b] @ mat2[b] + beta * addend; batch < 0: plain matrices
 Tensor run_gemm(const Tensor& a_in, const Tensor& mat2, const c10::optional<Tensor>& addend, double alpha, double beta,
                 int64_t batch) {
     const bool mfma = wants_mfma(a_in);
     Tensor a = as_rows(a_in, mfma), bt = as_nt_operand(mat2, mfma);
     const int64_t M = a.size(-2), K = a.size(-1), N = bt.size(-2);
-    std::vector<int64_t> shape = batch > 0 ? std::vector<int64_t>{batch, M, N} : std::vector<int64_t>{M, N};
+    std::vector<int64_t> shape = batch >= 0 ? std::vector<int64_t>{batch, M, N} : std::vector<int64_t>{M, N};
     Tensor out = at::empty(shape, a.options());
     if (out.numel() == 0) return out;
     const void* add_ptr = nullptr;
@@ -60,14 +60,14 @@ Tensor run_gemm(const Tensor& a_in, const Tensor& mat2, const c10::optional<Tens
         add_ptr = add.data_ptr();
         ld_add = add.stride(-2);
     }
-    const int64_t nb = batch > 0 ? batch : 1;
+    const int64_t nb = batch >= 0 ? batch : 1;
     const int code = require_float_code(a, "paras gemm");
     // few-row products (decode-time projections) run faster with a workspace for split partial sums
     const size_t ws_bytes = paras_gemm_nt_workspace(M, N, K, nb, code);
     Tensor ws;
     if (ws_bytes > 0) ws = at::empty({static_cast<int64_t>(ws_bytes)}, a.options().dtype(c10::kByte));
     check(paras_gemm_nt_ws(a.data_ptr(), bt.data_ptr(), add_ptr, out.data_ptr(), M, N, K, a.stride(-2), bt.stride(-2), N, ld_add,
-                           nb, batch > 0 ? a.stride(0) : 0, batch > 0 ? bt.stride(0) : 0, M * N, s_add, alpha, beta, code,
+                           nb, batch >= 0 ? a.stride(0) : 0, batch >= 0 ? bt.stride(0) : 0, M * N, s_add, alpha, beta, code,
                            ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, stream_for(a)));
     return out;
 }
@@ -77,7 +77,7 @@ Tensor mm(const Tensor& self, const Tensor& mat2) {
     TORCH_CHECK(self.size(1) == mat2.size(0), "paras mm: shapes cannot be multiplied (", self.size(0), "x", self.size(1), " and ",
                 mat2.size(0), "x", mat2.size(1), ")");
     check_dtypes(self, mat2, "mm");
-    return run_gemm(self, mat2, c10::nullopt, 1.0, 0.0, 0);
+    return run_gemm(self, mat2, c10::nullopt, 1.0, 0.0, -1);
 }
 
 Tensor bmm(const Tensor& self, const Tensor& mat2) {
@@ -98,7 +98,7 @@ Tensor addmm(const Tensor& self, const Tensor& mat1, const Tensor& mat2, const a
     check_dtypes(mat1, mat2, "addmm");
     TORCH_CHECK(self.scalar_type() == mat1.scalar_type(), "paras addmm: operand dtypes differ");
     require_same_device("addmm", mat1, {{"self", &self}});
-    return run_gemm(mat1, mat2, self, alpha.toDouble(), beta.toDouble(), 0);
+    return run_gemm(mat1, mat2, self, alpha.toDouble(), beta.toDouble(), -1);
 }
 
 }  // namespace

@@ -741,3 +741,51 @@ def test_reference_device_numbering_on_the_gpu():
     """PARAS_DEVICE_BASE=1 with a GPU present: ops run on `paras:1`, `paras:0` raises."""
     from test_package_cpu import test_reference_device_numbering_is_an_opt_in
     test_reference_device_numbering_is_an_opt_in()
+
+
+def test_empty_and_degenerate_shapes_match_the_cpu(device):
+    """Zero-sized batches, rows, key lengths and contraction sizes, rank-3 and rank-5 attention
+    inputs, one-element and zero-dimensional operands: same shapes, dtypes and values as torch's
+    CPU ops (the reference's tests compare with torch-CPU the same way)."""
+    sd = F.scaled_dot_product_attention
+
+    def first(r):
+        return r[0] if isinstance(r, (tuple, list)) else r
+
+    def same(name, fn, *args):
+        want = first(fn(*args))
+        got = first(fn(*[a.to(device) if torch.is_tensor(a) else a for a in args])).cpu()
+        assert got.shape == want.shape and got.dtype == want.dtype, f"{name}: {tuple(got.shape)} {got.dtype} vs {tuple(want.shape)} {want.dtype}"
+        assert torch.allclose(got.float(), want.float(), rtol=2e-2, atol=2e-2, equal_nan=True), name
+
+    for dt in (torch.bfloat16, torch.float32):
+        z = lambda *s: torch.zeros(*s, dtype=dt)
+        r = lambda *s: torch.randn(*s).to(dt)
+        same(f"sdpa Lq=0 {dt}", sd, z(1, 2, 0, 16), r(1, 2, 5, 16), r(1, 2, 5, 16))
+        same(f"sdpa Lk=0 {dt}", sd, r(1, 2, 3, 16), z(1, 2, 0, 16), z(1, 2, 0, 16))
+        same(f"sdpa B=0 {dt}", sd, z(0, 2, 3, 16), z(0, 2, 3, 16), z(0, 2, 3, 16))
+        same(f"sdpa D=1 {dt}", sd, r(1, 2, 3, 1), r(1, 2, 4, 1), r(1, 2, 4, 1))
+        same(f"sdpa rank 3 {dt}", sd, r(2, 3, 16), r(2, 4, 16), r(2, 4, 16))
+        same(f"sdpa rank 5 {dt}", sd, r(2, 2, 3, 5, 16), r(2, 2, 3, 7, 16), r(2, 2, 3, 7, 16))
+        same(f"sdpa one key, causal {dt}", lambda q, k, v: sd(q, k, v, is_causal=True), r(1, 2, 5, 128), r(1, 2, 1, 128), r(1, 2, 1, 128))
+        same(f"sdpa D=256 {dt}", sd, r(1, 2, 9, 256), r(1, 2, 11, 256), r(1, 2, 11, 256))
+        same(f"mm K=0 {dt}", torch.mm, z(3, 0), z(0, 4))
+        same(f"mm M=0 {dt}", torch.mm, z(0, 8), r(8, 4))
+        same(f"mm 1x1 {dt}", torch.mm, r(1, 1), r(1, 1))
+        same(f"bmm empty batch {dt}", torch.bmm, z(0, 3, 4), z(0, 4, 5))
+        same(f"bmm K=0 {dt}", torch.bmm, z(2, 3, 0), z(2, 0, 5))
+        same(f"linear of a vector {dt}", F.linear, r(64), r(5, 64), r(5))
+        same(f"matmul of vectors {dt}", torch.matmul, r(8), r(8))
+        same(f"softmax of empty rows {dt}", lambda x: torch.softmax(x, -1), z(3, 0))
+        same(f"softmax 0-d {dt}", lambda x: torch.softmax(x, 0), r(()))
+        same(f"topk k=0 {dt}", lambda x: torch.topk(x, 0), r(3, 5))
+        same(f"add empty {dt}", torch.add, z(0, 3), z(0, 3))
+        same(f"add 0-d {dt}", torch.add, r(3, 4), r(()))
+        same(f"cat with an empty piece {dt}", lambda a, b, c: torch.cat([a, b, c], 0), r(2, 3), z(0, 3), r(1, 3))
+        same(f"index_select with no indices {dt}", lambda x, i: torch.index_select(x, 0, i), r(4, 3), torch.zeros(0, dtype=torch.long))
+        same(f"rms_norm over two dims {dt}", lambda x, w: F.rms_norm(x, [3, 16], w, 1e-5), r(2, 3, 16), r(3, 16))
+    lg = torch.zeros(0, 8).to(device)
+    topi, topw, order, inverse, counts, offsets = torch.ops.paras.moe_route(lg, 2)
+    assert topi.shape == (0, 2) and counts.cpu().tolist() == [0] * 8 and offsets.cpu().tolist() == [0] * 9
+    out, rstd = torch.ops.paras.rms_norm(torch.zeros(0, 64).to(device), torch.ones(64).to(device), 1e-6)
+    assert out.shape == (0, 64) and rstd.numel() == 0
