@@ -4,8 +4,9 @@
 // engine's binary_kernel (csrc/ops/pointwise_ops.cpp:63-85, 262-302: both
 // operands in the output dtype, a wrapped scalar narrowed to it first,
 // result = T(a op alpha*b) in double); paras_binary_strided does the same on the
-// GPU for float tensors of one dtype, with broadcasting.  Anything else
-// (integer tensors, mixed dtypes that promote) takes ATen on host copies.
+// GPU for float tensors, with broadcasting (two float dtypes are converted to the
+// promoted one on the device first).  Anything else (integer tensors) takes ATen
+// on host copies.
 #include "paras_torch.h"
 
 #include <ATen/ExpandUtils.h>
@@ -36,7 +37,9 @@ Tensor host_route(int op, const Tensor& self, const Tensor& other, const at::Sca
     return r.to(is_paras(self) ? self.device() : other.device());
 }
 
-Tensor run(int op, const Tensor& self, const Tensor& other, double alpha) {
+// `into`, when given, is a dense tensor of the broadcast shape that receives the result (the
+// in-place forms pass `self`: element i is read before it is written by the same lane).
+Tensor run(int op, const Tensor& self, const Tensor& other, double alpha, const Tensor* into = nullptr) {
     Tensor b = other;
     if (!is_paras(other)) {
         // the number, narrowed to the tensor's dtype as the reference does, as a one-element device tensor
@@ -46,7 +49,7 @@ Tensor run(int op, const Tensor& self, const Tensor& other, double alpha) {
     const std::vector<int64_t> shape = at::infer_size(self.sizes(), b.sizes());
     TORCH_CHECK(shape.size() <= 8, "paras: tensor rank ", shape.size(), " exceeds kernel limit of 8");
     const Tensor a = self.expand(shape), bb = b.expand(shape);
-    Tensor out = at::empty(shape, self.options());
+    Tensor out = into != nullptr ? *into : at::empty(shape, self.options());
     if (out.numel() == 0) return out;
     check(paras_binary_strided(op, a.data_ptr(), bb.data_ptr(), out.data_ptr(), static_cast<int>(shape.size()), shape.data(),
                                a.strides().data(), bb.strides().data(), alpha, require_float_code(self, "paras binary op"),
@@ -54,16 +57,49 @@ Tensor run(int op, const Tensor& self, const Tensor& other, double alpha) {
     return out;
 }
 
+bool float_pair_on_one_device(const Tensor& a, const Tensor& b) {
+    return is_paras(a) && is_paras(b) && a.device() == b.device() && float_code(a.scalar_type()) >= 0 &&
+           float_code(b.scalar_type()) >= 0;
+}
+
 Tensor binary(int op, const Tensor& self, const Tensor& other, const at::Scalar& alpha) {
     if (device_takes(self, other)) return run(op, self, other, alpha.toDouble());
     // number (op) tensor: add and mul commute; the others go to the host
     if ((op == kAdd || op == kMul) && is_host_number(self) && device_takes(other, self)) return run(op, other, self, alpha.toDouble());
+    // Float tensors of two dtypes: both are brought to the promoted dtype on the device (the
+    // reference's binary_kernel converts both operands to the output's dtype, which the structured
+    // op has set to the promoted one; csrc/ops/pointwise_ops.cpp:66-69).
+    if (float_pair_on_one_device(self, other)) {
+        const auto common = at::result_type(self, other);
+        if (float_code(common) >= 0) return run(op, self.to(common), other.to(common), alpha.toDouble());
+    }
     return host_route(op, self, other, alpha);
 }
 
+// True when writing `self` element by element while `other` is being read cannot change what is read:
+// different storages, or the very same view.
+bool safe_to_write_in_place(const Tensor& self, const Tensor& other) {
+    if (!is_paras(other) || !other.storage().is_alias_of(self.storage())) return true;
+    return other.data_ptr() == self.data_ptr() && other.sizes() == self.sizes() && other.strides() == self.strides();
+}
+
+// In-place forms keep self's dtype: the reference converts `other` to it first and computes there
+// (binary_kernel(self, other, self), csrc/ops/pointwise_ops.cpp:292-296).
 Tensor& binary_(int op, Tensor& self, const Tensor& other, const at::Scalar& alpha) {
-    Tensor r = binary(op, self, other, alpha);
+    Tensor b = other;
+    if (float_pair_on_one_device(self, other) && other.scalar_type() != self.scalar_type()) b = other.to(self.scalar_type());
+    if (device_takes(self, b)) {
+        const std::vector<int64_t> shape = at::infer_size(self.sizes(), b.sizes());
+        TORCH_CHECK(self.sizes().equals(shape), "paras: output with shape ", self.sizes(), " doesn't match the broadcast shape ", shape);
+        if (self.is_contiguous() && safe_to_write_in_place(self, b)) {
+            run(op, self, b, alpha.toDouble(), &self);
+            return self;
+        }
+    }
+    Tensor r = binary(op, self, b, alpha);
     TORCH_CHECK(r.sizes() == self.sizes(), "paras: output with shape ", self.sizes(), " doesn't match the broadcast shape ", r.sizes());
+    TORCH_CHECK(at::canCast(r.scalar_type(), self.scalar_type()), "result type ", r.scalar_type(),
+                " can't be cast to the desired output type ", self.scalar_type());
     self.copy_(r);
     return self;
 }

@@ -599,12 +599,57 @@ def test_elementwise_binary_ops_on_device_match_the_host_engine(device):
         for fn, code in ops:
             got, want = fn(zz.to(device), tt.to(device)).cpu(), O.binary(code, zz, tt)
             assert_bit_exact(got, want, f"{fn.__name__} {dt} special values")
-    # integer tensors and promoting mixes are not part of the device surface: host route, same values as the CPU
+    # integer tensors take the host route; a promoting mix of float dtypes is computed on the device: same values as the CPU
     i = torch.arange(12).view(3, 4)
     assert torch.equal((i.to(device) + i.to(device)).cpu(), i + i)
     m = torch.randn(4, 4).bfloat16()
     f = torch.randn(4, 4)
     assert torch.equal((m.to(device) + f.to(device)).cpu(), m + f)
+
+
+def test_binary_ops_of_two_float_dtypes_and_in_place_forms(device):
+    """Two float dtypes: both operands are converted to the promoted dtype and the op is evaluated there
+    (the reference's to_compute, csrc/ops/pointwise_ops.cpp:55-69).  The in-place forms keep self's
+    dtype and storage: `other` is narrowed to it first (binary_kernel(self, other, self), :292-296),
+    so the result differs from torch's CPU one, which adds in float before narrowing.  Operands that
+    overlap self in memory still give the value of the out-of-place op; an integer self with a float
+    other raises as torch does."""
+    torch.manual_seed(41)
+    codes = (("add", O.OP_ADD), ("sub", O.OP_SUB), ("mul", O.OP_MUL), ("div", O.OP_DIV))
+    bf, h, f, d = torch.randn(6, 40).bfloat16(), torch.randn(6, 40).half(), torch.randn(6, 40), torch.randn(6, 40).double()
+    for name, code in codes:
+        for x, y in ((bf, f), (h, bf), (f, d), (h, f), (f, bf)):
+            common = torch.result_type(x, y)
+            got = getattr(torch, name)(x.to(device), y.to(device))
+            assert got.dtype == common
+            assert_bit_exact(got.cpu(), O.binary(code, x.to(common), y.to(common)), f"{name} {x.dtype} {y.dtype}")
+            xd = x.to(device)
+            where = xd.data_ptr()
+            getattr(xd, name + "_")(y.to(device))
+            assert xd.data_ptr() == where and xd.dtype == x.dtype
+            assert_bit_exact(xd.cpu(), O.binary(code, x, y.to(x.dtype)), f"{name}_ {x.dtype} by {y.dtype}")
+    # a zero-dim device tensor of a wider dtype does not promote
+    got = h.to(device) * torch.tensor(0.3, dtype=torch.float64).to(device)
+    assert got.dtype == torch.float16
+    assert_bit_exact(got.cpu(), O.binary_scalar(O.OP_MUL, h, 0.3), "f16 * 0-dim f64")
+    # self read and written by the same call
+    x = torch.randn(6, 8).bfloat16()
+    xd = x.to(device)
+    xd += xd
+    assert_bit_exact(xd.cpu(), O.binary(O.OP_ADD, x, x), "x += x")
+    x = torch.randn(6, 8)
+    xd = x.to(device)
+    xd[1:] += xd[:-1]
+    want = x.clone()
+    want[1:] = x[1:] + x[:-1]
+    assert torch.equal(xd.cpu(), want)
+    xd = x.to(device)
+    xd.t().mul_(xd.t())
+    assert torch.equal(xd.cpu(), x * x)
+    with pytest.raises(RuntimeError, match="can't be cast"):
+        torch.arange(6).to(device).add_(torch.randn(6).to(device))
+    with pytest.raises(RuntimeError, match="broadcast shape"):
+        torch.randn(5).to(device).add_(torch.randn(4, 5).to(device))
 
 
 def test_decoder_block_runs_without_any_host_fallback():
