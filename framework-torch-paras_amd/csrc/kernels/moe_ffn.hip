@@ -351,12 +351,13 @@ int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up, const voi
     PARAS_REQUIRE(T >= 0 && E >= 1 && k >= 1 && H >= 1 && I >= 1, "paras_moe_ffn: bad shape");
     if (T == 0) return PARAS_OK;
     PARAS_REQUIRE(dtype == PARAS_BF16 || dtype == PARAS_F16, "paras_moe_ffn: dtype must be bf16 or f16");
-    const bool tiles = H % kBK == 0 && I % kBK == 0;     // else: the general kernels (any size, any alignment)
     PARAS_REQUIRE(x && w_gate && w_up && w_down && topw && order && inv_order && offsets && out && workspace,
                   "paras_moe_ffn: null pointer");
-    PARAS_REQUIRE(!tiles || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_gate) | reinterpret_cast<uintptr_t>(w_up) |
-                              reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0,
-                  "paras_moe_ffn: tensors must be 16-byte aligned");
+    // The MFMA tiles take hidden and intermediate sizes that are multiples of 64 and 16-byte aligned
+    // tensors; anything else goes to the general kernels (any size, any alignment).
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_gate) | reinterpret_cast<uintptr_t>(w_up) |
+                           reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0;
+    const bool tiles = H % kBK == 0 && I % kBK == 0 && aligned;
     PARAS_REQUIRE(T * k <= 0x3fffffffLL, "paras_moe_ffn: too many routed rows");
     if (T * H >= (1LL << 32) || T * k * I >= (1LL << 32) || I * H >= (1LL << 32))
         return fail(PARAS_ERR_UNSUPPORTED, "paras_moe_ffn: an operand (x, the routed intermediate, or one expert's weight matrix) spans 2^32 elements or more");

@@ -209,7 +209,7 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
         const auto* row = logits + t * E;
         double val[kSmall ? 8 : 1];
         if constexpr (kSmall) {
-            if (sizeof(typename El::store_t) == 2 && E == 8) {     // the row is one aligned 16-byte load
+            if (sizeof(typename El::store_t) == 2 && E == 8 && (reinterpret_cast<std::uintptr_t>(logits) & 15) == 0) {     // the row is one aligned 16-byte load
                 const u32x4 w = load16(row);
 #pragma unroll
                 for (int j = 0; j < 8; ++j)

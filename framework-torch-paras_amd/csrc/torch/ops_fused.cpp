@@ -126,7 +126,12 @@ Tensor moe_ffn(const Tensor& x, const Tensor& w_gate, const Tensor& w_up, const 
     TORCH_CHECK(topw.scalar_type() == c10::kFloat, "paras moe_ffn: topw must be float32");
     TORCH_CHECK(order.scalar_type() == c10::kLong && inv_order.scalar_type() == c10::kLong && offsets.scalar_type() == c10::kLong,
                 "paras moe_ffn: order, inv_order and offsets must be int64");
-    Tensor xc = x.contiguous(), wg = w_gate.contiguous(), wu = w_up.contiguous(), wd = w_down.contiguous();
+    // dense, and on a 16-byte boundary (a view at an odd storage offset is copied): what the MFMA tiles take
+    auto dense16 = [](const Tensor& t) {
+        Tensor c = t.contiguous();
+        return (reinterpret_cast<uintptr_t>(c.data_ptr()) & 15) == 0 ? c : c.clone();
+    };
+    Tensor xc = dense16(x), wg = dense16(w_gate), wu = dense16(w_up), wd = dense16(w_down);
     Tensor tw = topw.contiguous(), od = order.contiguous(), iv = inv_order.contiguous(), of = offsets.contiguous();
     Tensor out = at::empty({T, H}, xc.options());
     if (T == 0) return out;

@@ -296,8 +296,9 @@ PARAS_API int paras_moe_route_noalloc(const void* logits, int64_t T, int64_t E, 
 /*                                    pointwise_ops.cpp:280-284,766-774)      */
 /* x: [T, H]; w_gate, w_up: [E, I, H]; w_down: [E, H, I]; out: [T, H];        */
 /* all dtype `dtype` (bf16 or f16), GEMMs accumulate in fp32.  H and I that   */
-/* are multiples of 64 (16-byte aligned tensors) run on the MFMA tiles; other */
-/* sizes on general kernels (at most 65535 routed rows), never on the host.   */
+/* are multiples of 64, with 16-byte aligned tensors, run on the MFMA tiles;  */
+/* other sizes or alignments on general kernels (at most 65535 routed rows,   */
+/* far slower), never on the host.                                            */
 /* `workspace`: paras_moe_ffn_workspace(T,k,H,I) bytes of device memory.      */
 /* ------------------------------------------------------------------------- */
 PARAS_API size_t paras_moe_ffn_workspace(int64_t T, int64_t k, int64_t H, int64_t I,

@@ -118,6 +118,35 @@ def test_ffn_sizes_the_tiles_do_not_take(shape, dtype):
     assert_ffn_close(out, want, dtype)
 
 
+def _at_offset(t, elems=1):
+    """The same values in device memory that starts `elems` elements past an allocation's start."""
+    flat = torch.empty(t.numel() + elems, dtype=t.dtype, device="cuda")
+    view = flat[elems:].view(t.shape)
+    view.copy_(t)
+    return view
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_operands_that_are_not_16_byte_aligned(dtype):
+    """A view at an odd storage offset: routing reads its 8-expert rows element by element and the FFN
+    runs on the general kernels; same results as from aligned memory (routing exactly)."""
+    T, E, k, H, I = 300, 8, 2, 128, 256
+    x, logits = torch.randn(T, H).to(dtype), torch.randn(T, E).to(dtype)
+    wg, wu = (0.05 * torch.randn(E, I, H)).to(dtype), (0.05 * torch.randn(E, I, H)).to(dtype)
+    wd = (0.05 * torch.randn(E, H, I)).to(dtype)
+    want_route = O.moe_route(logits, k)
+    for elems in (1, 3):
+        got = capi.moe_route(_at_offset(logits, elems), k)
+        for g, w in zip(got, want_route):
+            assert torch.equal(g.cpu(), w)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    want = O.moe_ffn(x, wg, wu, wd, want_route[1], want_route[2], want_route[3], want_route[5], k, gemm="aten")
+    out = capi.moe_ffn(_at_offset(x), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    assert_ffn_close(out, want, dtype)
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), _at_offset(wu, 3), wd.cuda(), topw, order, inv, offsets, k)
+    assert_ffn_close(out, want, dtype)
+
+
 def test_config5_routing_exact_and_sampled_tokens():
     """BASELINE config 5 (T=8192 H=4096 E=8 top-2 I=14336 bf16) at full size:
     routing bit-exact on all tokens, the FFN on 48 sampled tokens against the

@@ -320,6 +320,11 @@ def test_moe_layer(device):
     out = paras_nn.moe_layer(x.to(device), logits.to(device), wg.to(device), wu.to(device), wd.to(device), k)
     ref = O.moe_ffn(x, wg, wu, wd, want[1], want[2], want[3], want[5], k, gemm="aten")
     assert out.shape == (T, H) and (out.cpu().float() - ref.float()).abs().max().item() <= 2e-2
+    # a view at an odd storage offset is moved onto a 16-byte boundary for the MFMA tiles: the same bits
+    shifted = torch.empty(T * H + 1, dtype=dt).to(device)[1:].view(T, H)
+    shifted.copy_(x.to(device))
+    again = paras_nn.moe_layer(shifted, logits.to(device), wg.to(device), wu.to(device), wd.to(device), k)
+    assert_bit_exact(again.cpu(), out.cpu(), "moe_layer from a misaligned view")
 
 
 # ---- copies and plumbing (reference tests/test_attention_norm_ops.py:172-216) -----
