@@ -72,7 +72,16 @@ void prepare(const Tensor& query, const Tensor& key, const Tensor& value, const 
         // Without GQA the head dims must agree or broadcast (Hk == 1), as matmul would.
         TORCH_CHECK(Hk == Hq || Hk == 1, "paras sdpa: key/value heads (", Hk, ") do not match query heads (", Hq, ")");
     }
-    auto last_contig = [](Tensor t) { return t.stride(-1) == 1 || t.size(-1) <= 1 ? t : t.contiguous(); };
+    // A contiguous last dim is required; 16-bit operands are also moved onto what the MFMA kernels
+    // take (a 16-byte boundary, strides that are multiples of 8 elements) when a view is not: the
+    // copy costs far less than the general kernel such a view would otherwise run on.
+    auto last_contig = [](Tensor t) {
+        if (!(t.stride(-1) == 1 || t.size(-1) <= 1)) return t.contiguous();
+        if (t.element_size() != 2 || t.numel() == 0 || t.size(-1) % 8 != 0) return t;   // (a dense copy would not help an odd head size)
+        bool ok = (reinterpret_cast<uintptr_t>(t.data_ptr()) & 15) == 0;
+        for (int64_t d = 0; d < 3; ++d) ok = ok && (t.size(d) <= 1 || t.stride(d) % 8 == 0);
+        return ok ? t : t.clone(c10::MemoryFormat::Contiguous);
+    };
     p->q = last_contig(p->q);
     p->k = last_contig(p->k);
     p->v = last_contig(p->v);

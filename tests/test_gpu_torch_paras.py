@@ -178,6 +178,25 @@ def test_sdpa_bf16_takes_the_flash_and_decode_kernels(device):
 
 
 # ---- aten::rms_norm / torch_paras::swiglu (reference tests/test_attention_norm_ops.py:115-165)
+def test_sdpa_views_at_odd_offsets_still_take_the_mfma_kernels(device):
+    """q / k / v that start off a 16-byte boundary, or whose strides are not multiples of 8 elements,
+    are copied dense before the call: no general-kernel launch, same values as from fresh tensors."""
+    import torch_paras
+    B, H, L, D = 1, 4, 256, 128
+    q, k, v = (torch.randn(B, H, L, D).bfloat16() for _ in range(3))
+    want = F.scaled_dot_product_attention(q.to(device), k.to(device), v.to(device), is_causal=True).cpu()
+
+    def shifted(t, extra_row=0):
+        buf = torch.empty(B * H * L * (D + extra_row) + 1, dtype=t.dtype).to(device)
+        view = buf[1:].view(B, H, L, D + extra_row)[..., :D]
+        view.copy_(t.to(device))
+        return view
+    got = F.scaled_dot_product_attention(shifted(q), shifted(k), shifted(v), is_causal=True).cpu()
+    assert_bit_exact(got, want, "sdpa from views one element off a boundary")
+    got = F.scaled_dot_product_attention(shifted(q, 3), shifted(k, 3), shifted(v, 3), is_causal=True).cpu()
+    assert_bit_exact(got, want, "sdpa from views with odd row strides")
+
+
 def test_rms_norm_no_weight(device):
     x = torch.randn(4, 6, 32)
     assert_close(torch.ops.aten.rms_norm(x.to(device), [32], None, None), torch.ops.aten.rms_norm(x, [32], None, 1e-6), "no weight")
