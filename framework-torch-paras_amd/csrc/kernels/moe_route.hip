@@ -16,12 +16,12 @@
 // them resident at once.  A lane owns a token: its row of logits arrives as one 16-byte
 // load (E = 8 of a 16-bit type) and stays in registers for the k selection scans; the
 // workgroup counts its tokens per expert with wavefront ballots, publishes the counts,
-// and meets the other workgroups at a counter in device memory (a bounded wait); then
+// stamped with the launch's epoch, and polls the stamped counts of the other workgroups
+// (a bounded wait; no counter, no clearing, nothing between the launches of two calls); then
 // every workgroup adds up the counts of all workgroups (expert offsets) and of the
 // workgroups before it (its own start positions) and scatters its (token, slot) pairs.
 // A workgroup whose wait runs out (the others kept off the chip by unrelated work) does
 // not depend on them any more: it counts every token's choices itself, from the logits.
-// The counter is cleared by a one-workgroup fill kernel queued in front.
 //
 // More tokens than that: three launches over 256-token workgroups,
 //   route_topk     one lane per token; LDS histogram of the workgroup's expert ids
@@ -31,7 +31,9 @@
 //                  hits an expert at most once), plus the start position
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
+#include <cstdint>
 #include <cstdlib>
 #include <mutex>
 
@@ -171,16 +173,24 @@ __global__ __launch_bounds__(kBlock) void route_scatter_kernel(const long* __res
 
 
 // ---------------------------------------------------------------------------------------
-// One-launch routing.  Scratch layout (bytes): [0] arrival counter (u32, zero at launch),
-// [4] set to 1 by a workgroup whose bounded wait ran out (outputs are undefined then),
-// [kScratchHeader ...] int counts[nblk][E].
+// One-launch routing.  Scratch layout (bytes): [0, kScratchHeader) unused by this path,
+// [kScratchHeader ...] u64 words[nblk][E], word = (epoch << 16) | tokens of workgroup b that
+// chose expert e.  A word is valid for a launch when its upper bits equal the launch's epoch,
+// so the workgroups need no counter to meet at: each polls the words it needs.  Two ways to
+// make stale words invalid: the library's own scratch is only ever written by this kernel and
+// every launch on it gets an epoch no launch before it had (no clearing at all); scratch a
+// caller hands in holds anything, so a fill kernel queued in front zeroes the words and the
+// launch uses epoch 1 (this also is the form a graph can replay: the epoch is a kernel
+// argument and would be the same on every replay).
 constexpr int  kScratchHeader   = 256;
 constexpr int  kFusedMaxBlocks  = 256;          // 256-thread workgroups: all resident on 256 CUs
 constexpr long kFusedMaxTokens  = static_cast<long>(kFusedMaxBlocks) * kBlock;
-constexpr int  kSpinLimit       = 1 << 20;      // polls of ~64 clocks each: tens of milliseconds, then the workgroup counts for itself
+constexpr int  kSpinLimit       = 1 << 15;      // polls of a word, each a round trip to memory: tens of milliseconds, then the workgroup counts for itself
+constexpr int  kEpochShift      = 16;           // a workgroup's count is at most kBlock
 
-__global__ __launch_bounds__(64) void route_clear_kernel(unsigned* __restrict__ header) {
-    if (threadIdx.x < 2) header[threadIdx.x] = 0u;
+__global__ __launch_bounds__(kBlock) void route_clear_kernel(unsigned long long* __restrict__ words, long n) {
+    const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i < n) words[i] = 0ull;
 }
 
 // kSmall: E <= 8 and k <= 8, the row and the selection live in registers.
@@ -188,23 +198,29 @@ template <typename T, bool kSmall>
 __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     const typename Elem<T>::store_t* __restrict__ logits, long T_, int E, int k, long* __restrict__ topi,
     float* __restrict__ topw, long* __restrict__ order, long* __restrict__ inv_order, long* __restrict__ counts,
-    long* __restrict__ offsets, unsigned char* __restrict__ scratch, int spin_limit) {
+    long* __restrict__ offsets, unsigned char* __restrict__ scratch, unsigned long long epoch, int spin_limit) {
     using El = Elem<T>;
     __shared__ int wave_cnt[kWavesPerBlock][kMaxExperts];
     __shared__ long tot[kMaxExperts + 1];     // after the meeting: exclusive expert offsets
+    __shared__ int  all_cnt[kMaxExperts];     // tokens of expert e in all workgroups
     __shared__ int  pre[kMaxExperts];         // tokens of expert e in the workgroups before this one
     __shared__ int  gave_up;
     __shared__ int  recount[2][kMaxExperts];  // only used by a workgroup whose wait ran out
-    unsigned* header = reinterpret_cast<unsigned*>(scratch);
-    int* block_cnt = reinterpret_cast<int*>(scratch + kScratchHeader);
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(scratch + kScratchHeader);
     const int nblk = gridDim.x, bid = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const long t = static_cast<long>(bid) * kBlock + tid;
     const bool live = t < T_;
     if (tid == 0) gave_up = 0;
+    if (tid < kMaxExperts) {
+        all_cnt[tid] = 0;
+        pre[tid] = 0;
+    }
 
-    // ---- top-k and gate weights of this lane's token ---------------------------------
+    // ---- top-k of this lane's token ---------------------------------
     int sel[kSmall ? 8 : 1];                  // chosen expert per slot (small path)
+    double kept[kSmall ? 8 : 1];              // the kept values as fp32 (the softmax input is topv.float())
+    double vmax = -INFINITY;
     if (live) {
         const auto* row = logits + t * E;
         double val[kSmall ? 8 : 1];
@@ -219,10 +235,9 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
                 for (int j = 0; j < 8; ++j) val[j] = j < E ? El::to_f64(row[j]) : 0.0;
             }
         }
-        double prev_val = 0.0, vmax = -INFINITY;
+        double prev_val = 0.0;
         int prev_idx = -1;
         bool has_prev = false;
-        double kept[kSmall ? 8 : 1];          // the kept values as fp32 (the softmax input is topv.float())
         for (int s = 0; s < k; ++s) {
             double best_val = 0.0;
             int best_idx = -1;
@@ -258,7 +273,13 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
                     }
             }
         }
-        // gate weights: exp(v - max) / sum in fp64, narrowed to fp32
+    }
+    // gate weights: exp(v - max) / sum in fp64, narrowed to fp32 (evaluated after the counts are
+    // published, while they travel)
+    auto write_gate_weights = [&]() {
+        if (!live) return;
+        const auto* row = logits + t * E;
+        (void)row;
         if constexpr (kSmall) {
             double ex[8], sum = 0.0;
 #pragma unroll
@@ -281,7 +302,7 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
                 topw[t * k + s] = static_cast<float>(exp(static_cast<double>(El::to_f32(row[idx >= 0 ? idx : 0])) - vmax) / sum);
             }
         }
-    }
+        };
     // slot in which this lane's token chose expert e, or -1 (a token chooses an expert at most once)
     auto slot_of = [&](int e) -> int {
         int mine = -1;
@@ -308,26 +329,37 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
         int c = 0;
 #pragma unroll
         for (int w = 0; w < kWavesPerBlock; ++w) c += wave_cnt[w][tid];
-        __hip_atomic_store(&block_cnt[static_cast<long>(bid) * E + tid], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __hip_atomic_store(&words[static_cast<long>(bid) * E + tid], (epoch << kEpochShift) | static_cast<unsigned long long>(c),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __syncthreads();
+    write_gate_weights();
 
-    // ---- meet: every workgroup of the grid has published ------------------------------
-    if (tid == 0) {
-        __hip_atomic_fetch_add(&header[0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        int polls = 0;
-        while (__hip_atomic_load(&header[0], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < static_cast<unsigned>(nblk)) {
-            if (++polls >= spin_limit) {
-                gave_up = 1;
-                __hip_atomic_store(&header[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
+    // ---- meet: a lane polls a word until it carries this launch's epoch -------------------
+    {
+        bool ran_out = false;
+        const long n_words = static_cast<long>(nblk) * E;
+        for (long i = tid; i < n_words; i += kBlock) {
+            const unsigned long long* wp = &words[i];
+            unsigned long long w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            int polls = 1;
+            while ((w >> kEpochShift) != epoch) {
+                if (polls >= spin_limit) {
+                    ran_out = true;
+                    break;
+                }
+                ++polls;
+                __builtin_amdgcn_s_sleep(1);
+                w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            __builtin_amdgcn_s_sleep(1);
+            if (ran_out) break;
+            const int c = static_cast<int>(w & ((1ull << kEpochShift) - 1));
+            const int j = static_cast<int>(i / E), e = static_cast<int>(i % E);
+            atomicAdd(&all_cnt[e], c);
+            if (j < bid) atomicAdd(&pre[e], c);
         }
+        if (ran_out) gave_up = 1;
     }
     __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 
     // ---- totals (expert offsets) and the share of the workgroups before this one ---------
     if (gave_up) {
@@ -371,37 +403,28 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
         }
         __syncthreads();
         for (int e = tid; e < E; e += kBlock) {
-            tot[e] = recount[0][e];
+            all_cnt[e] = recount[0][e];
             pre[e] = recount[1][e];
         }
-    } else
-    for (int e = wave; e < E; e += kWavesPerBlock) {
-        int all = 0, before = 0;
-        for (int j = lane; j < nblk; j += kWave) {
-            const int c = __hip_atomic_load(&block_cnt[static_cast<long>(j) * E + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            all += c;
-            before += j < bid ? c : 0;
-        }
-        all = wave_allreduce(all, [](int a, int b) { return a + b; });
-        before = wave_allreduce(before, [](int a, int b) { return a + b; });
-        if (lane == 0) {
-            tot[e] = all;
-            pre[e] = before;
-        }
+        __syncthreads();
     }
-    __syncthreads();
-    if (tid == 0) {
-        long run = 0;
-        for (int e = 0; e < E; ++e) {
-            const long c = tot[e];
-            if (bid == 0) {
-                counts[e] = c;
-                offsets[e] = run;
-            }
-            tot[e] = run;
-            run += c;
+    // exclusive scan over the experts by the first wave (E <= 64, totals below 2^31)
+    if (wave == 0) {
+        const int c = lane < E ? all_cnt[lane] : 0;
+        int incl = c;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const int up = __shfl_up(incl, d, kWave);
+            if (lane >= d) incl += up;
         }
-        if (bid == 0) offsets[E] = run;
+        if (lane < E) {
+            tot[lane] = incl - c;
+            if (bid == 0) {
+                counts[lane] = c;
+                offsets[lane] = incl - c;
+                if (lane == E - 1) offsets[E] = incl;
+            }
+        }
     }
     __syncthreads();
 
@@ -419,41 +442,51 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     }
 }
 
+// epoch 0: `scratch` may hold anything -- its words are zeroed by a fill kernel queued in front and
+// the launch runs as epoch 1.  Otherwise `scratch` is the library's own and `epoch` is new to it.
 template <typename T>
 void launch_fused(const void* logits, long T_, int E, int k, long* topi, float* topw, long* order, long* inv_order,
-                  long* counts, long* offsets, unsigned char* scratch, hipStream_t s) {
+                  long* counts, long* offsets, unsigned char* scratch, unsigned long long epoch, hipStream_t s) {
     using store_t = typename Elem<T>::store_t;
-    const dim3 grid(static_cast<unsigned>((T_ + kBlock - 1) / kBlock)), block(kBlock);
+    const long nblk = (T_ + kBlock - 1) / kBlock;
+    const dim3 grid(static_cast<unsigned>(nblk)), block(kBlock);
     // PARAS_ROUTE_SPIN_LIMIT: polls before a workgroup stops waiting for the others (tests set 1 to
     // drive the workgroups through the path that counts for itself)
     const char* env = std::getenv("PARAS_ROUTE_SPIN_LIMIT");
     const int spin = env != nullptr && std::atoi(env) > 0 ? std::atoi(env) : kSpinLimit;
-    hipLaunchKernelGGL(route_clear_kernel, dim3(1), dim3(64), 0, s, reinterpret_cast<unsigned*>(scratch));
+    if (epoch == 0) {
+        const long n_words = nblk * E;
+        hipLaunchKernelGGL(route_clear_kernel, dim3(static_cast<unsigned>((n_words + kBlock - 1) / kBlock)), block, 0, s,
+                           reinterpret_cast<unsigned long long*>(scratch + kScratchHeader), n_words);
+        epoch = 1;
+    }
     if (E <= 8 && k <= 8)
         hipLaunchKernelGGL((route_fused_kernel<T, true>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, spin);
+                           topw, order, inv_order, counts, offsets, scratch, epoch, spin);
     else
         hipLaunchKernelGGL((route_fused_kernel<T, false>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, spin);
+                           topw, order, inv_order, counts, offsets, scratch, epoch, spin);
 }
 
 // Shared by the entry points: routes on `scratch` (device memory of route_scratch_bytes(T, E)).
 int route_on(const void* logits, long T_, int E, int k, int dtype, long* topi, float* topw, long* order, long* inv_order,
-             long* counts, long* offsets, unsigned char* scratch, hipStream_t s) {
+             long* counts, long* offsets, unsigned char* scratch, unsigned long long epoch, hipStream_t s) {
     switch (dtype) {
-        case PARAS_F32:  launch_fused<float>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
-        case PARAS_F64:  launch_fused<double>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
-        case PARAS_BF16: launch_fused<bf16_t>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
-        case PARAS_F16:  launch_fused<f16_t>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, s); break;
+        case PARAS_F32:  launch_fused<float>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, epoch, s); break;
+        case PARAS_F64:  launch_fused<double>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, epoch, s); break;
+        case PARAS_BF16: launch_fused<bf16_t>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, epoch, s); break;
+        case PARAS_F16:  launch_fused<f16_t>(logits, T_, E, k, topi, topw, order, inv_order, counts, offsets, scratch, epoch, s); break;
         default: return fail(PARAS_ERR_INVALID, "paras_moe_route: unknown dtype %d", dtype);
     }
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
 }
 
+// Bytes a caller's workspace must hold: the words of the one-launch path (8 bytes each), which also
+// covers the int histograms of the three-launch path.
 size_t route_scratch_bytes(long T_, long E) {
     const long nblk = (T_ + kBlock - 1) / kBlock;
-    return static_cast<size_t>(kScratchHeader) + static_cast<size_t>(nblk * E) * sizeof(int);
+    return static_cast<size_t>(kScratchHeader) + static_cast<size_t>(nblk * E) * sizeof(unsigned long long);
 }
 
 
@@ -461,7 +494,7 @@ size_t route_scratch_bytes(long T_, long E) {
 // Scratch of the allocation-free entry point: one copy per GPU, held until the process ends.
 // Its name is a host-side stand-in, not a device address: host code only ever uses the
 // per-device address hipGetSymbolAddress returns (static_scratch_for below).
-constexpr size_t kStaticScratchBytes = static_cast<size_t>(kScratchHeader) + static_cast<size_t>(kFusedMaxBlocks) * kMaxExperts * sizeof(int);
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(kScratchHeader) + static_cast<size_t>(kFusedMaxBlocks) * kMaxExperts * sizeof(unsigned long long);
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxGpus = 64;
@@ -482,6 +515,46 @@ int static_scratch_for(unsigned char** out) {
     }
     *out = g_scratch_ptr[dev];
     return PARAS_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// The library's own scratch for paras_moe_route: kEpochSlots areas per GPU that only
+// route_fused_kernel ever writes (zero when the module is loaded), handed out in turn so that
+// calls running side by side on different streams rarely share one.  If two launches do share
+// an area, each sees the other's epoch in some words, waits its polls out and counts for itself:
+// slow, never wrong.  As for `scratch`, host code uses the per-device address only.
+constexpr int kEpochSlots = 4;
+static __device__ __align__(256) unsigned char epoch_scratch[kEpochSlots * kStaticScratchBytes];
+unsigned char* g_epoch_scratch_ptr[kMaxGpus] = {};
+std::atomic<unsigned long long> g_epoch{2};        // 0: "clear first", 1: the epoch of a cleared area
+std::atomic<unsigned> g_epoch_slot{0};
+
+int epoch_scratch_for(unsigned char** out) {
+    int dev = -1;
+    PARAS_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxGpus) {
+        *out = nullptr;          // beyond the table: the caller's workspace serves
+        return PARAS_OK;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_epoch_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        PARAS_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(epoch_scratch)));
+        if (ptr == nullptr) return fail(PARAS_ERR_HIP, "paras_moe_route: no device address for the routing scratch");
+        g_epoch_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+    }
+    *out = g_epoch_scratch_ptr[dev];
+    return PARAS_OK;
+}
+
+// True when work queued on `s` now is being recorded into a graph (or that cannot be told).
+bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
 }
 
 }  // namespace
@@ -518,9 +591,25 @@ int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dty
     const long nblk = (T + kBlock - 1) / kBlock;
     PARAS_REQUIRE(nblk <= 0x7fffffffL && T * k <= 0x7fffffffL, "paras_moe_route: too many routed rows");
     long* ti = reinterpret_cast<long*>(topi);
-    if (T <= kFusedMaxTokens)
+    if (T <= kFusedMaxTokens) {
+        // One launch on the library's own scratch with a fresh epoch.  A stream that is being captured
+        // into a graph gets the replayable form instead (the workspace's words zeroed by a fill kernel
+        // in front, epoch 1); PARAS_ROUTE_OWN_SCRATCH=0 asks for that form everywhere.
+        unsigned char* area = static_cast<unsigned char*>(workspace);
+        unsigned long long epoch = 0;
+        const char* own = std::getenv("PARAS_ROUTE_OWN_SCRATCH");
+        if ((own == nullptr || std::atoi(own) != 0) && !stream_is_capturing(s)) {
+            unsigned char* base = nullptr;
+            rc = epoch_scratch_for(&base);
+            if (rc != PARAS_OK) return rc;
+            if (base != nullptr) {
+                area = base + static_cast<size_t>(g_epoch_slot.fetch_add(1, std::memory_order_relaxed) % kEpochSlots) * kStaticScratchBytes;
+                epoch = g_epoch.fetch_add(1, std::memory_order_relaxed);
+            }
+        }
         return route_on(logits, T, (int)E, (int)k, dtype, ti, topw, reinterpret_cast<long*>(order), reinterpret_cast<long*>(inv_order),
-                        reinterpret_cast<long*>(counts), reinterpret_cast<long*>(offsets), static_cast<unsigned char*>(workspace), s);
+                        reinterpret_cast<long*>(counts), reinterpret_cast<long*>(offsets), area, epoch, s);
+    }
     int* hist = reinterpret_cast<int*>(static_cast<unsigned char*>(workspace) + kScratchHeader);
     const dim3 grid(static_cast<unsigned>(nblk)), block(kBlock);
     switch (dtype) {
@@ -565,10 +654,10 @@ int paras_moe_route_noalloc(const void* logits, int64_t T, int64_t E, int64_t k,
     unsigned char* ptr = nullptr;
     rc = static_scratch_for(&ptr);
     if (rc != PARAS_OK) return rc;
-    // The counter in the scratch header is cleared by the fill kernel route_on queues first;
-    // the per-workgroup counts behind it are rewritten before they are read.
+    // Epoch 0: the words of the scratch that this call uses are zeroed by the fill kernel route_on
+    // queues first (the form a graph can replay).
     return route_on(logits, T, (int)E, (int)k, dtype, reinterpret_cast<long*>(topi), topw, reinterpret_cast<long*>(order),
-                    reinterpret_cast<long*>(inv_order), reinterpret_cast<long*>(counts), reinterpret_cast<long*>(offsets), ptr, s);
+                    reinterpret_cast<long*>(inv_order), reinterpret_cast<long*>(counts), reinterpret_cast<long*>(offsets), ptr, 0ull, s);
 }
 
 }  // extern "C"

@@ -258,9 +258,14 @@ PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 /* inv_order: [T*k] int64 (position of flat slot in `order`; may be NULL);    */
 /* counts: [E] int64; offsets: [E+1] int64.  1 <= k <= E <= 64.               */
 /* `workspace`: paras_moe_route_workspace(T,E,k) bytes of device memory        */
-/* (an arrival counter and per-workgroup expert counts; contents on entry do   */
-/* not matter).  Up to 65536 tokens the whole routing is one kernel whose      */
-/* workgroups meet at that counter.                                            */
+/* (per-workgroup expert counts; contents on entry do not matter).  Up to      */
+/* 65536 tokens the whole routing is one kernel: its workgroups publish their  */
+/* counts stamped with the call's epoch and poll each other's.  Outside graph  */
+/* capture that kernel is the only launch and the stamped counts live in the   */
+/* library's own device memory (4 areas of 131,328 bytes per GPU, taken in     */
+/* turn; calls that overlap on one area stay exact and turn slow); on a stream */
+/* that is being captured, or with PARAS_ROUTE_OWN_SCRATCH=0, they live in     */
+/* `workspace`, which a fill kernel queued in front clears.                    */
 /* ------------------------------------------------------------------------- */
 PARAS_API size_t paras_moe_route_workspace(int64_t T, int64_t E, int64_t k);
 PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k,
@@ -271,9 +276,9 @@ PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t 
 /* paras_moe_route for callers that cannot allocate (code under HIP graph
  * capture, serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments and same outputs, bit for bit,
- * without the workspace: the per-workgroup counts and the arrival counter live
- * in a fixed array in the library's device image (65,792 bytes per GPU, held
- * until the process ends).  Limits: 1 <= T <= 65536 tokens, E <= 64; larger
+ * without the workspace: the per-workgroup counts live in a fixed array in the
+ * library's device image (131,328 bytes per GPU, held until the process ends),
+ * cleared by a fill kernel queued in front of the routing kernel.  Limits: 1 <= T <= 65536 tokens, E <= 64; larger
  * inputs are PARAS_ERR_INVALID.  The call allocates nothing and frees nothing.
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU
  * (two streams, two threads) race; calls queued on one stream do not. */

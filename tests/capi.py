@@ -199,7 +199,7 @@ def sdpa(q, k, v, mask=None, is_causal=False, scale=None, want_attn=False, want_
     return out, attn, lse, name
 
 
-def moe_route(logits, k):
+def moe_route(logits, k, workspace=None):
     logits = logits.contiguous()
     T, E = logits.shape
     dev = logits.device
@@ -209,7 +209,9 @@ def moe_route(logits, k):
     inv = torch.empty(T * k, dtype=torch.int64, device=dev)
     counts = torch.empty(E, dtype=torch.int64, device=dev)
     offsets = torch.empty(E + 1, dtype=torch.int64, device=dev)
-    ws = torch.empty(max(1, lib().paras_moe_route_workspace(T, E, k)), dtype=torch.uint8, device=dev)
+    ws = workspace
+    if ws is None:
+        ws = torch.empty(max(1, lib().paras_moe_route_workspace(T, E, k)), dtype=torch.uint8, device=dev)
     check(lib().paras_moe_route(_ptr(logits), T, E, k, DT[logits.dtype], _ptr(topi), _ptr(topw), _ptr(order),
                                 _ptr(inv), _ptr(counts), _ptr(offsets), _ptr(ws), _stream()))
     return topi, topw, order, inv, counts, offsets

@@ -212,3 +212,79 @@ def test_route_when_the_workgroups_do_not_wait_for_each_other(shape, monkeypatch
     got = capi.moe_route_noalloc(logits.cuda(), k)
     for name, g, w in zip(NAMES, got, want):
         assert_bit_exact(g, w, f"moe_route_noalloc {name} without waiting")
+
+
+def test_route_calls_of_changing_shapes_one_after_another():
+    """The one-launch routing keeps its scratch inside the library and never clears it: what an
+    earlier call of another shape left there must not count for a later one."""
+    torch.manual_seed(77)
+    for T, E, k, dtype in [(65536, 8, 2, torch.bfloat16), (300, 64, 8, torch.float32), (65536, 8, 2, torch.bfloat16),
+                           (8192, 8, 2, torch.bfloat16), (65000, 64, 4, torch.float16), (8192, 8, 2, torch.bfloat16),
+                           (1, 8, 2, torch.bfloat16), (257, 3, 1, torch.float32)]:
+        logits = torch.randn(T, E).to(dtype)
+        for _ in range(2):
+            got = capi.moe_route(logits.cuda(), k)
+            for name, g, w in zip(NAMES, got, O.moe_route(logits, k)):
+                assert_bit_exact(g, w, f"moe_route {name} T{T} E{E} k{k}")
+
+
+def test_route_on_a_callers_workspace_that_holds_stale_counts(monkeypatch):
+    """PARAS_ROUTE_OWN_SCRATCH=0: the form used under graph capture.  The workspace is the caller's
+    and may hold anything, here words that look like published counts: they are cleared first."""
+    monkeypatch.setenv("PARAS_ROUTE_OWN_SCRATCH", "0")
+    torch.manual_seed(78)
+    for T, E, k, dtype in [(8192, 8, 2, torch.bfloat16), (3000, 64, 6, torch.float32)]:
+        logits = torch.randn(T, E).to(dtype)
+        n = capi.lib().paras_moe_route_workspace(T, E, k)
+        ws = torch.empty((n + 7) // 8, dtype=torch.int64, device="cuda")
+        for stale in ((1 << 16) | 77, -1):
+            ws.fill_(stale)
+            got = capi.moe_route(logits.cuda(), k, workspace=ws)
+            for name, g, w in zip(NAMES, got, O.moe_route(logits, k)):
+                assert_bit_exact(g, w, f"moe_route {name} on a workspace of stale words")
+
+
+def test_route_calls_side_by_side_on_many_streams():
+    """More streams than the library has scratch areas: calls that share one may see each other's
+    epochs, wait their polls out and count for themselves.  Slow then, and still exact."""
+    torch.manual_seed(79)
+    k = 2
+    streams = [torch.cuda.Stream() for _ in range(6)]
+    inputs = [torch.randn(4096 + 512 * i, 8).bfloat16() for i in range(len(streams))]
+    on_dev = [x.cuda() for x in inputs]
+    torch.cuda.synchronize()
+    results = []
+    for _ in range(3):
+        for s, x in zip(streams, on_dev):
+            with torch.cuda.stream(s):
+                results.append((x, capi.moe_route(x, k)))
+    torch.cuda.synchronize()
+    want = {id(x): O.moe_route(c, k) for x, c in zip(on_dev, inputs)}
+    for x, got in results:
+        for name, g, w in zip(NAMES, got, want[id(x)]):
+            assert_bit_exact(g, w, f"moe_route {name} T{x.shape[0]} among other streams")
+
+
+def test_route_recorded_into_a_graph_and_replayed():
+    """A stream that is being captured gets the replayable form of the routing (a fill kernel clears
+    the caller's workspace, no epoch from the host).  Replays with new logits, eager calls and
+    synchronizations in between, each checked against the oracle."""
+    torch.manual_seed(80)
+    T, E, k = 8192, 8, 2
+    static_logits = torch.randn(T, E).bfloat16().cuda()
+    capi.moe_route(static_logits, k)                     # everything one-time is done before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = capi.moe_route(static_logits, k)
+    for trial in range(4):
+        fresh = torch.randn(T, E).bfloat16()
+        static_logits.copy_(fresh.cuda())
+        eager = capi.moe_route(static_logits, k)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = O.moe_route(fresh, k)
+        for name, g, e, w in zip(NAMES, recorded, eager, want):
+            assert_bit_exact(g, w, f"replay {trial}: moe_route {name}")
+            assert_bit_exact(e, w, f"eager call {trial}: moe_route {name}")
