@@ -12,16 +12,23 @@
 // lands on the other side of a rounding boundary (one unit in the last place of T, for about one
 // weight in a thousand), and `out` differs by the accumulation order of the products.
 //
-// Two passes over the keys per block of 128 queries (4 wavefronts x 32 queries, a lane owns a
-// query as in the flash kernel: S^T = K Q^T on v_mfma_f32_32x32x16, O^T = V^T W^T):
-//   pass 1   scores tile by tile, running row max and row sum (each lane over its own half of the
-//            keys; the two halves of a query are merged once at the end)
+// Two passes over the keys per block of 128 queries (a lane owns a query as in the flash kernel:
+// S^T = K Q^T on v_mfma_f32_32x32x16, O^T = V^T W^T):
+//   pass 1   scores tile by tile, running row max and row sum (each lane over its own share of the
+//            keys; the shares of a query are merged once at the end)
 //   pass 2   scores again, weights written to `attn`, and the product with V accumulated
-// K / V tiles of 64 keys go global -> registers -> LDS (one buffer each, two barriers per tile:
-// this path feeds callers that ask for O(Lq Lk) output, its time is dominated by writing it).
+// The arithmetic per score, not memory, sets the pace (two roundings, a scaling, the mask, an
+// exponential, a narrowing), so the work of a query block is spread over eight wavefronts: four
+// groups of 32 queries times two halves of every 128-key tile.  K / V tiles go global -> registers
+// -> LDS, double buffered: the next tile's loads are in flight while the current one is computed,
+// one barrier per tile.  Under a causal mask a workgroup takes a pair of query blocks, the i-th
+// from the end and the i-th from the start, so every workgroup walks the same number of key tiles;
+// blocks of 32 keys that lie wholly below the diagonal skip the per-key tests.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <mutex>
+#include <set>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
@@ -31,7 +38,8 @@
 namespace paras {
 namespace {
 
-constexpr int kBN = 64;    // keys per tile
+constexpr int kBN = 64;    // keys per key group and tile
+constexpr int kTile = 128; // keys per staged tile: two key groups
 constexpr int kBM = 128;   // queries per workgroup: 4 waves x 32
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -50,6 +58,7 @@ struct WeightsParams {
     int  B, Hq, Hkv, Lq, Lk;
     int  n_qblocks;
     double scale;           // multiplies T(q k^T) in double, as the host engine's mul_out does
+    int    scale_is_f32;    // the scale is a float: an fp32 multiply gives the same rounded product
     const unsigned char* mask;
     long ms_b, ms_h, ms_q;  // element strides (0 = broadcast); the key stride is 1
 };
@@ -77,57 +86,61 @@ __device__ __forceinline__ void halves(float x, float& lo, float& hi) {
 }
 
 // kMode: 0 no mask, 1 bool mask bytes (nonzero = attend), 2 additive mask of type T, 3 causal.
+//
+// Eight wavefronts per workgroup: wave = query group (0..3, 32 queries each) + 4 * key group
+// (0..1).  A staged tile holds 128 keys; key group g works on its keys [64 g, 64 g + 64).  The two
+// waves that share queries merge their row maxima and sums after pass 1 and their partial W V
+// products after pass 2, both through LDS.
 template <typename T, int D, int kMode>
-__global__ __launch_bounds__(256, 2) void weights_fwd_kernel(const WeightsParams p) {
+__global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams p) {
     using El = Elem<T>;
-    constexpr int NW = 4;
+    constexpr int NW = 8;
     constexpr int KSTEPS = D / 16;
     constexpr int DBLK = D / 32;
     constexpr int CHUNKS = D / 8;          // 16-byte chunks per row
     constexpr int RPI = 64 / CHUNKS;       // rows one wave moves per instruction
-    constexpr int NI = kBN / (RPI * NW);
+    constexpr int NI = kTile / (RPI * NW);
     auto ksw = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
     auto vsw = [](int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
-    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds[kBN * D];
-    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds[kBN * D];
+    // [K stage 0][K stage 1][V stage 0][V stage 1], kTile * D elements each (the launcher sizes it)
+    extern __shared__ __attribute__((aligned(1024))) std::uint16_t tiles[];
+    __shared__ float x_m[2][kBM], x_l[2][kBM];
+    auto k_buf = [&](int stage) { return tiles + stage * (kTile * D); };
+    auto v_buf = [&](int stage) { return tiles + (2 + stage) * (kTile * D); };
 
     const int nq = p.n_qblocks;
-    const int bh = blockIdx.x / nq, qblock = nq - 1 - blockIdx.x % nq;   // heaviest causal blocks first
+    const int per_bh = kMode == 3 ? (nq + 1) / 2 : nq;            // workgroups per (batch, head)
+    const int bh = blockIdx.x / per_bh, slot_in_bh = blockIdx.x % per_bh;
     const int b = bh / p.Hq, hq = bh % p.Hq;
     const int hkv = hq / (p.Hq / p.Hkv);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qw = wave & 3, kg = wave >> 2;
     const int lq = lane & 31, lh = lane >> 5;
-    const int q0 = qblock * kBM + wave * 32;
-    const int my_q = q0 + lq;
-    const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
-
-    i16x8 qreg[KSTEPS];
-    {
-        const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) qreg[ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
-    }
     const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
     const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
-
-    int n_tiles = (p.Lk + kBN - 1) / kBN;
-    if (kMode == 3) {   // keys beyond the workgroup's last query carry zero weight: written as zeros below, not computed
-        const int last_q = min(qblock * kBM + kBM, p.Lq) - 1;
-        n_tiles = (min(last_q + 1, p.Lk) + kBN - 1) / kBN;
-    }
-
-    // staging: 64 rows of K (and V), 16 bytes per thread and step, rows past Lk as zeros; the 16-byte
-    // chunks of a row are XOR-swizzled so that operand reads and transposed reads are conflict free
     const int srow = wave * RPI + lane / CHUNKS, slot = lane % CHUNKS;
-    auto stage = [&](const std::uint16_t* base, long row_stride, int first, std::uint16_t* tile, bool is_v) {
-        u32x4 regs[NI];
+    const int grp = lane >> 4, m16 = lane & 15;
+    int k_rd[KSTEPS], v_rd[DBLK];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) k_rd[ks] = (kg * kBN + lq) * D + (((2 * ks + lh) ^ ksw(lq)) * 8);
+    {
+        const int vrow = 4 * lh + (m16 >> 2);
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+            v_rd[db] = (kg * kBN + vrow) * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
+    }
+    // staging: 128 rows of K (and V), 16 bytes per thread and step, rows past Lk as zeros; the 16-byte
+    // chunks of a row are XOR-swizzled so that operand reads and transposed reads are conflict free
+    auto fetch = [&](const std::uint16_t* base, long row_stride, int first, u32x4 (&regs)[NI]) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int row = first + i * RPI * NW + srow;
             regs[i] = u32x4{0u, 0u, 0u, 0u};
             if (row < p.Lk) regs[i] = load16(base + static_cast<long>(row) * row_stride + slot * 8);
         }
+    };
+    auto put = [&](const u32x4 (&regs)[NI], std::uint16_t* tile, bool is_v) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int r = i * RPI * NW + srow;
@@ -135,196 +148,292 @@ __global__ __launch_bounds__(256, 2) void weights_fwd_kernel(const WeightsParams
             *reinterpret_cast<u32x4*>(tile + r * D + ((slot ^ sw) * 8)) = regs[i];
         }
     };
+    // Rounds to T and widens again.  For the intermediate roundings the conversion instructions serve:
+    // they round like the host, and a NaN stays a NaN (its payload does not matter here, only the
+    // final narrowing of a weight decides the bits that are written).
+    auto round_T = [](float x) { return El::to_f32(El::from_f32_finite(x)); };
+    const float scale_f = static_cast<float>(p.scale);
 
-    const int grp = lane >> 4, m16 = lane & 15;
-    int k_rd[KSTEPS], v_rd[DBLK];
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) k_rd[ks] = lq * D + (((2 * ks + lh) ^ ksw(lq)) * 8);
-    {
-        const int vrow = 4 * lh + (m16 >> 2);
-#pragma unroll
-        for (int db = 0; db < DBLK; ++db)
-            v_rd[db] = vrow * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
-    }
+    // causal: the query block `slot_in_bh` from the end, then the same from the start
+    const int n_parts = (kMode == 3 && slot_in_bh != nq - 1 - slot_in_bh) ? 2 : 1;
+    for (int part = 0; part < n_parts; ++part) {
+        const int qblock = kMode == 3 ? (part == 0 ? nq - 1 - slot_in_bh : slot_in_bh) : slot_in_bh;
+        const int q0 = qblock * kBM + qw * 32;
+        const int my_q = q0 + lq;
+        const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
 
-    const unsigned char* mrow = nullptr;
-    if constexpr (kMode == 1 || kMode == 2)
-        mrow = p.mask + (static_cast<long>(b) * p.ms_b + static_cast<long>(hq) * p.ms_h + static_cast<long>(qrow) * p.ms_q) * (kMode == 1 ? 1 : 2);
-
-    // Narrowed, scaled and masked scores of one 32-key block (block `jb` of the staged tile,
-    // first key `key0`): accumulator register r of lane (query lq, half lh) is key
-    // key0 + (r/4)*8 + 4*lh + r%4.
-    auto scores = [&](int jb, int key0, float16_t& sc) {
+        i16x8 qreg[KSTEPS];
+        {
+            const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks)
-            sc = Mma16<T>::run(*reinterpret_cast<const i16x8*>(&k_lds[jb * 32 * D + k_rd[ks]]), qreg[ks], sc);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
-            float s = El::to_f32(El::from_f32(sc[r]));                 // T(q k^T)
-            s = El::to_f32(El::from_f64(static_cast<double>(s) * p.scale));   // T(s1 * scale), evaluated in double
-            bool dead = key >= p.Lk;
-            if constexpr (kMode == 3) dead = dead || key > my_q;
-            if constexpr (kMode == 1) dead = dead || (key < p.Lk && mrow[key] == 0);
-            if constexpr (kMode == 2) {
-                if (key < p.Lk) {
-                    const float m = El::to_f32(*reinterpret_cast<const std::uint16_t*>(mrow + 2 * static_cast<long>(key)));
-                    s = El::to_f32(El::from_f32(s + m));               // T(s2 + mask)
-                }
-            }
-            sc[r] = dead ? -INFINITY : s;
+            for (int ks = 0; ks < KSTEPS; ++ks) qreg[ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
         }
-    };
-
-    // ---- pass 1: row max and row sum of exp over the narrowed scores
-    float m_run = -INFINITY, l_run = 0.f;
-    for (int t = 0; t < n_tiles; ++t) {
-        stage(kbase, p.ks_l, t * kBN, k_lds, false);
-        __syncthreads();
-#pragma unroll
-        for (int jb = 0; jb < 2; ++jb) {
-            const int key0 = t * kBN + jb * 32;
-            if (key0 >= p.Lk || (kMode == 3 && key0 > q0 + 31)) continue;   // wave-uniform
-            float16_t sc;
-            scores(jb, key0, sc);
-            float mx = sc[0];
-#pragma unroll
-            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
-            const float m_new = fmaxf(m_run, mx);
-            if (m_new != -INFINITY) {
-                float add = 0.f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) add += __expf(sc[r] - m_new);
-                l_run = (m_run == -INFINITY ? 0.f : l_run * __expf(m_run - m_new)) + add;
-                m_run = m_new;
-            }
+        int n_tiles = (p.Lk + kTile - 1) / kTile;
+        if (kMode == 3) {   // keys beyond the workgroup's last query carry zero weight: written as zeros below, not computed
+            const int last_q = min(qblock * kBM + kBM, p.Lq) - 1;
+            n_tiles = (min(last_q + 1, p.Lk) + kTile - 1) / kTile;
         }
-        __syncthreads();
-    }
-    {   // merge the two halves of each query
-        float m_lo, m_hi, l_lo, l_hi;
-        halves(m_run, m_lo, m_hi);
-        halves(l_run, l_lo, l_hi);
-        const float m_all = fmaxf(m_lo, m_hi);
-        float l_all = 0.f;
-        if (m_all != -INFINITY) {
-            if (m_lo != -INFINITY) l_all += l_lo * __expf(m_lo - m_all);
-            if (m_hi != -INFINITY) l_all += l_hi * __expf(m_hi - m_all);
-        }
-        m_run = m_all;
-        l_run = l_all;
-    }
-    // A row without a visible key: max = -inf, every exp(-inf - -inf) is NaN, as in the reference's softmax.
-    const float inv_l = 1.0f / l_run;
 
-    // ---- pass 2: weights out, product with V
-    float16_t oacc[DBLK];
+        const unsigned char* mrow = nullptr;
+        if constexpr (kMode == 1 || kMode == 2)
+            mrow = p.mask + (static_cast<long>(b) * p.ms_b + static_cast<long>(hq) * p.ms_h + static_cast<long>(qrow) * p.ms_q) * (kMode == 1 ? 1 : 2);
+
+        // Narrowed, scaled and masked scores of one 32-key block (block `jb` of this key group's half of
+        // the staged tile, first key `key0`): accumulator register r of lane (query lq, half lh) is key
+        // key0 + (r/4)*8 + 4*lh + r%4.  `edge`: the block reaches past the row's end or past the diagonal
+        // (wave-uniform); only then the keys are tested one by one.
+        auto scores = [&](const std::uint16_t* k_lds, int jb, int key0, float16_t& sc) {
 #pragma unroll
-    for (int i = 0; i < DBLK; ++i)
+            for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-    std::uint16_t* arow = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + qrow) * p.Lk;
-    const bool row_live = my_q < p.Lq;
-    const bool wide = (p.Lk % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.attn) & 7) == 0);   // 8-byte runs of four weights
-    for (int t = 0; t < n_tiles; ++t) {
-        stage(kbase, p.ks_l, t * kBN, k_lds, false);
-        stage(vbase, p.vs_l, t * kBN, v_lds, true);
-        __syncthreads();
+            for (int ks = 0; ks < KSTEPS; ++ks)
+                sc = Mma16<T>::run(*reinterpret_cast<const i16x8*>(&k_lds[jb * 32 * D + k_rd[ks]]), qreg[ks], sc);
+            // T(T(q k^T) * scale).  The host multiplies in double; when the scale is a float the product
+            // of it and a value of T is exact in double, so one fp32 multiply rounds to the same float.
+            if (p.scale_is_f32) {
 #pragma unroll
-        for (int jb = 0; jb < 2; ++jb) {
-            const int key0 = t * kBN + jb * 32;
-            if (key0 >= p.Lk) continue;
-            const bool skipped = kMode == 3 && key0 > q0 + 31;   // wave-uniform: this wave's queries see none of these keys
-            float16_t sc;
-            std::uint32_t pw[8];
-            if (!skipped) {
-                scores(jb, key0, sc);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float w0 = __expf(sc[2 * i] - m_run) * inv_l, w1 = __expf(sc[2 * i + 1] - m_run) * inv_l;
-                    pw[i] = static_cast<std::uint32_t>(El::from_f32(w0)) | (static_cast<std::uint32_t>(El::from_f32(w1)) << 16);
-                }
+                for (int r = 0; r < 16; ++r) sc[r] = round_T(round_T(sc[r]) * scale_f);
             } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) pw[i] = 0u;
+                for (int r = 0; r < 16; ++r)
+                    sc[r] = round_T(static_cast<float>(static_cast<double>(round_T(sc[r])) * p.scale));
             }
+            const bool edge = key0 + 32 > p.Lk || (kMode == 3 && key0 + 31 > q0);
+            if (kMode == 1 || kMode == 2 || edge) {
+                // masks, without a branch per element (reads past the row's end are clamped into it)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                    const int key_in = key < p.Lk ? key : p.Lk - 1;
+                    float s = sc[r];
+                    bool dead = key >= p.Lk;
+                    if constexpr (kMode == 3) dead = dead || key > my_q;
+                    if constexpr (kMode == 1) dead = dead || mrow[key_in] == 0;
+                    if constexpr (kMode == 2)
+                        s = round_T(s + El::to_f32(*reinterpret_cast<const std::uint16_t*>(mrow + 2 * static_cast<long>(key_in))));   // T(s2 + mask)
+                    sc[r] = dead ? -INFINITY : s;
+                }
+            }
+        };
+
+        // ---- pass 1: row max and row sum of exp over the narrowed scores
+        float m_run = -INFINITY, l_run = 0.f;
+        u32x4 kreg[NI], vreg[NI];
+        __syncthreads();                       // (second part: everyone is done with the buffers of the first)
+        fetch(kbase, p.ks_l, 0, kreg);
+        put(kreg, k_buf(0), false);
+        __syncthreads();
+        for (int t = 0; t < n_tiles; ++t) {
+            const std::uint16_t* k_lds = k_buf(t & 1);
+            if (t + 1 < n_tiles) fetch(kbase, p.ks_l, (t + 1) * kTile, kreg);   // in flight during this tile's work
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb) {
+                const int key0 = t * kTile + kg * kBN + jb * 32;
+                if (key0 >= p.Lk || (kMode == 3 && key0 > q0 + 31)) continue;   // wave-uniform
+                float16_t sc;
+                scores(k_lds, jb, key0, sc);
+                float mx = sc[0];
+#pragma unroll
+                for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+                const float m_new = fmaxf(m_run, mx);
+                if (m_new != -INFINITY) {
+                    float add = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) add += __expf(sc[r] - m_new);
+                    l_run = (m_run == -INFINITY ? 0.f : l_run * __expf(m_run - m_new)) + add;
+                    m_run = m_new;
+                }
+            }
+            // the other buffer was last read one tile ago, before the barrier that ended that tile
+            if (t + 1 < n_tiles) put(kreg, k_buf((t + 1) & 1), false);
+            __syncthreads();
+        }
+        {   // merge the two halves of each query, then the two key groups
+            float m_lo, m_hi, l_lo, l_hi;
+            halves(m_run, m_lo, m_hi);
+            halves(l_run, l_lo, l_hi);
+            auto merge = [](float ma, float la, float mb, float lb, float& m_out, float& l_out) {
+                const float m_all = fmaxf(ma, mb);
+                float l_all = 0.f;
+                if (m_all != -INFINITY) {
+                    if (ma != -INFINITY) l_all += la * __expf(ma - m_all);
+                    if (mb != -INFINITY) l_all += lb * __expf(mb - m_all);
+                }
+                m_out = m_all;
+                l_out = l_all;
+            };
+            merge(m_lo, l_lo, m_hi, l_hi, m_run, l_run);
+            if (lh == 0) {
+                x_m[kg][qw * 32 + lq] = m_run;
+                x_l[kg][qw * 32 + lq] = l_run;
+            }
+            __syncthreads();
+            // both groups combine in the same order (group 0 first), so they agree to the bit
+            merge(x_m[0][qw * 32 + lq], x_l[0][qw * 32 + lq], x_m[1][qw * 32 + lq], x_l[1][qw * 32 + lq], m_run, l_run);
+        }
+        // A row without a visible key: max = -inf, every exp(-inf - -inf) is NaN, as in the reference's softmax.
+        const float inv_l = 1.0f / l_run;
+
+        // ---- pass 2: weights out, product with V
+        float16_t oacc[DBLK];
+#pragma unroll
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+        std::uint16_t* arow = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + qrow) * p.Lk;
+        const bool row_live = my_q < p.Lq;
+        const bool wide = (p.Lk % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.attn) & 7) == 0);   // 8-byte runs of four weights
+        fetch(kbase, p.ks_l, 0, kreg);
+        fetch(vbase, p.vs_l, 0, vreg);
+        put(kreg, k_buf(0), false);            // (pass 1 ended with barriers: nobody reads stage 0 any more)
+        put(vreg, v_buf(0), true);
+        __syncthreads();
+        for (int t = 0; t < n_tiles; ++t) {
+            const std::uint16_t* k_lds = k_buf(t & 1);
+            const std::uint16_t* v_lds = v_buf(t & 1);
+            if (t + 1 < n_tiles) {
+                fetch(kbase, p.ks_l, (t + 1) * kTile, kreg);
+                fetch(vbase, p.vs_l, (t + 1) * kTile, vreg);
+            }
+#pragma unroll
+            for (int jb = 0; jb < 2; ++jb) {
+                const int key0 = t * kTile + kg * kBN + jb * 32;
+                if (key0 >= p.Lk) continue;
+                const bool skipped = kMode == 3 && key0 > q0 + 31;   // wave-uniform: this wave's queries see none of these keys
+                float16_t sc;
+                std::uint32_t pw[8];
+                if (!skipped) {
+                    scores(k_lds, jb, key0, sc);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const float w0 = __expf(sc[2 * i] - m_run) * inv_l, w1 = __expf(sc[2 * i + 1] - m_run) * inv_l;
+                        pw[i] = static_cast<std::uint32_t>(El::from_f32(w0)) | (static_cast<std::uint32_t>(El::from_f32(w1)) << 16);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) pw[i] = 0u;
+                }
+                if (row_live) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int key = key0 + g * 8 + 4 * lh;
+                        if (wide && key + 3 < p.Lk) {
+                            *reinterpret_cast<u32x2*>(arow + key) = u32x2{pw[2 * g], pw[2 * g + 1]};
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (key + e < p.Lk) arow[key + e] = static_cast<std::uint16_t>(pw[2 * g + (e >> 1)] >> (16 * (e & 1)));
+                        }
+                    }
+                }
+                if (!skipped) {
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        const u32x4 pv = {pw[4 * s2], pw[4 * s2 + 1], pw[4 * s2 + 2], pw[4 * s2 + 3]};
+#pragma unroll
+                        for (int db = 0; db < DBLK; ++db) {
+                            const std::uint16_t* vp = v_lds + jb * 32 * D + v_rd[db] + 16 * s2 * D;
+                            const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+                            const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
+                            const i16x8 vf = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                            oacc[db] = Mma16<T>::run(vf, __builtin_bit_cast(i16x8, pv), oacc[db]);
+                        }
+                    }
+                }
+            }
+            if (t + 1 < n_tiles) {
+                put(kreg, k_buf((t + 1) & 1), false);
+                put(vreg, v_buf((t + 1) & 1), true);
+            }
+            __syncthreads();
+        }
+        // causal: the keys past the workgroup's last query were never visited; their weights are zero.
+        // The two waves of a query group clear that part of alternate rows, a row at a time with
+        // 16-byte stores where the row starts allow it.
+        if (kMode == 3 && n_tiles * kTile < p.Lk) {
+            const int first = n_tiles * kTile;
+            const bool rows16 = (p.Lk % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.attn) & 15) == 0);
+            for (int rr = kg; rr < 32; rr += 2) {
+                const int row = q0 + rr;
+                if (row >= p.Lq) break;
+                std::uint16_t* zr = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + row) * p.Lk;
+                if (rows16) {
+                    for (int key = first + lane * 8; key < p.Lk; key += 64 * 8) store16(zr + key, u32x4{0u, 0u, 0u, 0u});
+                } else {
+                    for (int key = first + lane; key < p.Lk; key += 64) zr[key] = 0;
+                }
+            }
+        }
+
+        // The two key groups' partial products add up: group 1 hands its over through LDS (the tile
+        // buffers are free after the last tile's barrier), element (db, r) of lane l of query group qw
+        // at [(db*16 + r)][qw*64 + l].
+        float* xo = reinterpret_cast<float*>(tiles);
+        if (kg == 1) {
+#pragma unroll
+            for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) xo[(db * 16 + r) * 256 + qw * 64 + lane] = oacc[db][r];
+        }
+        __syncthreads();
+        if (kg == 0) {
+#pragma unroll
+            for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] += xo[(db * 16 + r) * 256 + qw * 64 + lane];
             if (row_live) {
+                std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int key = key0 + g * 8 + 4 * lh;
-                    if (wide && key + 3 < p.Lk) {
-                        *reinterpret_cast<u32x2*>(arow + key) = u32x2{pw[2 * g], pw[2 * g + 1]};
-                    } else {
+                for (int db = 0; db < DBLK; ++db)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (key + e < p.Lk) arow[key + e] = static_cast<std::uint16_t>(pw[2 * g + (e >> 1)] >> (16 * (e & 1)));
+                    for (int g = 0; g < 4; ++g) {
+                        const int d = db * 32 + g * 8 + 4 * lh;
+                        u32x2 w;
+                        w[0] = static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 0])) | (static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 1])) << 16);
+                        w[1] = static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 2])) | (static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 3])) << 16);
+                        *reinterpret_cast<u32x2*>(op + d) = w;
                     }
-                }
-            }
-            if (!skipped) {
-#pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
-                    const u32x4 pv = {pw[4 * s2], pw[4 * s2 + 1], pw[4 * s2 + 2], pw[4 * s2 + 3]};
-#pragma unroll
-                    for (int db = 0; db < DBLK; ++db) {
-                        const std::uint16_t* vp = v_lds + jb * 32 * D + v_rd[db] + 16 * s2 * D;
-                        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
-                        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
-                        const i16x8 vf = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        oacc[db] = Mma16<T>::run(vf, __builtin_bit_cast(i16x8, pv), oacc[db]);
-                    }
-                }
+                if (p.lse != nullptr && lh == 0)
+                    p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run + logf(l_run);
             }
         }
-        __syncthreads();
-    }
-    // causal: the keys past the workgroup's last query were never visited; their weights are zero.
-    // Each wave clears that part of its 32 rows, a row at a time with 16-byte stores where the
-    // row starts allow it.
-    if (kMode == 3 && n_tiles * kBN < p.Lk) {
-        const int first = n_tiles * kBN;
-        const bool rows16 = (p.Lk % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.attn) & 15) == 0);
-        for (int rr = 0; rr < 32; ++rr) {
-            const int row = q0 + rr;
-            if (row >= p.Lq) break;
-            std::uint16_t* zr = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + row) * p.Lk;
-            if (rows16) {
-                for (int key = first + lane * 8; key < p.Lk; key += 64 * 8) store16(zr + key, u32x4{0u, 0u, 0u, 0u});
-            } else {
-                for (int key = first + lane; key < p.Lk; key += 64) zr[key] = 0;
-            }
-        }
-    }
-
-    if (row_live) {
-        std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
-#pragma unroll
-        for (int db = 0; db < DBLK; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int d = db * 32 + g * 8 + 4 * lh;
-                u32x2 w;
-                w[0] = static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 0])) | (static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 1])) << 16);
-                w[1] = static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 2])) | (static_cast<std::uint32_t>(El::from_f32(oacc[db][4 * g + 3])) << 16);
-                *reinterpret_cast<u32x2*>(op + d) = w;
-            }
-        if (p.lse != nullptr && lh == 0)
-            p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run + logf(l_run);
-    }
+    }   // part
 }
 
 template <typename T, int D>
 int launch_t(WeightsParams p, int mode, hipStream_t s) {
     p.n_qblocks = (p.Lq + kBM - 1) / kBM;
-    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
-    const dim3 grid(static_cast<unsigned>(blocks)), wg(256);
+    const long per_bh = mode == 3 ? (p.n_qblocks + 1) / 2 : p.n_qblocks;      // causal: query blocks in pairs
+    const long blocks = static_cast<long>(p.B) * p.Hq * per_bh;
+    const dim3 grid(static_cast<unsigned>(blocks)), wg(512);
+    constexpr unsigned kLdsBytes = 4u * kTile * D * 2u;     // K and V, two stages each
+    // More than 64 KB of LDS has to be asked for by name, once per kernel.
+    auto allow = [&](const void* fn) {
+        static std::mutex mu;
+        static std::set<const void*> done;
+        std::lock_guard<std::mutex> g(mu);
+        if (done.count(fn)) return hipSuccess;
+        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes));
+        if (e == hipSuccess) done.insert(fn);
+        return e;
+    };
     switch (mode) {
-        case 0: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 0>), grid, wg, 0, s, p); break;
-        case 1: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 1>), grid, wg, 0, s, p); break;
-        case 2: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 2>), grid, wg, 0, s, p); break;
-        default: hipLaunchKernelGGL((weights_fwd_kernel<T, D, 3>), grid, wg, 0, s, p); break;
+        case 0:
+            PARAS_HIP_TRY(allow(reinterpret_cast<const void*>(&weights_fwd_kernel<T, D, 0>)));
+            hipLaunchKernelGGL((weights_fwd_kernel<T, D, 0>), grid, wg, kLdsBytes, s, p);
+            break;
+        case 1:
+            PARAS_HIP_TRY(allow(reinterpret_cast<const void*>(&weights_fwd_kernel<T, D, 1>)));
+            hipLaunchKernelGGL((weights_fwd_kernel<T, D, 1>), grid, wg, kLdsBytes, s, p);
+            break;
+        case 2:
+            PARAS_HIP_TRY(allow(reinterpret_cast<const void*>(&weights_fwd_kernel<T, D, 2>)));
+            hipLaunchKernelGGL((weights_fwd_kernel<T, D, 2>), grid, wg, kLdsBytes, s, p);
+            break;
+        default:
+            PARAS_HIP_TRY(allow(reinterpret_cast<const void*>(&weights_fwd_kernel<T, D, 3>)));
+            hipLaunchKernelGGL((weights_fwd_kernel<T, D, 3>), grid, wg, kLdsBytes, s, p);
+            break;
     }
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
@@ -366,6 +475,7 @@ int launch_weights(const paras_sdpa_args& a, hipStream_t s) {
     p.Lq = static_cast<int>(a.Lq); p.Lk = static_cast<int>(a.Lk);
     p.n_qblocks = 0;
     p.scale = a.scale;
+    p.scale_is_f32 = static_cast<double>(static_cast<float>(a.scale)) == a.scale ? 1 : 0;
     p.mask = static_cast<const unsigned char*>(a.mask);
     p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2];
     const int mode = a.is_causal ? 3 : a.mask_kind;
