@@ -40,6 +40,7 @@ namespace {
 
 constexpr int kBN = 64;    // keys per key group and tile
 constexpr int kTile = 128; // keys per staged tile: two key groups
+constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kBM = 128;   // queries per workgroup: 4 waves x 32
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -237,10 +238,12 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
                 for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
                 const float m_new = fmaxf(m_run, mx);
                 if (m_new != -INFINITY) {
+                    // exp(s - m) as 2^(s log2(e) - m log2(e)): one fused multiply-add and the exponential
+                    const float shift = -m_new * kLog2e;
                     float add = 0.f;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) add += __expf(sc[r] - m_new);
-                    l_run = (m_run == -INFINITY ? 0.f : l_run * __expf(m_run - m_new)) + add;
+                    for (int r = 0; r < 16; ++r) add += __builtin_amdgcn_exp2f(fmaf(sc[r], kLog2e, shift));
+                    l_run = (m_run == -INFINITY ? 0.f : l_run * __builtin_amdgcn_exp2f(fmaf(m_run, kLog2e, shift))) + add;
                     m_run = m_new;
                 }
             }
@@ -273,6 +276,7 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
         }
         // A row without a visible key: max = -inf, every exp(-inf - -inf) is NaN, as in the reference's softmax.
         const float inv_l = 1.0f / l_run;
+        const float w_shift = -m_run * kLog2e;
 
         // ---- pass 2: weights out, product with V
         float16_t oacc[DBLK];
@@ -304,10 +308,23 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
                 std::uint32_t pw[8];
                 if (!skipped) {
                     scores(k_lds, jb, key0, sc);
+                    // The weights are narrowed by the conversion instructions; a NaN among them (a row
+                    // without a visible key, a NaN or an infinity in the inputs) shows in their sum, and
+                    // then the block is narrowed again the way the host writes NaNs.
+                    float w[16], total = 0.f;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        const float w0 = __expf(sc[2 * i] - m_run) * inv_l, w1 = __expf(sc[2 * i + 1] - m_run) * inv_l;
-                        pw[i] = static_cast<std::uint32_t>(El::from_f32(w0)) | (static_cast<std::uint32_t>(El::from_f32(w1)) << 16);
+                    for (int r = 0; r < 16; ++r) {
+                        w[r] = __builtin_amdgcn_exp2f(fmaf(sc[r], kLog2e, w_shift)) * inv_l;
+                        total += w[r];
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        pw[i] = static_cast<std::uint32_t>(El::from_f32_finite(w[2 * i])) | (static_cast<std::uint32_t>(El::from_f32_finite(w[2 * i + 1])) << 16);
+                    if (__builtin_amdgcn_ballot_w64(!(total == total)) != 0) {
+                        asm volatile("" ::: "memory");
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            pw[i] = static_cast<std::uint32_t>(El::from_f32(w[2 * i])) | (static_cast<std::uint32_t>(El::from_f32(w[2 * i + 1])) << 16);
                     }
                 } else {
 #pragma unroll
