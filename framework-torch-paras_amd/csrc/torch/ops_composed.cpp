@@ -26,14 +26,19 @@ Tensor rms_norm(const Tensor& input, c10::IntArrayRef normalized_shape, const c1
     if (has_w)
         TORCH_CHECK(weight->sizes().equals(normalized_shape), "paras rms_norm: weight shape must equal normalized_shape");
     Tensor in = input.contiguous();
+    // A weight of another dtype: the reference's last step is `out * weight`, which promotes
+    // (csrc/ops/rms_swiglu_ops.cpp:70-72), so the normalised tensor is formed in the input's dtype
+    // and the product taken by the device's multiply in the promoted one.
+    const bool fused_w = has_w && weight->scalar_type() == in.scalar_type();
     Tensor w;
-    if (has_w) w = weight->to(in.scalar_type()).contiguous();
+    if (fused_w) w = weight->contiguous();
     Tensor out = at::empty_like(in);
     const int64_t rows = H > 0 ? in.numel() / H : 0;
-    if (rows == 0 || H == 0) return out;
-    check(paras_rms_norm_composed_fwd(in.data_ptr(), has_w ? w.data_ptr() : nullptr, out.data_ptr(), rows, H,
-                                      eps.has_value() ? *eps : 1e-6, require_float_code(in, "paras rms_norm"),
-                                      stream_for(in)));
+    if (rows > 0 && H > 0)
+        check(paras_rms_norm_composed_fwd(in.data_ptr(), fused_w ? w.data_ptr() : nullptr, out.data_ptr(), rows, H,
+                                          eps.has_value() ? *eps : 1e-6, require_float_code(in, "paras rms_norm"),
+                                          stream_for(in)));
+    if (has_w && !fused_w) return at::mul(out, *weight);
     return out;
 }
 

@@ -226,6 +226,12 @@ def test_composed_ops_narrow_like_the_host_engine(device):
         u = torch.randn(33, 70).to(dt)
         got = torch.ops.torch_paras.swiglu(u.to(device), g.to(device))
         assert_bit_exact(got.cpu(), O.swiglu_composed(u, g), f"torch_paras::swiglu {dt}")
+    # a weight of another dtype promotes the result, as the reference's final `out * weight` does
+    x, w = torch.randn(9, 64).bfloat16(), 1 + 0.02 * torch.randn(64)
+    got = torch.ops.aten.rms_norm(x.to(device), [64], w.to(device), 1e-5)
+    assert got.dtype == torch.float32
+    want = O.binary(O.OP_MUL, O.rms_norm_composed(x, [64], None, 1e-5).float(), w.expand(9, 64).contiguous())
+    assert_bit_exact(got.cpu(), want, "aten::rms_norm bf16 input, fp32 weight")
 
 
 def test_composed_ops_streaming_kernels_are_exact(device):
