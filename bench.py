@@ -111,7 +111,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "sdpa_prefill", "rmsnorm_swiglu", "sdpa_decode", "moe", "linear", "backward_ops", "copy"],
+                    choices=["all", "sdpa_prefill", "sdpa_weights", "rmsnorm_swiglu", "sdpa_decode", "moe", "linear", "backward_ops", "copy"],
                     help="'copy' is the counter calibration: a plain 1 GiB device copy, not part of 'all'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg (baseline timing and parity check)")
     args = ap.parse_args()
@@ -192,6 +192,44 @@ def main() -> int:
                     "slice": "queries 0..255 of heads (0,0) and (3,31), queries 4032..4095 of head (1,7)"}
         checks["sdpa_prefill"] = check_prefill
         del q, k, v, out
+
+    # ------------------------------------------------------------------ the math op with its weights returned
+    if want("sdpa_weights"):
+        torch.manual_seed(0)
+        B, H, S, D = 2, 16, 2048, 128
+        qc, kc, vc = draw(B, H, S, D), draw(B, H, S, D), draw(B, H, S, D)
+        q, k, v = qc.to(dev), kc.to(dev), vc.to(dev)
+        out = torch.empty_like(q)
+        attn = torch.empty(B, H, S, S, dtype=bf, device=dev)
+        scale = float(torch.tensor(D ** -0.5).to(bf))          # narrowed to the tensors' dtype, as the op layer passes it
+        a = capi.sdpa_args(q, k, v, out, attn=attn, is_causal=True, scale=scale)
+        assert L.paras_sdpa_kernel_name(C.byref(a)) == b"math_mfma"
+        ms, wall = timer.run(lambda i: must(L.paras_sdpa_fwd(C.byref(a), None, st)), steps, warmup, SETTLE_MFMA_MS)
+        nbytes = attn.numel() * 2 + 4 * q.numel() * 2          # the weights written, q / k / v read, out written
+        gbs = nbytes / ms / 1e6
+        flops = 4 * B * H * S * S * D / 2
+        results["sdpa_weights"] = {
+            "workload": "bf16 causal SDPA with the attention weights returned (the math op) B=2 H=16 S=2048 D=128",
+            "value": round(gbs, 1), "unit": "GB/s", "ms_per_step": round(ms, 4), "tflops_causal_halved": round(flops / ms / 1e9, 1),
+            "kernel": "weights_fwd_kernel<bf16,128,causal>", "algorithmic_bytes_per_launch": nbytes,
+            "roofline": roofline("hbm", gbs, "weights_fwd_kernel"),
+        }
+        log(f"sdpa_weights: {ms * 1e3:.1f} us  {gbs:.0f} GB/s ({gbs / HBM_PEAK_GBS:.1%})  {flops / ms / 1e9:.0f} TFLOP/s (causal-halved count)")
+        w_got, o_got = attn[1, 5, :192, :192].cpu(), out[1, 5, :192].cpu()
+
+        def check_weights(O, qc=qc, kc=kc, vc=vc, w_got=w_got, o_got=o_got, scale=scale):
+            # a causal query sees its prefix only: the first 192 queries of a head stand alone
+            ref_o, ref_w = O.sdpa_math(qc[1:2, 5:6, :192], kc[1:2, 5:6, :192], vc[1:2, 5:6, :192], is_causal=True, scale=scale, gemm="aten")
+            diff = w_got.view(torch.int16).int() - ref_w[0, 0].view(torch.int16).int()
+            off_by_more = int((diff.abs() > 1).sum())
+            differing = int((diff != 0).sum())
+            err_o = (o_got.float() - ref_o[0, 0].float()).abs().max().item()
+            n = w_got.numel()
+            return {"weights_differing": differing, "weights_off_by_more_than_one_ulp": off_by_more, "elements": n, "out_max_abs_err": err_o,
+                    "tolerance": "weights: at most 5e-3 of the elements differ, 5e-4 by more than one ulp; out 2e-2",
+                    "ok": differing <= 5e-3 * n and off_by_more <= 5e-4 * n and err_o <= 2e-2, "slice": "queries and keys 0..191 of head (1,5)"}
+        checks["sdpa_weights"] = check_weights
+        del q, k, v, out, attn
 
     # ------------------------------------------------------------------ configs[1]
     if want("rmsnorm_swiglu"):
@@ -509,6 +547,8 @@ def main() -> int:
 CPU_SAMPLES = {
     "sdpa_prefill": ({"B": 4, "H": 32, "S": 4096, "D": 128}, lambda s: 4 * s["B"] * s["H"] * s["S"] ** 2 * s["D"] / 2 / 1e12, "TFLOP/s",
                      "the whole workload once: B=4, H=32, S=4096, D=128"),
+    "sdpa_weights": ({"B": 1, "H": 2, "S": 2048, "D": 128}, lambda s: (s["B"] * s["H"] * s["S"] ** 2 * 2 + 4 * s["B"] * s["H"] * s["S"] * s["D"] * 2) / 1e9, "GB/s",
+                     "2 of the 32 heads (1/16 of the workload)"),
     "rmsnorm_swiglu": ({"rows": 16384, "H": 4096, "I": 14336}, lambda s: (2 * s["rows"] * s["H"] * 2 + 3 * s["rows"] * s["I"] * 2) / 1e9, "GB/s",
                        "the whole workload once: 16384 rows"),
     "sdpa_decode": ({"B": 32, "Hq": 32, "Hkv": 8, "Lk": 8192, "D": 128}, lambda s: 2 * s["B"] * s["Hkv"] * s["Lk"] * s["D"] * 2 / 1e9, "GB/s",

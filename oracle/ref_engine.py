@@ -194,6 +194,16 @@ def time_workload(name: str, sample: dict) -> dict:
         out = torch.ops.aten._scaled_dot_product_attention_math(dq, dk, dv, None, 0.0, True, None, scale=None, enable_gqa=False)[0]
         out.cpu()
         return {"seconds": time.perf_counter() - t0}
+    if name == "sdpa_weights":
+        B, H, S, D = sample["B"], sample["H"], sample["S"], sample["D"]
+        q, k, v = (torch.randn(B, H, S, D).to(bf) for _ in range(3))
+        sdpa_math(q[:, :1, :64], k[:, :1, :64], v[:, :1, :64], is_causal=True)
+        dq, dk, dv = _dev(q), _dev(k), _dev(v)
+        t0 = time.perf_counter()
+        out, attn = torch.ops.aten._scaled_dot_product_attention_math(dq, dk, dv, None, 0.0, True, None, scale=None, enable_gqa=False)
+        out.cpu()
+        attn.cpu()
+        return {"seconds": time.perf_counter() - t0}
     if name == "rmsnorm_swiglu":
         rows, H, I = sample["rows"], sample["H"], sample["I"]
         x, w = torch.randn(rows, H).to(bf), (1 + 0.02 * torch.randn(H)).to(bf)
