@@ -11,8 +11,8 @@
 //            exact for every float dtype; indices are int64.
 //
 // Rows of up to 256 elements: one wave per row, the row in registers.  Longer rows: one
-// workgroup per row, re-read from L2 between passes (these ops sit on router logits and
-// attention rows: thousands of elements, not millions).
+// workgroup per row; the softmax re-reads it from L2 between passes, the top-k keeps one
+// candidate per thread and refreshes only the one that was taken (fp64 rows: a pass per slot).
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -193,6 +193,171 @@ __global__ __launch_bounds__(kBlock) void topk_rows_kernel(const typename Elem<T
     }
 }
 
+// ---- long rows of bf16 / fp16 / fp32 (vocabulary-sized logits, k a few dozen): the same result
+// without a pass over the row per slot.  An element becomes one 64-bit key, its value made
+// monotone in the upper half and 2^32 - 1 - index in the lower, so that "comes before" in the
+// reference's (value, index) order is "has the larger key" and "strictly after the previous slot"
+// is "key below the previous slot's key"; NaNs get key 0 = no element, -0 is keyed as +0 (the
+// reference compares them equal and lets the index decide).  Thread t owns the 16-byte groups of
+// elements t, t + kThreads, ... and keeps the best key of them that is still below the bound.
+// A slot is then: the best of the wavefronts' bests (LDS), and only the thread that owned it looks
+// for its next candidate -- its wavefront does that together, a group per lane.  When nothing is
+// left (NaNs, or k beyond the eligible elements) the reference reports (0, -1) and carries on from
+// there, i.e. with the bound at (value 0, index -1): every thread scans again.
+typedef unsigned long long u64;
+
+template <typename T>
+__device__ __forceinline__ u64 topk_key(typename Elem<T>::store_t raw, long j, bool largest) {
+    const float f = Elem<T>::to_f32(raw);
+    if (f != f) return 0ull;
+    std::uint32_t u = __builtin_bit_cast(std::uint32_t, f);
+    if ((u << 1) == 0u) u = 0u;                                    // -0 -> +0
+    std::uint32_t mono = (u >> 31) ? ~u : (u | 0x80000000u);
+    if (!largest) mono = ~mono;
+    return (static_cast<u64>(mono) << 32) | static_cast<u64>(0xFFFFFFFFu - static_cast<std::uint32_t>(j));
+}
+
+// Maximum of a 64-bit key over the wave, in every lane, without the LDS crossbar: four DPP
+// exchanges inside each row of 16 lanes, then the four row maxima through v_readlane.
+template <int kCtrl>
+__device__ __forceinline__ u64 dpp_move_u64(u64 v) {
+    const int lo = static_cast<int>(v), hi = static_cast<int>(v >> 32);
+    const int lo2 = __builtin_amdgcn_update_dpp(lo, lo, kCtrl, 0xf, 0xf, false);
+    const int hi2 = __builtin_amdgcn_update_dpp(hi, hi, kCtrl, 0xf, 0xf, false);
+    return (static_cast<u64>(static_cast<std::uint32_t>(hi2)) << 32) | static_cast<std::uint32_t>(lo2);
+}
+__device__ __forceinline__ u64 readlane_u64(u64 v, int lane) {
+    const std::uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(v), lane);
+    const std::uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(v >> 32), lane);
+    return (static_cast<u64>(hi) << 32) | lo;
+}
+__device__ __forceinline__ u64 wave_max_u64(u64 v) {
+    auto mx = [](u64 a, u64 b) { return a > b ? a : b; };
+    v = mx(v, dpp_move_u64<0xB1>(v));    // quad_perm [1,0,3,2]: lane ^ 1
+    v = mx(v, dpp_move_u64<0x4E>(v));    // quad_perm [2,3,0,1]: lane ^ 2
+    v = mx(v, dpp_move_u64<0x141>(v));   // row_half_mirror
+    v = mx(v, dpp_move_u64<0x140>(v));   // row_mirror
+    return mx(mx(readlane_u64(v, 0), readlane_u64(v, 16)), mx(readlane_u64(v, 32), readlane_u64(v, 48)));
+}
+
+template <typename T, int kThreads>
+__global__ __launch_bounds__(kThreads) void topk_rows_select_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                                    typename Elem<T>::store_t* __restrict__ values,
+                                                                    long* __restrict__ indices, long n, long k, int largest_i) {
+    using E = Elem<T>;
+    using S = typename E::store_t;
+    constexpr int kNW = kThreads / kWave;
+    __shared__ u64 wbest[kNW];
+    const bool largest = largest_i != 0;
+    const S* xr = x + static_cast<long>(blockIdx.x) * n;
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    constexpr int GE = 16 / static_cast<int>(sizeof(S));          // elements per 16-byte group
+    const long ngroups = (n + GE - 1) / GE;
+    // rows that start on a 16-byte boundary and are whole groups long: one load per group
+    const bool wide = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && n % GE == 0;
+
+    // best key below `bound` among the elements of group g
+    auto group_best = [&](long g, u64 bound) -> u64 {
+        u64 best = 0ull;
+        const long j0 = g * GE;
+        if (wide) {
+            const u32x4 v = load16(xr + j0);
+            const S* e = reinterpret_cast<const S*>(&v);
+#pragma unroll
+            for (int i = 0; i < GE; ++i) {
+                const u64 key = topk_key<T>(e[i], j0 + i, largest);
+                if (key < bound && key > best) best = key;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < GE; ++i) {
+                const long j = j0 + i;
+                if (j < n) {
+                    const u64 key = topk_key<T>(xr[j], j, largest);
+                    if (key < bound && key > best) best = key;
+                }
+            }
+        }
+        return best;
+    };
+    auto scan_own = [&](u64 bound) -> u64 {
+        u64 best = 0ull;
+        for (long g = tid; g < ngroups; g += kThreads) {
+            const u64 b = group_best(g, bound);
+            best = b > best ? b : best;
+        }
+        return best;
+    };
+    // the bound "after (value 0, index -1)": every element whose value key does not exceed that of 0
+    const u64 zero_bound = ((topk_key<T>(static_cast<S>(0), 0, largest) >> 32) + 1ull) << 32;
+
+    const bool first_is_nan = n > 0 && E::to_f64(xr[0]) != E::to_f64(xr[0]);
+    u64 bound = ~0ull, mine = 0ull;
+    bool rescan_all = true;
+    for (long s = 0; s < k; ++s) {
+        S* vout = values + static_cast<long>(blockIdx.x) * k + s;
+        long* iout = indices + static_cast<long>(blockIdx.x) * k + s;
+        if (first_is_nan && s < 2) {
+            // a NaN first element is slot 0; nothing comes "after" a NaN, so slot 1 is (0, -1)
+            if (tid == 0) {
+                *vout = s == 0 ? E::from_f64(E::to_f64(xr[0])) : E::from_f64(0.0);
+                *iout = s == 0 ? 0 : -1;
+            }
+            bound = zero_bound;
+            rescan_all = true;
+            continue;
+        }
+        if (rescan_all) {
+            mine = scan_own(bound);
+            const u64 wb = wave_max_u64(mine);
+            if (lane == 0) wbest[wave] = wb;
+            rescan_all = false;
+        }
+        __syncthreads();
+        u64 best = 0ull;
+        int best_wave = 0;
+#pragma unroll
+        for (int w = 0; w < kNW; ++w) {
+            const u64 c = wbest[w];
+            if (c > best) {
+                best = c;
+                best_wave = w;
+            }
+        }
+        __syncthreads();                                   // everyone has read the wavefronts' bests
+        if (best == 0ull) {                                // nothing eligible: (0, -1), go on from there
+            if (tid == 0) {
+                *vout = E::from_f64(0.0);
+                *iout = -1;
+            }
+            bound = zero_bound;
+            rescan_all = true;
+            continue;
+        }
+        const long idx = static_cast<long>(0xFFFFFFFFu - static_cast<std::uint32_t>(best));
+        if (tid == 0) {
+            *vout = xr[idx];
+            *iout = idx;
+        }
+        bound = best;
+        if (wave == best_wave) {
+            // the lane whose candidate was taken gets its next one: its groups, a group per lane
+            const u64 owners = __ballot(mine == best);
+            const int owner_lane = __ffsll(static_cast<long long>(owners)) - 1;
+            const long owner_tid = static_cast<long>(wave) * kWave + owner_lane;
+            u64 next = 0ull;
+            for (long g = owner_tid + static_cast<long>(lane) * kThreads; g < ngroups; g += static_cast<long>(kWave) * kThreads) {
+                const u64 b = group_best(g, bound);
+                next = b > next ? b : next;
+            }
+            next = wave_max_u64(next);
+            if (lane == owner_lane) mine = next;
+            const u64 wb = wave_max_u64(mine);
+            if (lane == 0) wbest[wave] = wb;
+        }
+    }
+}
+
 // ---- short rows (n <= 64 * EPL): one wave per row, four rows per workgroup, the row in
 // registers (lane l holds elements l, l + 64, ...), no LDS and no barrier.  Router logits and
 // other rows of a few dozen elements would otherwise leave most of a 256-thread workgroup idle.
@@ -288,6 +453,68 @@ __global__ __launch_bounds__(kBlock) void topk_rows_wave_kernel(const typename E
     }
 }
 
+// Short rows of bf16 / fp16 / fp32 with the same keys: a lane holds the keys of its elements, a
+// slot is a wave maximum, and the lane that held it writes the element out and retires the key.
+template <typename T, int EPL>
+__global__ __launch_bounds__(kBlock) void topk_rows_wave_keys_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                                     typename Elem<T>::store_t* __restrict__ values,
+                                                                     long* __restrict__ indices, long rows, int n, int k, int largest_i) {
+    using E = Elem<T>;
+    using S = typename E::store_t;
+    const bool largest = largest_i != 0;
+    const int lane = threadIdx.x % kWave;
+    const long row = static_cast<long>(blockIdx.x) * kWaves + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const S* xr = x + row * n;
+    S raw[EPL];
+    u64 orig[EPL], live[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int j = lane + i * kWave;
+        raw[i] = j < n ? xr[j] : static_cast<S>(0);
+        orig[i] = j < n ? topk_key<T>(raw[i], j, largest) : 0ull;
+        live[i] = orig[i];
+    }
+    const u64 zero_bound = ((topk_key<T>(static_cast<S>(0), 0, largest) >> 32) + 1ull) << 32;
+    auto restart = [&]() {                       // go on from (value 0, index -1): everything not above zero is eligible again
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) live[i] = orig[i] < zero_bound ? orig[i] : 0ull;
+    };
+    const S x0 = xr[0];
+    const bool first_is_nan = E::to_f64(x0) != E::to_f64(x0);
+    S* vout = values + row * k;
+    long* iout = indices + row * k;
+    for (int s = 0; s < k; ++s) {
+        if (first_is_nan && s < 2) {
+            if (lane == 0) {
+                vout[s] = s == 0 ? E::from_f64(E::to_f64(x0)) : E::from_f64(0.0);
+                iout[s] = s == 0 ? 0 : -1;
+            }
+            restart();
+            continue;
+        }
+        u64 m = live[0];
+#pragma unroll
+        for (int i = 1; i < EPL; ++i) m = live[i] > m ? live[i] : m;
+        const u64 best = wave_max_u64(m);
+        if (best == 0ull) {
+            if (lane == 0) {
+                vout[s] = E::from_f64(0.0);
+                iout[s] = -1;
+            }
+            restart();
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < EPL; ++i)
+            if (live[i] == best) {
+                vout[s] = raw[i];
+                iout[s] = lane + i * kWave;
+                live[i] = 0ull;
+            }
+    }
+}
+
 template <typename TI>
 int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, hipStream_t s) {
     using SI = typename Elem<TI>::store_t;
@@ -332,12 +559,29 @@ int launch_topk(const void* x, void* values, long* indices, long rows, long n, l
     using S = typename Elem<T>::store_t;
     if (n <= 4 * kWave) {
         const dim3 gw(static_cast<unsigned>((rows + kWaves - 1) / kWaves)), b(kBlock);
-        if (n <= kWave)
+        if constexpr (sizeof(S) <= 4) {
+            if (n <= kWave)
+                hipLaunchKernelGGL((topk_rows_wave_keys_kernel<T, 1>), gw, b, 0, s, static_cast<const S*>(x), static_cast<S*>(values), indices, rows, (int)n, (int)k, largest);
+            else
+                hipLaunchKernelGGL((topk_rows_wave_keys_kernel<T, 4>), gw, b, 0, s, static_cast<const S*>(x), static_cast<S*>(values), indices, rows, (int)n, (int)k, largest);
+        } else if (n <= kWave)
             hipLaunchKernelGGL((topk_rows_wave_kernel<T, 1>), gw, b, 0, s, static_cast<const S*>(x), static_cast<S*>(values), indices, rows, (int)n, (int)k, largest);
         else
             hipLaunchKernelGGL((topk_rows_wave_kernel<T, 4>), gw, b, 0, s, static_cast<const S*>(x), static_cast<S*>(values), indices, rows, (int)n, (int)k, largest);
         PARAS_HIP_TRY(hipGetLastError());
         return PARAS_OK;
+    }
+    if constexpr (sizeof(S) <= 4) {
+        if (n < (1LL << 32)) {
+            if (n <= 8192)
+                hipLaunchKernelGGL((topk_rows_select_kernel<T, 256>), dim3(static_cast<unsigned>(rows)), dim3(256), 0, s, static_cast<const S*>(x),
+                                   static_cast<S*>(values), indices, n, k, largest);
+            else
+                hipLaunchKernelGGL((topk_rows_select_kernel<T, 1024>), dim3(static_cast<unsigned>(rows)), dim3(1024), 0, s, static_cast<const S*>(x),
+                                   static_cast<S*>(values), indices, n, k, largest);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
     }
     hipLaunchKernelGGL((topk_rows_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(kBlock), 0, s, static_cast<const S*>(x),
                        static_cast<S*>(values), indices, n, k, largest);

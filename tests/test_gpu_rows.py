@@ -111,3 +111,37 @@ def test_topk_rows_with_nans_follow_the_host_scan(dtype, n):
                 assert_bit_exact(gv, wv, f"topk values {dtype} n={n} k={k} largest={largest}")
             else:
                 assert torch.equal(gv.cpu().isnan(), wv.isnan()) and torch.equal(gv.cpu().nan_to_num(7.0), wv.nan_to_num(7.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("largest", [True, False])
+def test_topk_long_rows_keep_one_candidate_per_thread(dtype, largest):
+    """Vocabulary-sized rows run on the kernel that keeps one candidate per thread and refreshes only
+    the one that was taken: quantised values (thousands of ties, signed zeros), k up to a few
+    hundred, rows with NaNs, and rows with fewer eligible elements than k, where the host reports
+    (0, -1) and goes on from there."""
+    torch.manual_seed(91)
+    for (rows, n), k in (((3, 9000), 50), ((2, 20000), 300), ((1, 128256), 50), ((4, 300), 300), ((2, 8192), 64), ((2, 8200), 7)):
+        x = ((torch.randn(rows, n) * 4).round() / 4).to(dtype)
+        x[0, 17] = -0.0
+        x[0, 3] = 0.0
+        if rows > 1:
+            x[1, 5::3] = float("nan")
+            x[1, 1] = float("inf")
+        gv, gi = capi.topk_rows(x.cuda(), k, largest)
+        wv, wi = O.topk_last(x, k, largest)
+        assert_bit_exact(gi, wi, f"topk indices {(rows, n)} k={k}")
+        assert_bit_exact(gv, wv, f"topk values {(rows, n)} k={k}")
+    # fewer eligible elements than k; a NaN first; everything NaN but the first
+    x = torch.randn(5, 600).to(dtype)
+    x[0, 10:] = float("nan")
+    x[1, 0] = float("nan")
+    x[2, 1:] = float("nan")
+    x[3, :] = float("nan")
+    x[4, ::2] = float("nan")
+    x[4, 1] = 0.0
+    for k in (5, 40, 600):
+        gv, gi = capi.topk_rows(x.cuda(), k, largest)
+        wv, wi = O.topk_last(x, k, largest)
+        assert_bit_exact(gi, wi, f"topk indices with few eligible elements k={k}")
+        assert torch.equal(gv.cpu().isnan(), wv.isnan()) and torch.equal(gv.cpu().nan_to_num(7.0), wv.nan_to_num(7.0))
