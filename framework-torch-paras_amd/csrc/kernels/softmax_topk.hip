@@ -34,18 +34,22 @@ __device__ __forceinline__ double wave_max_f64(double v) {
     return v;
 }
 
-template <typename TI, typename TO>
-__global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const typename Elem<TI>::store_t* __restrict__ x,
-                                                              typename Elem<TO>::store_t* __restrict__ out, long n) {
+// Any row length: three passes over the row (it stays in L2), kThreads threads per row -- 1024 for
+// the long rows of which there are few (vocabulary-sized logits), so that a row has a CU's worth
+// of wavefronts behind its fp64 exponentials.
+template <typename TI, typename TO, int kThreads>
+__global__ __launch_bounds__(kThreads) void softmax_rows_kernel(const typename Elem<TI>::store_t* __restrict__ x,
+                                                                typename Elem<TO>::store_t* __restrict__ out, long n) {
     using EI = Elem<TI>;
     using EO = Elem<TO>;
-    __shared__ double slots[kWaves];
+    constexpr int kNW = kThreads / kWave;
+    __shared__ double slots[kNW];
     const auto* xr = x + static_cast<long>(blockIdx.x) * n;
     auto* outr = out + static_cast<long>(blockIdx.x) * n;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
 
     double m = -INFINITY;
-    for (long j = threadIdx.x; j < n; j += kBlock) {
+    for (long j = threadIdx.x; j < n; j += kThreads) {
         const double v = EI::to_f64(xr[j]);
         if (v > m) m = v;                       // as the host: a NaN never replaces the max
     }
@@ -54,19 +58,19 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_kernel(const typename Ele
     __syncthreads();
     m = slots[0];
 #pragma unroll
-    for (int i = 1; i < kWaves; ++i) m = fmax(m, slots[i]);
+    for (int i = 1; i < kNW; ++i) m = fmax(m, slots[i]);
     __syncthreads();
 
     double s = 0.0;
-    for (long j = threadIdx.x; j < n; j += kBlock) s += exp(EI::to_f64(xr[j]) - m);
+    for (long j = threadIdx.x; j < n; j += kThreads) s += exp(EI::to_f64(xr[j]) - m);
     s = wave_sum(s);
     if (lane == 0) slots[wave] = s;
     __syncthreads();
     s = 0.0;
 #pragma unroll
-    for (int i = 0; i < kWaves; ++i) s += slots[i];
+    for (int i = 0; i < kNW; ++i) s += slots[i];
 
-    for (long j = threadIdx.x; j < n; j += kBlock) outr[j] = EO::from_f64(exp(EI::to_f64(xr[j]) - m) / s);
+    for (long j = threadIdx.x; j < n; j += kThreads) outr[j] = EO::from_f64(exp(EI::to_f64(xr[j]) - m) / s);
 }
 
 // Rows of up to kBlock * EPT elements: the same, with each thread's exponentials kept in
@@ -546,10 +550,15 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
         PARAS_HIP_TRY(hipGetLastError());
         return PARAS_OK;
     }
-    if (dtype_out == PARAS_F32 && sizeof(SI) == 2)
-        hipLaunchKernelGGL((softmax_rows_kernel<TI, float>), g, b, 0, s, static_cast<const SI*>(x), static_cast<float*>(out), n);
+    const bool widen_long = dtype_out == PARAS_F32 && sizeof(SI) == 2;
+    if (rows <= 2048) {           // few long rows: a CU's worth of wavefronts per row
+        const dim3 b4(1024);
+        if (widen_long) hipLaunchKernelGGL((softmax_rows_kernel<TI, float, 1024>), g, b4, 0, s, static_cast<const SI*>(x), static_cast<float*>(out), n);
+        else            hipLaunchKernelGGL((softmax_rows_kernel<TI, TI, 1024>), g, b4, 0, s, static_cast<const SI*>(x), static_cast<SI*>(out), n);
+    } else if (widen_long)
+        hipLaunchKernelGGL((softmax_rows_kernel<TI, float, kBlock>), g, b, 0, s, static_cast<const SI*>(x), static_cast<float*>(out), n);
     else
-        hipLaunchKernelGGL((softmax_rows_kernel<TI, TI>), g, b, 0, s, static_cast<const SI*>(x), static_cast<SI*>(out), n);
+        hipLaunchKernelGGL((softmax_rows_kernel<TI, TI, kBlock>), g, b, 0, s, static_cast<const SI*>(x), static_cast<SI*>(out), n);
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
 }
