@@ -11,6 +11,7 @@
 // `addend` is a matrix with row stride ld_add; ld_add = 0 broadcasts one row
 // (a bias) over all rows.
 #include <hip/hip_runtime.h>
+#include <cstdlib>
 
 #include <type_traits>
 
@@ -400,8 +401,17 @@ __global__ __launch_bounds__(256) void skinny_splitk_finish_kernel(const DensePa
 
 // Splits of the contraction for the workspace kernel (0 = it does not apply): enough workgroups to
 // fill the chip twice, at least two slabs each.
+// Few rows but many columns (a vocabulary projection, a fused gate-up projection at M = 64 ... 128):
+// from about 200 tiles of 128 x 128 the tile kernel streams the weights faster than the few-row
+// kernels do (M = 128, N = 128256, K = 4096: 267 against 649 us; N = 28672: 75 against 106 us; at
+// N = 6144 the few-row kernels win, 47 against 67 us).  Up to 32 rows the few-row kernels stay.
+bool few_rows_by_tiles(long M, long N, long batch) {
+    return M > 32 && M <= kSkinnyMaxM && (N + gemm::kBN - 1) / gemm::kBN * batch >= 192;
+}
+
 int splitk_plan(long M, long N, long K, long batch, int* pieces_per_split) {
     if (M < 32 || M > kSkinnyMaxM || K % 64 != 0 || N < 512) return 0;   // up to 16 rows the activations are no load
+    if (few_rows_by_tiles(M, N, batch)) return 0;
     const long pieces = K / 64;
     const long groups = (N + 127) / 128 * batch;
     long splits = (512 + groups - 1) / groups;
@@ -600,7 +610,7 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
             return PARAS_OK;
         }
     }
-    if (M <= kSkinnyMaxM && batch <= 65535 && (N + 15) / 16 <= 0x7fffffffLL) {
+    if (!few_rows_by_tiles(M, N, batch) && M <= kSkinnyMaxM && batch <= 65535 && (N + 15) / 16 <= 0x7fffffffLL) {
         if (dtype == PARAS_BF16) launch_skinny<bf16_t>(p, batch, s);
         else                     launch_skinny<f16_t>(p, batch, s);
         PARAS_HIP_TRY(hipGetLastError());
