@@ -37,11 +37,17 @@ struct DenseParams {
     int  m_tiles, n_units;      // row tiles (128 or 256 rows), column units (128 or 256 columns)
     float alpha, beta;
     double alpha64, beta64;     // the same, for fp64 tensors
+    int  splits;                // kPartial kernels: parts of the contraction, one workgroup each per tile
+    long k_per_split;           // contraction elements per part (a multiple of 64)
+    float* partial;             // [batch][split][M][N] fp32
 };
 
 // S = Tile256 (8 waves, 256 x 256; for problems with at least 144 such tiles), Tile128 (4 waves,
 // 128 x 256) or Tile128x128 (4 waves, one column group; when there would be fewer than 512 tiles of 128 x 256).
-template <typename T, typename S>
+// kPartial: the contraction is split over p.splits workgroups per tile (the few-tile problems of 33 to
+// 128 rows: a projection at decode batch sizes has 32 to 112 tiles for 256 CUs); each writes its
+// fp32 partial tile, and skinny_splitk_finish_kernel adds them in split order and applies the epilogue.
+template <typename T, typename S, bool kPartial = false>
 __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_gemm_nt_kernel(const DenseParams p) {
     using El = Elem<T>;
     __shared__ __attribute__((aligned(16))) typename S::Lds lds;
@@ -49,11 +55,15 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
     // Column units innermost: the workgroups running together share the A row panel
     // (and, across m-tiles, stream the same B panels through L2).
     const long per_batch = static_cast<long>(p.m_tiles) * p.n_units;
-    const long bidx = blockIdx.x / per_batch, rem = blockIdx.x % per_batch;
+    const long tile_id = kPartial ? blockIdx.x / p.splits : blockIdx.x;
+    const long split = kPartial ? blockIdx.x % p.splits : 0;
+    const long k_first = kPartial ? split * p.k_per_split : 0;
+    const long k_count = kPartial ? (k_first + p.k_per_split < p.K ? p.k_per_split : p.K - k_first) : p.K;
+    const long bidx = tile_id / per_batch, rem = tile_id % per_batch;
     const int mt = static_cast<int>(rem / p.n_units), nu = static_cast<int>(rem % p.n_units);
     const long row0 = static_cast<long>(mt) * S::kBM, n0 = static_cast<long>(nu) * S::kGroups * kBN;
-    const std::uint16_t* A = p.a + bidx * p.sa;
-    const std::uint16_t* B = p.b + bidx * p.sb;
+    const std::uint16_t* A = p.a + bidx * p.sa + k_first;
+    const std::uint16_t* B = p.b + bidx * p.sb + k_first;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lh = lane >> 5;
@@ -81,8 +91,26 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
 #pragma unroll
     for (int g = 0; g < G; ++g) b_base[g] = B;
     float16_t acc[G][2][2];
-    S::template mainloop<T>(A, a_off, b_base, b_off, p.K, lds, acc);
+    S::template mainloop<T>(A, a_off, b_base, b_off, k_count, lds, acc);
 
+    if constexpr (kPartial) {
+        float* dst = p.partial + (bidx * p.splits + split) * (p.M * p.N);
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni) {
+                    const long col = n0 + g * kBN + wn * 64 + ni * 32 + lr;
+                    if (col >= p.N) continue;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const long row = row0 + wm * 64 + mi * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                        if (row < p.M) dst[row * p.N + col] = acc[g][mi][ni][r];
+                    }
+                }
+        return;
+    }
     std::uint16_t* C = p.c + bidx * p.sc;
     const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
 #pragma unroll
@@ -409,6 +437,23 @@ bool few_rows_by_tiles(long M, long N, long batch) {
     return M > 32 && M <= kSkinnyMaxM && (N + gemm::kBN - 1) / gemm::kBN * batch >= 192;
 }
 
+// Parts of the contraction for the 128 x 128 tile kernel with a workspace (0 = it does not apply): 49 to
+// 128 rows and too few tiles to fill the chip; about 384 workgroups in all (measured 128 ... 1024: fewer
+// leave CUs idle, more only add partial tiles for the finishing kernel to read), at least four k-tiles each.
+int tile_splitk_plan(long M, long N, long K, long batch, long* k_per_split) {
+    if (M <= 48 || M > kSkinnyMaxM || K % 64 != 0 || N < 128 || few_rows_by_tiles(M, N, batch)) return 0;
+    const long tiles = (N + gemm::kBN - 1) / gemm::kBN * batch;      // one row tile
+    const long k_tiles = K / 64;
+    long splits = (384 + tiles - 1) / tiles;
+    if (splits > k_tiles / 4) splits = k_tiles / 4;
+    if (splits < 2) return 0;
+    const long per = (k_tiles + splits - 1) / splits;
+    splits = (k_tiles + per - 1) / per;
+    if (splits < 2 || tiles * splits > 0x7fffffffL) return 0;
+    *k_per_split = per * 64;
+    return static_cast<int>(splits);
+}
+
 int splitk_plan(long M, long N, long K, long batch, int* pieces_per_split) {
     if (M < 32 || M > kSkinnyMaxM || K % 64 != 0 || N < 512) return 0;   // up to 16 rows the activations are no load
     if (few_rows_by_tiles(M, N, batch)) return 0;
@@ -525,7 +570,9 @@ size_t paras_gemm_nt_workspace(int64_t M, int64_t N, int64_t K, int64_t batch, i
     using namespace paras;
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || (dtype != PARAS_BF16 && dtype != PARAS_F16)) return 0;
     int per = 0;
-    const int splits = splitk_plan(M, N, K, batch, &per);
+    long kper = 0;
+    int splits = tile_splitk_plan(M, N, K, batch, &kper);
+    if (splits == 0) splits = splitk_plan(M, N, K, batch, &per);
     return static_cast<size_t>(splits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
 }
 
@@ -588,6 +635,26 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
     PARAS_REQUIRE(m_tiles * n_units * batch <= 0x7fffffffLL, "paras_gemm_nt: too many tiles");
     p.m_tiles = static_cast<int>(m_tiles); p.n_units = static_cast<int>(n_units);
     if (workspace != nullptr && batch <= 65535) {
+        long kper = 0;
+        const int tsplits = tile_splitk_plan(M, N, K, batch, &kper);
+        const size_t tneed = static_cast<size_t>(tsplits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
+        if (tsplits >= 2 && workspace_bytes >= tneed && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+            p.m_tiles = 1;
+            p.n_units = static_cast<int>((N + gemm::kBN - 1) / gemm::kBN);
+            p.splits = tsplits;
+            p.k_per_split = kper;
+            p.partial = static_cast<float*>(workspace);
+            const unsigned blocks = static_cast<unsigned>(static_cast<long>(p.n_units) * batch * tsplits);
+            const bool bf = dtype == PARAS_BF16;
+            if (bf) hipLaunchKernelGGL((dense_gemm_nt_kernel<bf16_t, gemm::Tile128x128, true>), dim3(blocks), dim3(gemm::Tile128x128::kThreads), 0, s, p);
+            else    hipLaunchKernelGGL((dense_gemm_nt_kernel<f16_t, gemm::Tile128x128, true>), dim3(blocks), dim3(gemm::Tile128x128::kThreads), 0, s, p);
+            PARAS_HIP_TRY(hipGetLastError());
+            const dim3 fgrid(static_cast<unsigned>((M * N + 255) / 256), static_cast<unsigned>(batch));
+            if (bf) hipLaunchKernelGGL((skinny_splitk_finish_kernel<bf16_t>), fgrid, dim3(256), 0, s, p, p.partial, tsplits);
+            else    hipLaunchKernelGGL((skinny_splitk_finish_kernel<f16_t>), fgrid, dim3(256), 0, s, p, p.partial, tsplits);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
         int per = 0;
         const int splits = splitk_plan(M, N, K, batch, &per);
         const size_t need = static_cast<size_t>(splits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);

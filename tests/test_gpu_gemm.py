@@ -198,11 +198,12 @@ def test_gemm_nt_few_rows_batched():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(32, 4096, 4096), (64, 4096, 1024), (64, 1027, 4096), (100, 1536, 2048), (128, 2050, 4096),
-                                   (33, 640, 1088)])
+                                   (33, 640, 1088), (48, 4096, 2048), (49, 384, 4096), (128, 4096, 14336), (77, 130, 704)])
 def test_gemm_nt_few_rows_with_workspace(shape, dtype):
     """32 to 128 rows with the workspace the library asks for: the contraction is split over
-    workgroups and the partial sums are added in a fixed order -- same bar as every other GEMM
-    kernel, same result on every call, with bias / scaled addend and ragged N and K splits."""
+    workgroups (of the few-row kernel up to 48 rows, of the 128 x 128 tile kernel above) and the
+    partial sums are added in a fixed order -- same bar as every other GEMM kernel, same result on
+    every call, with bias / scaled addend and ragged N and K splits."""
     M, N, K = shape
     torch.manual_seed(M + N + K)
     a = torch.randn(M, K).to(dtype)
@@ -218,6 +219,27 @@ def test_gemm_nt_few_rows_with_workspace(shape, dtype):
     got = capi.gemm_nt(a.cuda(), b.cuda(), addm.cuda(), alpha=0.5, beta=2.0, workspace=True)
     want = torch.addmm(addm.float(), a.float(), b.float().t(), beta=2.0, alpha=0.5)
     assert bool(((got.float().cpu() - want).abs() <= 2 * ulp16(want, dtype) + 1e-6).all())
+
+
+def test_gemm_nt_few_rows_and_many_columns_take_the_tile_kernel():
+    """33 to 128 rows against a vocabulary-sized weight matrix: enough 128 x 128 tiles to fill the
+    chip, so no workspace is asked for and the result is the tile kernel's."""
+    torch.manual_seed(44)
+    M, N, K = 100, 24576 + 70, 256
+    a = torch.randn(M, K).bfloat16()
+    b = (torch.randn(N, K) / 16).bfloat16()
+    assert capi.lib().paras_gemm_nt_workspace(M, N, K, 1, capi.BF16) == 0
+    got = capi.gemm_nt(a.cuda(), b.cuda(), workspace=True)
+    assert_gemm_close(got, O.matmul_nt(a, b), torch.bfloat16)
+    bias = torch.randn(N).bfloat16()
+    got = capi.gemm_nt(a.cuda(), b.cuda(), bias.cuda(), alpha=1.0, beta=1.0)
+    assert_gemm_close(got, torch.nn.functional.linear(a, b, bias), torch.bfloat16)
+    # batched: 3 x 64 tiles
+    a3 = torch.randn(3, 60, 256, device="cuda").bfloat16()
+    b3 = (torch.randn(3, 8192, 256, device="cuda") / 16).bfloat16()
+    out = capi.gemm_nt(a3, b3, workspace=True)
+    for i in range(3):
+        assert_gemm_close(out[i], O.matmul_nt(a3[i].cpu(), b3[i].cpu()), torch.bfloat16)
 
 
 def test_gemm_nt_workspace_batched_and_shapes_that_need_none():
