@@ -32,14 +32,27 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 // doubles used as two alternating sets: a call uses set `parity & 1`, so the readers of one call
 // never race with the writers of the next and a single barrier per call is enough (the set is
 // reused only two calls later, with this call's barrier in between).
+template <int NW = kWavesPerBlock>
 __device__ __forceinline__ double block_sum(double v, double* slots, int parity) {
     v = wave_sum(v);
-    double* set = slots + (parity & 1) * kWavesPerBlock;
+    if constexpr (NW == 1) return v;
+    double* set = slots + (parity & 1) * NW;
     if ((threadIdx.x & (kWave - 1)) == 0) set[threadIdx.x / kWave] = v;
     __syncthreads();
     double t = 0.0;
 #pragma unroll
-    for (int i = 0; i < kWavesPerBlock; ++i) t += set[i];
+    for (int i = 0; i < NW; ++i) t += set[i];
+    return t;
+}
+
+// The same for a number of waves known only at run time (sets of 16).
+__device__ __forceinline__ double block_sum_any(double v, double* slots, int parity, int nw) {
+    v = wave_sum(v);
+    double* set = slots + (parity & 1) * 16;
+    if ((threadIdx.x & (kWave - 1)) == 0) set[threadIdx.x / kWave] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (int i = 0; i < nw; ++i) t += set[i];
     return t;
 }
 
@@ -58,23 +71,29 @@ __device__ __forceinline__ double rsqrt_f64(double v) {
     return r;
 }
 
-// Register-resident row: H == vectors per row * kVec, vectors per row <= kBlock*NV.
-// (Four vectors per thread need more than the 64 registers that eight waves per SIMD leave.)
-template <typename T, int NV>
-__global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
+// Register-resident row: H == vectors per row * kVec, vectors per row <= BLOCK*NV.  The workgroup is
+// sized to the row (128 threads for a row of 1024 16-bit elements, 1024 for one of 16384), at most two
+// vectors per thread: four need more than the 64 registers that eight waves per SIMD leave.
+// PIPE (short rows): a workgroup walks many rows and asks for its next row before it works on the
+// current one -- a workgroup per row of 2 or 4 KB is bound by the rate at which workgroups start.
+// BLOCK = 0: the workgroup size is whatever the launch says (a multiple of 64 up to 1024), for rows
+// that would leave much of a power-of-two workgroup idle (5120 elements: 320 threads).
+template <typename T, int NV, int BLOCK, bool PIPE = false>
+__global__ __launch_bounds__((BLOCK == 0 ? 1024 : BLOCK), 8) void rms_norm_fwd_vec(
     const typename Elem<T>::store_t* __restrict__ x, const typename Elem<T>::store_t* __restrict__ w,
     typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, int H,
     double eps, double inv_h) {
     using E = Elem<T>;
     using S = typename E::store_t;
     constexpr int V = E::kVec;
-    __shared__ double slots[2 * kWavesPerBlock];
+    __shared__ double slots[2 * ((BLOCK == 0 ? 1024 : BLOCK) / kWave)];
+    const int block = BLOCK == 0 ? static_cast<int>(blockDim.x) : BLOCK;
 
     const int nvec = H / V;  // 16-byte vectors per row
     u32x4 wv[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int c = threadIdx.x + i * kBlock;
+        const int c = threadIdx.x + i * block;
         if (c < nvec) wv[i] = load16(w + static_cast<long>(c) * V);  // shared by every row: an L2 hit
     }
     // A NaN result must come out as the host's 16-bit types write it, which the fast tier's
@@ -88,7 +107,7 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             w_odd[i] = false;
-            const int c = threadIdx.x + i * kBlock;
+            const int c = threadIdx.x + i * block;
             if (c < nvec) {
 #pragma unroll
                 for (int p = 0; p < 4; ++p)
@@ -97,19 +116,27 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
         }
     }
     int sum_calls = 0;
-    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+    auto load_row = [&](long r, u32x4 (&dst)[NV]) {
         const S* xr = x + r * H;
-        S* outr = out + r * H;
-        u32x4 xv[NV];
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int c = threadIdx.x + i * kBlock;
-            if (c < nvec) xv[i] = load16_nt(xr + static_cast<long>(c) * V);
+            const int c = threadIdx.x + i * block;
+            if (c < nvec) dst[i] = load16_nt(xr + static_cast<long>(c) * V);
+        }
+    };
+    u32x4 xv[NV], xn[NV];
+    if (PIPE && blockIdx.x < rows) load_row(blockIdx.x, xv);
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        S* outr = out + r * H;
+        if constexpr (PIPE) {
+            if (r + gridDim.x < rows) load_row(r + gridDim.x, xn);
+        } else {
+            load_row(r, xv);
         }
         double ss = 0.0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int c = threadIdx.x + i * kBlock;
+            const int c = threadIdx.x + i * block;
             if (c < nvec) {
                 const S* e = reinterpret_cast<const S*>(&xv[i]);
 #pragma unroll
@@ -119,7 +146,8 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
                 }
             }
         }
-        ss = block_sum(ss, slots, sum_calls++);
+        if constexpr (BLOCK == 0) ss = block_sum_any(ss, slots, sum_calls++, block / kWave);
+        else ss = block_sum<(BLOCK == 0 ? 1 : BLOCK) / kWave>(ss, slots, sum_calls++);
         // 16-bit tensors: mean by the reciprocal and the refined rsqrt (outputs
         // cannot see the difference); fp32 / fp64 tensors: the host's own form.
         const double rs = sizeof(S) == 2 ? rsqrt_f64(fma(ss, inv_h, eps)) : 1.0 / sqrt(ss / static_cast<double>(H) + eps);
@@ -129,7 +157,7 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
             const bool row_odd = !(rs32 > 0.0f && rs32 <= 3.4028234663852886e38f);
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
-                const int c = threadIdx.x + i * kBlock;
+                const int c = threadIdx.x + i * block;
                 if (c < nvec) {
                     bool fix;
                     u32x4 o = scale_vec16_fast<T>(xv[i], wv[i], rs32, fix);
@@ -141,7 +169,7 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
         } else {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
-                const int c = threadIdx.x + i * kBlock;
+                const int c = threadIdx.x + i * block;
                 if (c < nvec) {
                     const S* e  = reinterpret_cast<const S*>(&xv[i]);
                     const S* we = reinterpret_cast<const S*>(&wv[i]);
@@ -152,6 +180,10 @@ __global__ __launch_bounds__(kBlock, (NV <= 2 ? 8 : 4)) void rms_norm_fwd_vec(
                     store16_nt(outr + static_cast<long>(c) * V, o);
                 }
             }
+        }
+        if constexpr (PIPE) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) xv[i] = xn[i];
         }
     }
 }
@@ -494,12 +526,31 @@ int launch_fwd(const void* x, const void* w, void* out, float* rstd, long rows, 
     const bool aligned = (H % V == 0) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
                                            reinterpret_cast<uintptr_t>(out)) % 16 == 0);
     const long nvec = H / V;
-    if (aligned && nvec <= kBlock * 1 && H <= INT32_MAX)
-        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 1>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps, 1.0 / static_cast<double>(H));
-    else if (aligned && nvec <= kBlock * 2)
-        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps, 1.0 / static_cast<double>(H));
-    else if (aligned && nvec <= kBlock * 4)
-        hipLaunchKernelGGL((rms_norm_fwd_vec<T, 4>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, (int)H, eps, 1.0 / static_cast<double>(H));
+#define PARAS_RMS_FWD(NV_, BLOCK_)                                                                                  \
+    hipLaunchKernelGGL((rms_norm_fwd_vec<T, NV_, BLOCK_>), dim3(grid), dim3(BLOCK_), 0, s, xs, ws, os, rstd, rows, \
+                       (int)H, eps, 1.0 / static_cast<double>(H))
+    // short rows: sixteen workgroups' worth of rows per CU at a time, each workgroup walking its share
+    int dev_id = 0;
+    (void)hipGetDevice(&dev_id);
+    auto* dst_ = DeviceContext::instance().device(dev_id);
+    const long pipe_cap = (dst_ ? dst_->compute_units : 256) * 16;
+    const int pgrid = static_cast<int>(rows < pipe_cap ? rows : pipe_cap);
+#define PARAS_RMS_FWD_PIPE(NV_, BLOCK_)                                                                                   \
+    hipLaunchKernelGGL((rms_norm_fwd_vec<T, NV_, BLOCK_, true>), dim3(pgrid), dim3(BLOCK_), 0, s, xs, ws, os, rstd, rows, \
+                       (int)H, eps, 1.0 / static_cast<double>(H))
+    if (aligned && nvec <= 128)       PARAS_RMS_FWD_PIPE(1, 128);
+    else if (aligned && nvec <= 256)  PARAS_RMS_FWD_PIPE(1, 256);
+#undef PARAS_RMS_FWD_PIPE
+    else if (aligned && nvec <= 2048) {
+        const int fit = static_cast<int>(((nvec + 1) / 2 + 63) / 64 * 64);     // threads that two vectors each fill
+        if (fit == 256)       PARAS_RMS_FWD(2, 256);
+        else if (fit == 512)  PARAS_RMS_FWD(2, 512);
+        else if (fit == 1024) PARAS_RMS_FWD(2, 1024);
+        else
+            hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2, 0>), dim3(grid), dim3(fit), 0, s, xs, ws, os, rstd, rows, (int)H, eps,
+                               1.0 / static_cast<double>(H));
+    }
+#undef PARAS_RMS_FWD
     else
         hipLaunchKernelGGL((rms_norm_fwd_any<T>), dim3(grid), dim3(kBlock), 0, s, xs, ws, os, rstd, rows, H, eps);
     PARAS_HIP_TRY(hipGetLastError());
