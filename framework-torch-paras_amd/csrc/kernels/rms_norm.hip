@@ -188,6 +188,76 @@ __global__ __launch_bounds__((BLOCK == 0 ? 1024 : BLOCK), 8) void rms_norm_fwd_v
     }
 }
 
+// Rows of at most 64 vectors (per-head norms: 128 elements): TPR lanes per row, 64 / TPR rows per
+// wave, no LDS and no barrier; the sum of squares meets over the row's lanes by exchanges inside the
+// wave.  Persistent, the next group of rows requested before the current one is worked on.
+template <typename T, int TPR>
+__global__ __launch_bounds__(256, 8) void rms_norm_fwd_small(
+    const typename Elem<T>::store_t* __restrict__ x, const typename Elem<T>::store_t* __restrict__ w,
+    typename Elem<T>::store_t* __restrict__ out, float* __restrict__ rstd, long rows, int H,
+    double eps, double inv_h) {
+    using E = Elem<T>;
+    using S = typename E::store_t;
+    constexpr int V = E::kVec;
+    constexpr int RPW = kWave / TPR;                      // rows per wave
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int sub = lane % TPR, rsel = lane / TPR;
+    const int nvec = H / V;
+    const bool have = sub < nvec;
+    u32x4 wv = u32x4{0u, 0u, 0u, 0u};
+    if (have) wv = load16(w + static_cast<long>(sub) * V);
+    bool w_odd = false;
+    if constexpr (sizeof(S) == 2) {
+        constexpr std::uint32_t kExp = __is_same(T, bf16_t) ? 0x7F80u : 0x7C00u;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) w_odd = w_odd || ((wv[p] & kExp) == kExp) || (((wv[p] >> 16) & kExp) == kExp);
+    }
+    const long step = static_cast<long>(gridDim.x) * (256 / kWave) * RPW;
+    long r = (static_cast<long>(blockIdx.x) * (256 / kWave) + wave) * RPW + rsel;
+    auto fetch = [&](long row) -> u32x4 {
+        return (have && row < rows) ? load16_nt(x + row * H + static_cast<long>(sub) * V) : u32x4{0u, 0u, 0u, 0u};
+    };
+    u32x4 xv = fetch(r);
+    for (; r - rsel < rows; r += step) {                  // wave-uniform: the wave's first row
+        const u32x4 xn = fetch(r + step);
+        const bool live = have && r < rows;
+        double ss = 0.0;
+        {
+            const S* e = reinterpret_cast<const S*>(&xv);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const double v = E::to_f64(e[j]);
+                ss = fma(v, v, ss);
+            }
+        }
+#pragma unroll
+        for (int off = TPR / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+        const double rs = sizeof(S) == 2 ? rsqrt_f64(fma(ss, inv_h, eps)) : 1.0 / sqrt(ss / static_cast<double>(H) + eps);
+        const float rs32 = static_cast<float>(rs);
+        if (sub == 0 && r < rows) rstd[r] = rs32;
+        if (live) {
+            S* outr = out + r * H + static_cast<long>(sub) * V;
+            if constexpr (sizeof(S) == 2) {
+                const bool row_odd = !(rs32 > 0.0f && rs32 <= 3.4028234663852886e38f);
+                bool fix;
+                u32x4 o = scale_vec16_fast<T>(xv, wv, rs32, fix);
+                fix = fix || row_odd || w_odd;
+                if (__builtin_expect(fix, 0)) o = scale_vec16_fix<T>(xv, wv, o, rs32, rs);
+                store16_nt(outr, o);
+            } else {
+                const S* e  = reinterpret_cast<const S*>(&xv);
+                const S* we = reinterpret_cast<const S*>(&wv);
+                u32x4 o;
+                S* oe = reinterpret_cast<S*>(&o);
+#pragma unroll
+                for (int j = 0; j < V; ++j) oe[j] = scale_one<T>(e[j], rs32, rs, we[j]);
+                store16_nt(outr, o);
+            }
+        }
+        xv = xn;
+    }
+}
+
 // Any H, any alignment: scalar accesses, row re-read for the second pass.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rms_norm_fwd_any(
@@ -538,9 +608,21 @@ int launch_fwd(const void* x, const void* w, void* out, float* rstd, long rows, 
 #define PARAS_RMS_FWD_PIPE(NV_, BLOCK_)                                                                                   \
     hipLaunchKernelGGL((rms_norm_fwd_vec<T, NV_, BLOCK_, true>), dim3(pgrid), dim3(BLOCK_), 0, s, xs, ws, os, rstd, rows, \
                        (int)H, eps, 1.0 / static_cast<double>(H))
-    if (aligned && nvec <= 128)       PARAS_RMS_FWD_PIPE(1, 128);
+#define PARAS_RMS_FWD_SMALL(TPR_)                                                                                      \
+    do {                                                                                                              \
+        const long groups = (rows + (4 * (kWave / TPR_)) - 1) / (4 * (kWave / TPR_));                                 \
+        const int sgrid = static_cast<int>(groups < pipe_cap ? groups : pipe_cap);                                    \
+        hipLaunchKernelGGL((rms_norm_fwd_small<T, TPR_>), dim3(sgrid), dim3(256), 0, s, xs, ws, os, rstd, rows, (int)H, \
+                           eps, 1.0 / static_cast<double>(H));                                                        \
+    } while (0)
+    if (aligned && nvec <= 8)         PARAS_RMS_FWD_SMALL(8);
+    else if (aligned && nvec <= 16)   PARAS_RMS_FWD_SMALL(16);
+    else if (aligned && nvec <= 32)   PARAS_RMS_FWD_SMALL(32);
+    else if (aligned && nvec <= 64)   PARAS_RMS_FWD_SMALL(64);
+    else if (aligned && nvec <= 128)  PARAS_RMS_FWD_PIPE(1, 128);
     else if (aligned && nvec <= 256)  PARAS_RMS_FWD_PIPE(1, 256);
 #undef PARAS_RMS_FWD_PIPE
+#undef PARAS_RMS_FWD_SMALL
     else if (aligned && nvec <= 2048) {
         const int fit = static_cast<int>(((nvec + 1) / 2 + 63) / 64 * 64);     // threads that two vectors each fill
         if (fit == 256)       PARAS_RMS_FWD(2, 256);

@@ -41,7 +41,9 @@ def test_golden_vectors(tag):
 
 
 @pytest.mark.parametrize("dtype", EXACT)
-@pytest.mark.parametrize("shape", [(7, 200), (33, 4096), (5, 8192), (3, 10000), (64, 1024), (2, 8), (1, 1), (300, 264)])
+@pytest.mark.parametrize("shape", [(7, 200), (33, 4096), (5, 8192), (3, 10000), (64, 1024), (2, 8), (1, 1), (300, 264),
+                                   (1000, 128), (37, 64), (515, 256), (77, 512), (9000, 1024), (5000, 2048), (40, 5120), (21, 2880),
+                                   (6, 16384), (3, 12288), (1031, 32)])
 def test_rms_norm_matches_oracle(dtype, shape):
     x = torch.randn(*shape).to(dtype)
     w = (1 + 0.02 * torch.randn(shape[1])).to(dtype)
