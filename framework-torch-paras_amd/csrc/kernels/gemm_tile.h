@@ -255,12 +255,71 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
     compute(lds.st[(k_tiles - 1) & 1], lds.st[k_tiles & 1], 0, std::false_type{});
 }
 
+// A 256-row tile of which at most 64 rows exist (the last tile of a group of rows): the eight
+// waves share those 64 rows instead of six of them idling through the whole contraction.  Wave w
+// takes row block w / 4 (32 rows) and the 32 columns w % 4 of BOTH column groups, so a gate / up
+// pair still meets in one lane: 2 MFMAs per k-step and wave instead of 8, every product summed in
+// the same order as in the full tile (bit-identical results).  Only the first 64 A rows are staged
+// (a_off0: this thread's chunk of them); two LDS stages, one barrier per k-tile.
+template <typename T>
+__device__ __forceinline__ void short_tile_mainloop(const std::uint16_t* a_base, unsigned a_off0,
+                                                    const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][2],
+                                                    long K, TileLds& lds, float16_t (&acc)[2]) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lr = lane & 31, lh = lane >> 5;
+    const int rb = wave >> 2, cb = wave & 3;
+    u32x4 a_st, b_st[2][2];
+    auto load_tile = [&](long k0) {
+        a_st = load16(a_base + k0 + a_off0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) b_st[g][i] = load16(b_base[g] + k0 + b_off[g][i]);
+    };
+    auto store_tile = [&](StageLds& st) {
+        *reinterpret_cast<u32x4*>(&st.a[(tid >> 3) * kLS + (tid & 7) * 8]) = a_st;
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int c = tid + i * kThreads;
+                *reinterpret_cast<u32x4*>(&st.b[g][(c >> 3) * kLS + (c & 7) * 8]) = b_st[g][i];
+            }
+    };
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[g][r] = 0.f;
+    const int a_o = (rb * 32 + lr) * kLS + lh * 8;
+    const int b_o = (cb * 32 + lr) * kLS + lh * 8;
+    const long k_tiles = K / kBK;
+    load_tile(0);
+    store_tile(lds.st[0]);
+    __syncthreads();
+    for (long kt = 0; kt < k_tiles; ++kt) {
+        const StageLds& cur = lds.st[kt & 1];
+        if (kt + 1 < k_tiles) load_tile((kt + 1) * kBK);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 16; ++ks) {
+            const i16x8 af = *reinterpret_cast<const i16x8*>(&cur.a[a_o + ks * 16]);
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const i16x8 bf = *reinterpret_cast<const i16x8*>(&cur.b[g][b_o + ks * 16]);
+                acc[g] = MmaT<T>::run(af, bf, acc[g]);
+            }
+        }
+        if (kt + 1 < k_tiles) store_tile(lds.st[(kt + 1) & 1]);
+        __syncthreads();
+    }
+}
+
 }  // namespace wide
 
 // The two tile shapes as a kernel sees them.
 template <int G>
 struct Tile128G {
     static constexpr int kBM = gemm::kBM, kThreads = gemm::kThreads, kBChunks = 4, kGroups = G;
+    static constexpr int kShortRows = 0;    // no short-tile form
     using Lds = TileLdsG<G>;
     template <typename T>
     __device__ static __forceinline__ void mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[4],
@@ -279,6 +338,13 @@ struct Tile256 {
                                                     const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][2],
                                                     long K, Lds& lds, float16_t (&acc)[2][2][2]) {
         wide::tile_mainloop<T>(a_base, a_off, b_base, b_off, K, lds, acc);
+    }
+    static constexpr int kShortRows = 64;   // a tile with no more valid rows than this can take short_mainloop
+    template <typename T>
+    __device__ static __forceinline__ void short_mainloop(const std::uint16_t* a_base, unsigned a_off0,
+                                                          const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][2],
+                                                          long K, Lds& lds, float16_t (&acc)[2]) {
+        wide::short_tile_mainloop<T>(a_base, a_off0, b_base, b_off, K, lds, acc);
     }
 };
 

@@ -116,6 +116,27 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
             if (wrow >= p.Nw) wrow = p.Nw - 1;
             b_off[g][i] = static_cast<unsigned>(wrow * p.K + (c & 7) * 8);
         }
+    // An expert's last tile with few rows: the waves share those rows (same sums, a fraction of
+    // the time) instead of most of them idling through the contraction.
+    if constexpr (S::kShortRows > 0) {
+        if (row_end - row0 <= S::kShortRows) {
+            float16_t sacc[2];
+            S::template short_mainloop<T>(p.a, a_off[0], b_base, b_off, p.K, lds, sacc);
+            const long col = n0 + (wave & 3) * 32 + lr;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const long prow = row0 + (wave >> 2) * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                if (prow >= row_end) continue;
+                if (kSwiglu) {
+                    if (col < p.N) p.c[prow * p.N + col] = swiglu_one<T>(El::from_f32(sacc[0][r]), El::from_f32(sacc[1][r]));
+                } else {
+                    if (col < p.N) p.c[prow * p.N + col] = El::from_f32(sacc[0][r]);
+                    if (col + kBN < p.N) p.c[prow * p.N + col + kBN] = El::from_f32(sacc[1][r]);
+                }
+            }
+            return;
+        }
+    }
     float16_t acc[2][2][2];
     S::template mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, acc);
 

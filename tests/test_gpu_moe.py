@@ -194,6 +194,35 @@ def test_ffn_256_row_tiles_with_ragged_tiny_and_empty_experts():
     assert_ffn_close(out.cpu()[sel], ref, dt)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_ffn_rows_in_the_last_tile_of_every_expert(dtype):
+    """256-row tiles and experts whose last tiles hold 1, 40, 64, 65, 200 and 256 rows (a tile of at
+    most 64 rows is shared out among the waves differently): every token with a row in some
+    expert's last tile, and a few others, against the oracle."""
+    torch.manual_seed(11)
+    want_counts = [1025, 1064, 1088, 1089, 1224, 1280]
+    E, k, H, I = len(want_counts), 2, 2048, 256
+    T = sum(want_counts) // k
+    rows = torch.repeat_interleave(torch.arange(E), torch.tensor(want_counts))   # token t: experts rows[t], rows[t + T]
+    logits = 0.1 * torch.randn(T, E)
+    logits[torch.arange(T), rows[:T]] += 5.0
+    logits[torch.arange(T), rows[T:]] += 4.0
+    perm = torch.randperm(T)
+    logits = logits[perm].to(dtype)
+    x = torch.randn(T, H).to(dtype)
+    wg, wu = (0.03 * torch.randn(E, I, H)).to(dtype), (0.03 * torch.randn(E, I, H)).to(dtype)
+    wd = (0.05 * torch.randn(E, H, I)).to(dtype)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    assert counts.cpu().tolist() == want_counts
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    off, ordr = offsets.cpu().tolist(), order.cpu()
+    tails = [ordr[off[e] + (want_counts[e] - 1) // 256 * 256: off[e + 1]] // k for e in range(E)]
+    sel = torch.unique(torch.cat(tails + [torch.randperm(T)[:32]]))
+    r = O.moe_route(logits[sel], k)
+    ref = O.moe_ffn(x[sel], wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
+    assert_ffn_close(out.cpu()[sel], ref, dtype)
+
+
 @pytest.mark.parametrize("shape", [(8192, 8, 2, torch.bfloat16), (5000, 64, 6, torch.float32), (700, 16, 4, torch.float16)])
 def test_route_when_the_workgroups_do_not_wait_for_each_other(shape, monkeypatch):
     """With a wait of one poll most workgroups of the one-kernel routing stop waiting for the others
