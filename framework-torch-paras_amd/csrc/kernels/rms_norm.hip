@@ -427,17 +427,22 @@ __device__ __forceinline__ double bwd_coef(double rr, int H, bool h_pow2, double
 // kFull: every thread of the workgroup owns a vector (H == 8 * BLOCK * NV).  Then no memory
 // instruction sits under a lane mask and the compiler can count exactly which of them a wait has
 // to cover: with a mask it waits, before the next row, for the row's own store as well.
+// BLOCK == 0: the workgroup is as wide as the launch makes it (a whole number of waves, every
+// thread with a vector of its own: rows of 512 * n elements that are not a power of two).
 template <typename T, int NV, int BLOCK, bool kFull, int kTeams = 1>
-__global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
+__global__ __launch_bounds__(BLOCK == 0 ? 1024 : BLOCK * kTeams, 4) void rms_norm_bwd_fused(
     const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
     const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
     using E = Elem<T>;
     constexpr int V = 8;
-    constexpr int kWaves = BLOCK / kWave;
+    constexpr bool kDyn = BLOCK == 0;
+    static_assert(!kDyn || (kTeams == 1 && kFull), "a workgroup of run-time width has one team and no idle thread");
+    constexpr int kWaves = kDyn ? 16 : BLOCK / kWave;      // slots per sum (run-time width: the most there can be)
     __shared__ double slots[2 * kTeams * kWaves];
     __shared__ double team_dw[kTeams > 1 ? (kTeams - 1) * BLOCK * NV * V : 1];
     const int nvec = H / V;
-    const int team = kTeams > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / BLOCK) : 0;
+    const int block = kDyn ? static_cast<int>(blockDim.x) : BLOCK;
+    const int team = kTeams > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / (kDyn ? 1 : BLOCK)) : 0;
     const int tid = kTeams > 1 ? static_cast<int>(threadIdx.x) - team * BLOCK : static_cast<int>(threadIdx.x);
     const long slab = blockIdx.x;
     // Rows are dealt out round-robin: workgroup b takes rows b, b + G, b + 2G, ... (G workgroups),
@@ -462,14 +467,14 @@ __global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i]) {
-                const int c = tid + i * BLOCK;
+                const int c = tid + i * block;
                 gs[i] = load16_nt(go + r * H + static_cast<long>(c) * V);
                 xs[i] = load16_nt(x + r * H + static_cast<long>(c) * V);
             }
     };
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int c = tid + i * BLOCK;
+        const int c = tid + i * block;
         have[i] = kFull || c < nvec;
         u32x4 wv = {0u, 0u, 0u, 0u};
         if (have[i]) wv = load16(w + static_cast<long>(c) * V);
@@ -499,14 +504,28 @@ __global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
             if ((tid & (kWave - 1)) == 0) slot[tid / kWave] = dot;
             lds_barrier();   // not __syncthreads(): the loads requested above stay in flight across it
             dot = 0.0;
+            if constexpr (kDyn) {
+                const int nw = block / kWave;
+                for (int i = 0; i < nw; ++i) dot += slot[i];
+            } else if constexpr (kWaves <= 8) {
 #pragma unroll
-            for (int i = 0; i < kWaves; ++i) dot += slot[i];
+                for (int i = 0; i < kWaves; ++i) dot += slot[i];
+            } else {
+                // sixteen waves: four slots at a time, so that the slot values never hold more than
+                // eight registers (all sixteen at once push the prefetched row out to scratch memory)
+#pragma unroll
+                for (int i = 0; i < kWaves; i += 4) {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) dot += slot[i + u];
+                    asm volatile("" : "+v"(dot) : : "memory");
+                }
+            }
         }
         const double cd = bwd_coef(rr, H, h_pow2, inv_h) * dot;
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (have[i])
-                store16_nt(gx + r * H + static_cast<long>(tid + i * BLOCK) * V, bwd_vec_second<T>(g64[i], x64[i], w64[i], rr, cd));
+                store16_nt(gx + r * H + static_cast<long>(tid + i * block) * V, bwd_vec_second<T>(g64[i], x64[i], w64[i], rr, cd));
     };
     // The first row is written out in front of the loop: entered straight from the prologue, the
     // loop header would inherit "first loads pending" and the compiler's wait insertion would then
@@ -534,10 +553,74 @@ __global__ __launch_bounds__(BLOCK * kTeams, 4) void rms_norm_bwd_fused(
 #pragma unroll
     for (int i = 0; i < NV; ++i)
         if (have[i]) {
-            double* dst = partial + slab * H + static_cast<long>(tid + i * BLOCK) * V;
+            double* dst = partial + slab * H + static_cast<long>(tid + i * block) * V;
 #pragma unroll
             for (int j = 0; j < V; ++j) dst[j] = dw[i][j];
         }
+}
+
+// Rows of at most 64 vectors (per-head norms: 128 elements), 16-bit tensors: TPR lanes per row,
+// 64 / TPR rows per wave, each lane group walking rows of its own with the next one requested
+// ahead; the row's dot product meets over its lanes by exchanges inside the wave, so the row loop
+// has no LDS and no barrier.  The same arithmetic as rms_norm_bwd_fused; the column sums of the
+// workgroup's 4 * 64 / TPR lane groups are added in LDS, in group order, into one partial sum.
+template <typename T, int TPR>
+__global__ __launch_bounds__(256, 4) void rms_norm_bwd_small(
+    const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
+    const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
+    using E = Elem<T>;
+    constexpr int V = 8, RPW = kWave / TPR, kGroups = (256 / kWave) * RPW;
+    __shared__ double dw_lds[kGroups][TPR * V];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int sub = lane % TPR, rsel = lane / TPR;
+    const int nvec = H / V;
+    const bool have = sub < nvec;
+    const double inv_h = 1.0 / static_cast<double>(H);
+    const bool h_pow2 = __builtin_amdgcn_readfirstlane((H & (H - 1)) == 0) != 0;
+    double w64[V], dw[V];
+    {
+        u32x4 wv = {0u, 0u, 0u, 0u};
+        if (have) wv = load16(w + static_cast<long>(sub) * V);
+        const std::uint16_t* we = reinterpret_cast<const std::uint16_t*>(&wv);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            w64[j] = E::to_f64(we[j]);
+            dw[j] = 0.0;
+        }
+    }
+    const long step = static_cast<long>(gridDim.x) * kGroups;
+    long r = (static_cast<long>(blockIdx.x) * (256 / kWave) + wave) * RPW + rsel;
+    auto fetch = [&](const std::uint16_t* base, long row) -> u32x4 {
+        return (have && row < rows) ? load16_nt(base + row * H + static_cast<long>(sub) * V) : u32x4{0u, 0u, 0u, 0u};
+    };
+    u32x4 gv = fetch(go, r), xv = fetch(x, r);
+    float rstd_now = r < rows ? rstd[r] : 0.0f;
+    for (; r - rsel < rows; r += step) {                  // wave-uniform: the wave's first row
+        const u32x4 gn = fetch(go, r + step), xn = fetch(x, r + step);
+        const float rstd_nx = r + step < rows ? rstd[r + step] : 0.0f;
+        const bool live = have && r < rows;
+        const double rr = static_cast<double>(rstd_now);
+        double dot = 0.0, g64[V], x64[V];
+        if (live) bwd_vec_first<T>(gv, xv, w64, rr, dot, dw, g64, x64);
+#pragma unroll
+        for (int off = TPR / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, kWave);
+        const double cd = bwd_coef(rr, H, h_pow2, inv_h) * dot;
+        if (live) store16_nt(gx + r * H + static_cast<long>(sub) * V, bwd_vec_second<T>(g64, x64, w64, rr, cd));
+        gv = gn;
+        xv = xn;
+        rstd_now = rstd_nx;
+    }
+    if (have) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) dw_lds[wave * RPW + rsel][sub * V + j] = dw[j];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < H; c += 256) {
+        double t = 0.0;
+#pragma unroll 8
+        for (int k = 0; k < kGroups; ++k) t += dw_lds[k][c];
+        partial[static_cast<long>(blockIdx.x) * H + c] = t;
+    }
 }
 
 // Column sums of the slabs in a fixed order: thread (column c of kDwFinalCols, lane l of
@@ -625,9 +708,23 @@ int launch_fwd(const void* x, const void* w, void* out, float* rstd, long rows, 
 #undef PARAS_RMS_FWD_SMALL
     else if (aligned && nvec <= 2048) {
         const int fit = static_cast<int>(((nvec + 1) / 2 + 63) / 64 * 64);     // threads that two vectors each fill
+        // Wider than 256 threads: as many workgroups as are resident at once (eight waves per SIMD),
+        // each walking its rows with the next one requested ahead.  With few, long rows a workgroup
+        // per row leaves the chip half empty while the first rows arrive and the last ones drain
+        // (8192 rows of 8192: 56 -> 52 us, 4096 of 16384: 59 -> 51 us); at 256 threads it is the
+        // other way round (46 us against 47.5).
+        const long fit_resident = (dst_ ? dst_->compute_units : 256) * (32 / (fit / kWave));
+        const int fgrid = static_cast<int>(rows < fit_resident ? rows : fit_resident);
         if (fit == 256)       PARAS_RMS_FWD(2, 256);
-        else if (fit == 512)  PARAS_RMS_FWD(2, 512);
-        else if (fit == 1024) PARAS_RMS_FWD(2, 1024);
+        else if (fit == 512)
+            hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2, 512, true>), dim3(fgrid), dim3(512), 0, s, xs, ws, os, rstd, rows, (int)H, eps,
+                               1.0 / static_cast<double>(H));
+        else if (fit == 1024)
+            hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2, 1024, true>), dim3(fgrid), dim3(1024), 0, s, xs, ws, os, rstd, rows, (int)H, eps,
+                               1.0 / static_cast<double>(H));
+        else if (fit > 256)
+            hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2, 0, true>), dim3(fgrid), dim3(fit), 0, s, xs, ws, os, rstd, rows, (int)H, eps,
+                               1.0 / static_cast<double>(H));
         else
             hipLaunchKernelGGL((rms_norm_fwd_vec<T, 2, 0>), dim3(grid), dim3(fit), 0, s, xs, ws, os, rstd, rows, (int)H, eps,
                                1.0 / static_cast<double>(H));
@@ -649,6 +746,30 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
         const bool aligned = (H % 8 == 0) && ((reinterpret_cast<uintptr_t>(go) | reinterpret_cast<uintptr_t>(x) |
                                                reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gx)) % 16 == 0);
         const long nvec = H / 8;
+        if (aligned && nvec <= 64) {
+            // short rows: several rows per wave; as many workgroups as are resident at once (four
+            // per compute unit), never more than the workspace has partial sums for
+            int dev = 0;
+            (void)hipGetDevice(&dev);
+            auto* dst = DeviceContext::instance().device(dev);
+            const long resident = (dst ? dst->compute_units : 256) * 4;
+            const unsigned sgrid = static_cast<unsigned>(slabs < resident ? slabs : resident);
+            auto* part = static_cast<double*>(workspace);
+#define PARAS_BWD_SMALL(TPR_)                                                                                            \
+    hipLaunchKernelGGL((rms_norm_bwd_small<T, TPR_>), dim3(sgrid), dim3(256), 0, s, static_cast<const std::uint16_t*>(go), \
+                       static_cast<const std::uint16_t*>(x), static_cast<const std::uint16_t*>(w), rstd,                \
+                       static_cast<std::uint16_t*>(gx), part, rows, (int)H)
+            if (nvec <= 8)       PARAS_BWD_SMALL(8);
+            else if (nvec <= 16) PARAS_BWD_SMALL(16);
+            else if (nvec <= 32) PARAS_BWD_SMALL(32);
+            else                 PARAS_BWD_SMALL(64);
+#undef PARAS_BWD_SMALL
+            PARAS_HIP_TRY(hipGetLastError());
+            hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + kDwFinalCols - 1) / kDwFinalCols)), dim3(kDwFinalLanes * kDwFinalCols), 0, s,
+                               part, static_cast<S*>(gw), static_cast<long>(sgrid), H);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
         if (aligned && nvec <= 512 * 2) {
             const auto* g16 = static_cast<const std::uint16_t*>(go);
             const auto* x16 = static_cast<const std::uint16_t*>(x);
@@ -663,7 +784,11 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
             (void)hipGetDevice(&dev);
             auto* dst = DeviceContext::instance().device(dev);
             const long cus = dst ? dst->compute_units : 256;
-            const long resident = (nvec <= kBlock ? 4 : nvec <= 512 ? 2 : 1) * cus;
+            // rows of a whole number of waves that are not 256, 512 or 1024 vectors: a workgroup of
+            // exactly that many threads
+            const bool exact_width = nvec % kWave == 0 && nvec != kBlock && nvec != 512 && nvec != 1024;
+            const long wg_waves = exact_width ? nvec / kWave : (nvec <= kBlock ? 4 : nvec <= 512 ? 8 : 16);
+            const long resident = (16 / wg_waves) * cus;
             const bool plenty = slabs >= resident;
             if (plenty) slabs = resident;
             // Rows of 2048 or 4096 elements, plenty of them: workgroups of 1024 threads in teams of
@@ -676,7 +801,9 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
     hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, FULL_>), grid, dim3(BLOCK_), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
 #define PARAS_BWD_LAUNCH_TEAMS(BLOCK_) \
     hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, BLOCK_, true, 1024 / BLOCK_>), grid, dim3(1024), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H)
-            if (teams && nvec == 512) PARAS_BWD_LAUNCH_TEAMS(512);
+            if (exact_width)
+                hipLaunchKernelGGL((rms_norm_bwd_fused<T, 1, 0, true>), grid, dim3(static_cast<unsigned>(nvec)), 0, s, g16, x16, w16, rstd, gx16, part, rows, (int)H);
+            else if (teams && nvec == 512) PARAS_BWD_LAUNCH_TEAMS(512);
             else if (teams)          PARAS_BWD_LAUNCH_TEAMS(kBlock);
             else if (nvec == kBlock) PARAS_BWD_LAUNCH(kBlock, true);
             else if (nvec < kBlock)  PARAS_BWD_LAUNCH(kBlock, false);

@@ -144,7 +144,9 @@ def test_full_size_rms_norm_and_swiglu_bf16():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("shape", [(70, 4096), (33, 2048), (16, 520), (300, 1024), (5, 8), (37, 8192), (20, 5120), (9, 8200)])
+@pytest.mark.parametrize("shape", [(70, 4096), (33, 2048), (16, 520), (300, 1024), (5, 8), (37, 8192), (20, 5120), (9, 8200),
+                                   (45, 6144), (50, 3072), (130, 1536), (70, 512), (31, 7168), (25, 2880),
+                                   (1000, 128), (37, 64), (100, 96), (3, 256), (515, 512), (1, 128), (70000, 128)])
 def test_rms_norm_backward_one_pass_kernel(shape, dtype):
     """Row sizes the one-pass backward kernel takes (16-byte aligned rows of up to 8192 elements; the
     last shape is beyond it), with slabs of rows that are full, ragged and single."""
@@ -162,7 +164,7 @@ def test_rms_norm_backward_many_rows_are_dealt_round_robin():
     """The one-pass kernel runs at most two workgroups per compute unit; with more rows than that
     times 16 every workgroup takes rows b, b + G, b + 2G, ...: row counts around the switch, with
     workgroups that get one row more than others."""
-    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520), (8192 + 7, 264)):
+    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520), (8192 + 7, 264), (4200, 5120), (9001, 3072), (4100, 8192)):
         torch.manual_seed(rows)
         x, w, go = torch.randn(rows, H).bfloat16(), (1 + 0.1 * torch.randn(H)).bfloat16(), torch.randn(rows, H).bfloat16()
         _, rstd = O.rms_norm(x, w, 1e-6)
