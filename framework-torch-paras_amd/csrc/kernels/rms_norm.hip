@@ -567,6 +567,151 @@ __global__ __launch_bounds__(BLOCK == 0 ? 1024 : BLOCK * kTeams, 4) void rms_nor
         }
 }
 
+// Rows of 8193 to 16384 elements, 16-bit tensors: two vectors per thread of a 1024-thread workgroup,
+// one workgroup per compute unit.  The registers of rms_norm_bwd_fused do not stretch to two
+// vectors (weights and column sums as doubles, the widened row, the row asked for ahead), so the
+// column sums live in LDS (128 KB: every thread adds into entries of its own, pairs of doubles 16
+// bytes apart from lane to lane), the weights stay 16-bit and are widened at use, and g and x are
+// widened twice, before and after the row's dot product is known.  Same arithmetic, same roundings.
+template <typename T>
+__global__ __launch_bounds__(1024, 4) void rms_norm_bwd_wide(
+    const std::uint16_t* __restrict__ go, const std::uint16_t* __restrict__ x, const std::uint16_t* __restrict__ w,
+    const float* __restrict__ rstd, std::uint16_t* __restrict__ gx, double* __restrict__ partial, long rows, int H) {
+    using E = Elem<T>;
+    typedef double f64x2 __attribute__((ext_vector_type(2)));
+    constexpr int V = 8, NV = 2, BLOCK = 1024, kWaves = BLOCK / kWave;
+    __shared__ f64x2 dw_lds[V / 2][NV * BLOCK];
+    __shared__ double slots[2 * kWaves];
+    const int tid = threadIdx.x;
+    const int nvec = H / V;
+    const double inv_h = 1.0 / static_cast<double>(H);
+    const bool h_pow2 = __builtin_amdgcn_readfirstlane((H & (H - 1)) == 0) != 0;
+    bool have[NV];
+    u32x4 wv[NV], gs[NV], xs[NV], gn[NV], xn[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = tid + i * BLOCK;
+        have[i] = c < nvec;
+        wv[i] = have[i] ? load16(w + static_cast<long>(c) * V) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int p = 0; p < V / 2; ++p) dw_lds[p][c] = f64x2{0.0, 0.0};
+    }
+    auto request = [&](long r, u32x4 (&g)[NV], u32x4 (&xx)[NV]) __attribute__((always_inline)) {
+        const std::uint16_t* gr = go + r * H;
+        const std::uint16_t* xr = x + r * H;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (have[i]) {
+                const unsigned at = static_cast<unsigned>(tid + i * BLOCK) * V;
+                g[i] = load16_nt(gr + at);
+                xx[i] = load16_nt(xr + at);
+            }
+    };
+    const long rstep = gridDim.x;
+    int sum_calls = 0;
+    float rstd_carry = 0.0f;
+    // One row from the register set (g, xx); the next row goes into the other set (gnext, xnext) as
+    // soon as this one has arrived.  Two elements at a time, in element order, each pair finished
+    // before the next is widened: all eight at once would not fit beside the row that is on its
+    // way.  For the same reason the compiler must not keep widened values from one half of the row
+    // to the other, or the widened weights from row to row: the packed registers are passed through
+    // empty asm statements, after which it has to widen again.
+    auto do_row = [&](long r, u32x4 (&g)[NV], u32x4 (&xx)[NV], u32x4 (&gnext)[NV], u32x4 (&xnext)[NV]) __attribute__((always_inline)) {
+        auto forget = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int p = 0; p < 4; ++p) asm volatile("" : "+v"(g[i][p]), "+v"(xx[i][p]), "+v"(wv[i][p]));
+        };
+        double dot = 0.0;
+        forget();                                            // waits for this row, so before the next one is asked for
+        asm volatile("" : "+v"(rstd_carry));
+        const double rr = static_cast<double>(rstd_carry);
+        if (r + rstep < rows) {
+            rstd_carry = rstd[r + rstep];                    // asked for with the row it belongs to
+            request(r + rstep, gnext, xnext);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (have[i]) {
+                const int c = tid + i * BLOCK;
+#pragma unroll
+                for (int p = 0; p < V / 2; ++p) {
+                    f64x2 d = dw_lds[p][c];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const std::uint32_t sh = 16 * h;
+                        const double gd = E::to_f64(static_cast<std::uint16_t>(g[i][p] >> sh));
+                        const double xd = E::to_f64(static_cast<std::uint16_t>(xx[i][p] >> sh));
+                        const double wd = E::to_f64(static_cast<std::uint16_t>(wv[i][p] >> sh));
+                        const double q = gd * xd;
+                        dot = fma(q, wd, dot);
+                        d[h] = fma(q, rr, d[h]);
+                    }
+                    dw_lds[p][c] = d;
+                    asm volatile("" : "+v"(dot) : : "memory");
+                }
+            }
+        {
+            dot = wave_sum(dot);
+            double* slot = slots + (sum_calls++ & 1) * kWaves;
+            if ((tid & (kWave - 1)) == 0) slot[tid / kWave] = dot;
+            lds_barrier();
+            dot = 0.0;
+#pragma unroll
+            for (int i = 0; i < kWaves; i += 4) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) dot += slot[i + u];
+                asm volatile("" : "+v"(dot) : : "memory");
+            }
+        }
+        const double cd = bwd_coef(rr, H, h_pow2, inv_h) * dot;
+        forget();
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (have[i]) {
+                float y[V];
+#pragma unroll
+                for (int p = 0; p < V / 2; ++p) {
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const std::uint32_t sh = 16 * h;
+                        const double gd = E::to_f64(static_cast<std::uint16_t>(g[i][p] >> sh));
+                        const double xd = E::to_f64(static_cast<std::uint16_t>(xx[i][p] >> sh));
+                        const double wd = E::to_f64(static_cast<std::uint16_t>(wv[i][p] >> sh));
+                        y[2 * p + h] = static_cast<float>(fma(gd * wd, rr, -(xd * cd)));
+                    }
+                    asm volatile("" : "+v"(y[2 * p]), "+v"(y[2 * p + 1]));
+                }
+                store16_nt(gx + r * H + static_cast<unsigned>(tid + i * BLOCK) * V, bwd_narrow_vec<T>(y));
+            }
+    };
+    long r = blockIdx.x;
+    if (r < rows) {
+        rstd_carry = rstd[r];
+        request(r, gs, xs);
+    }
+    while (r < rows) {
+        do_row(r, gs, xs, gn, xn);
+        r += rstep;
+        if (r >= rows) break;
+        do_row(r, gn, xn, gs, xs);
+        r += rstep;
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+        if (have[i]) {
+            const int c = tid + i * BLOCK;
+            double* dst = partial + static_cast<long>(blockIdx.x) * H + static_cast<long>(c) * V;
+#pragma unroll
+            for (int p = 0; p < V / 2; ++p) {
+                const f64x2 d = dw_lds[p][c];
+                dst[2 * p] = d[0];
+                dst[2 * p + 1] = d[1];
+            }
+        }
+}
+
 // Rows of at most 64 vectors (per-head norms: 128 elements), 16-bit tensors: TPR lanes per row,
 // 64 / TPR rows per wave, each lane group walking rows of its own with the next one requested
 // ahead; the row's dot product meets over its lanes by exchanges inside the wave, so the row loop
@@ -776,6 +921,22 @@ int launch_bwd(const void* go, const void* x, const void* w, const float* rstd, 
             PARAS_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + kDwFinalCols - 1) / kDwFinalCols)), dim3(kDwFinalLanes * kDwFinalCols), 0, s,
                                part, static_cast<S*>(gw), static_cast<long>(sgrid), H);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
+        if (aligned && nvec > 1024 && nvec <= 2048) {
+            int dev = 0;
+            (void)hipGetDevice(&dev);
+            auto* dst = DeviceContext::instance().device(dev);
+            const long cus = dst ? dst->compute_units : 256;
+            const unsigned wgrid = static_cast<unsigned>(slabs < cus ? slabs : cus);     // one partial sum each: the workspace has `slabs`
+            auto* part = static_cast<double*>(workspace);
+            hipLaunchKernelGGL((rms_norm_bwd_wide<T>), dim3(wgrid), dim3(1024), 0, s, static_cast<const std::uint16_t*>(go),
+                               static_cast<const std::uint16_t*>(x), static_cast<const std::uint16_t*>(w), rstd,
+                               static_cast<std::uint16_t*>(gx), part, rows, (int)H);
+            PARAS_HIP_TRY(hipGetLastError());
+            hipLaunchKernelGGL((rms_norm_bwd_dw_final_wide<T>), dim3(static_cast<unsigned>((H + kDwFinalCols - 1) / kDwFinalCols)), dim3(kDwFinalLanes * kDwFinalCols), 0, s,
+                               part, static_cast<S*>(gw), static_cast<long>(wgrid), H);
             PARAS_HIP_TRY(hipGetLastError());
             return PARAS_OK;
         }

@@ -146,10 +146,12 @@ def test_full_size_rms_norm_and_swiglu_bf16():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(70, 4096), (33, 2048), (16, 520), (300, 1024), (5, 8), (37, 8192), (20, 5120), (9, 8200),
                                    (45, 6144), (50, 3072), (130, 1536), (70, 512), (31, 7168), (25, 2880),
-                                   (1000, 128), (37, 64), (100, 96), (3, 256), (515, 512), (1, 128), (70000, 128)])
+                                   (1000, 128), (37, 64), (100, 96), (3, 256), (515, 512), (1, 128), (70000, 128),
+                                   (6, 16384), (5, 12288), (300, 9216), (40, 16376)])
 def test_rms_norm_backward_one_pass_kernel(shape, dtype):
-    """Row sizes the one-pass backward kernel takes (16-byte aligned rows of up to 8192 elements; the
-    last shape is beyond it), with slabs of rows that are full, ragged and single."""
+    """Row sizes the one-pass backward kernels take (16-byte aligned rows: several rows per wave up
+    to 512 elements, a vector per thread up to 8192, two with the column sums in LDS up to 16384),
+    with slabs of rows that are full, ragged and single."""
     rows, H = shape
     torch.manual_seed(rows + H)
     x, w, go = torch.randn(rows, H).to(dtype), (1 + 0.1 * torch.randn(H)).to(dtype), torch.randn(rows, H).to(dtype)
@@ -164,7 +166,7 @@ def test_rms_norm_backward_many_rows_are_dealt_round_robin():
     """The one-pass kernel runs at most two workgroups per compute unit; with more rows than that
     times 16 every workgroup takes rows b, b + G, b + 2G, ...: row counts around the switch, with
     workgroups that get one row more than others."""
-    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520), (8192 + 7, 264), (4200, 5120), (9001, 3072), (4100, 8192)):
+    for rows, H in ((16384 + 32 + 5, 264), (16383, 264), (16384, 520), (8192 + 7, 264), (4200, 5120), (9001, 3072), (4100, 8192), (4200, 8200), (2100, 12288)):
         torch.manual_seed(rows)
         x, w, go = torch.randn(rows, H).bfloat16(), (1 + 0.1 * torch.randn(H)).bfloat16(), torch.randn(rows, H).bfloat16()
         _, rstd = O.rms_norm(x, w, 1e-6)
