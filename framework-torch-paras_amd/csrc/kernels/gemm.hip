@@ -113,6 +113,45 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
     }
     std::uint16_t* C = p.c + bidx * p.sc;
     const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
+    // The plain product (alpha = 1, nothing added) of a tile whose byte offsets fit 32 bits: one
+    // uniform base, a 32-bit offset per lane, rows and columns checked against counts in 32-bit
+    // registers, and the conversion instruction for the narrowing; a 32 x 32 block in which a NaN
+    // turns up is narrowed again in software, which writes NaNs as the host's types do.
+    if (p.alpha == 1.0f && ADD == nullptr && p.ldc < (1L << 22)) {
+        std::uint16_t* cb = C + row0 * p.ldc + n0;                       // uniform
+        const long rows_left = p.M - row0, cols_left = p.N - n0;
+        const int nrows = static_cast<int>(rows_left < S::kBM ? rows_left : S::kBM) - (wm * 64 + 4 * lh);
+        const int ncols = static_cast<int>(cols_left < G * kBN ? cols_left : G * kBN) - (wn * 64 + lr);
+        const unsigned ldc2 = static_cast<unsigned>(p.ldc) * 2u;
+        const unsigned lane_b = static_cast<unsigned>(wm * 64 + 4 * lh) * ldc2 + static_cast<unsigned>(wn * 64 + lr) * 2u;
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni) {
+                    if (g * kBN + ni * 32 >= ncols) continue;
+                    std::uint16_t o[16];
+                    float probe = 0.0f;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        o[r] = El::from_f32_finite(acc[g][mi][ni][r]);
+                        probe += acc[g][mi][ni][r];
+                    }
+                    if (__builtin_amdgcn_ballot_w64(probe != probe) != 0) {
+                        asm volatile("" ::: "memory");
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o[r] = El::from_f32(acc[g][mi][ni][r]);
+                    }
+                    char* blk = reinterpret_cast<char*>(cb) + (g * kBN + ni * 32) * 2;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
+                        if (ro < nrows) *reinterpret_cast<std::uint16_t*>(blk + (lane_b + static_cast<unsigned>(ro) * ldc2)) = o[r];
+                    }
+                }
+        return;
+    }
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll

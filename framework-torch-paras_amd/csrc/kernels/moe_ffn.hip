@@ -128,7 +128,7 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
                 const long prow = row0 + (wave >> 2) * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
                 if (prow >= row_end) continue;
                 if (kSwiglu) {
-                    if (col < p.N) p.c[prow * p.N + col] = swiglu_one<T>(El::from_f32(sacc[0][r]), El::from_f32(sacc[1][r]));
+                    if (col < p.N) p.c[prow * p.N + col] = swiglu_from_acc<T>(sacc[0][r], sacc[1][r]);
                 } else {
                     if (col < p.N) p.c[prow * p.N + col] = El::from_f32(sacc[0][r]);
                     if (col + kBN < p.N) p.c[prow * p.N + col + kBN] = El::from_f32(sacc[1][r]);
@@ -141,27 +141,56 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
     S::template mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, acc);
 
     // ---- epilogue.  Accumulator lane (column lr, half lh) holds rows (r/4)*8 + 4*lh + r%4.
+    // One uniform base, a 32-bit byte offset per lane (the launcher sends output rows of 2^22
+    // elements or more elsewhere), rows and columns checked against counts in 32-bit registers,
+    // narrowing by the conversion instruction; a 32 x 32 block of the plain product in which a NaN
+    // turns up is narrowed again in software, which writes NaNs as the host's types do.
+    {
+        char* cb = reinterpret_cast<char*>(p.c + row0 * p.N + n0);       // uniform
+        const long rows_left = row_end - row0, cols_left = p.N - n0;
+        const int nrows = static_cast<int>(rows_left < kBM ? rows_left : kBM) - (wm * 64 + 4 * lh);
+        const int ncols = static_cast<int>(cols_left < 2 * kBN ? cols_left : 2 * kBN) - (wn * 64 + lr);
+        const unsigned ld2 = static_cast<unsigned>(p.N) * 2u;
+        const unsigned lane_b = static_cast<unsigned>(wm * 64 + 4 * lh) * ld2 + static_cast<unsigned>(wn * 64 + lr) * 2u;
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+        for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const long col = n0 + wn * 64 + ni * 32 + lr;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const long prow = row0 + wm * 64 + mi * 32 + (r >> 2) * 8 + 4 * lh + (r & 3);
-                if (prow >= row_end) continue;
+            for (int ni = 0; ni < 2; ++ni) {
                 if (kSwiglu) {
-                    if (col < p.N) {
-                        const auto g = El::from_f32(acc[0][mi][ni][r]);
-                        const auto u = El::from_f32(acc[1][mi][ni][r]);
-                        p.c[prow * p.N + col] = swiglu_one<T>(g, u);
+                    if (ni * 32 >= ncols) continue;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
+                        if (ro < nrows)
+                            *reinterpret_cast<std::uint16_t*>(cb + ni * 64 + (lane_b + static_cast<unsigned>(ro) * ld2)) =
+                                swiglu_from_acc<T>(acc[0][mi][ni][r], acc[1][mi][ni][r]);
                     }
                 } else {
-                    if (col < p.N) p.c[prow * p.N + col] = El::from_f32(acc[0][mi][ni][r]);
-                    if (col + kBN < p.N) p.c[prow * p.N + col + kBN] = El::from_f32(acc[1][mi][ni][r]);
+#pragma unroll
+                    for (int g = 0; g < 2; ++g) {
+                        if (g * kBN + ni * 32 >= ncols) continue;
+                        std::uint16_t o[16];
+                        float probe = 0.0f;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            o[r] = El::from_f32_finite(acc[g][mi][ni][r]);
+                            probe += acc[g][mi][ni][r];
+                        }
+                        if (__builtin_amdgcn_ballot_w64(probe != probe) != 0) {
+                            asm volatile("" ::: "memory");
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) o[r] = El::from_f32(acc[g][mi][ni][r]);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
+                            if (ro < nrows)
+                                *reinterpret_cast<std::uint16_t*>(cb + (g * kBN + ni * 32) * 2 + (lane_b + static_cast<unsigned>(ro) * ld2)) = o[r];
+                        }
+                    }
                 }
             }
-        }
+    }
 }
 
 // out[t, :] = T( sum_slot T( y[inv[t*k+slot], :] * T(w[t, slot]) ) ), 8 columns per lane.
@@ -378,7 +407,7 @@ int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up, const voi
     // tensors; anything else goes to the general kernels (any size, any alignment).
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w_gate) | reinterpret_cast<uintptr_t>(w_up) |
                            reinterpret_cast<uintptr_t>(w_down) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0;
-    const bool tiles = H % kBK == 0 && I % kBK == 0 && aligned;
+    const bool tiles = H % kBK == 0 && I % kBK == 0 && aligned && H < (1LL << 22) && I < (1LL << 22);   // (the tiles' stores use 32-bit byte offsets within a tile)
     PARAS_REQUIRE(T * k <= 0x3fffffffLL, "paras_moe_ffn: too many routed rows");
     if (T * H >= (1LL << 32) || T * k * I >= (1LL << 32) || I * H >= (1LL << 32))
         return fail(PARAS_ERR_UNSUPPORTED, "paras_moe_ffn: an operand (x, the routed intermediate, or one expert's weight matrix) spans 2^32 elements or more");

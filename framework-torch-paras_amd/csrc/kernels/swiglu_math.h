@@ -86,6 +86,23 @@ __device__ __forceinline__ typename Elem<T>::store_t swiglu_one(typename Elem<T>
     }
 }
 
+// SwiGLU of two fp32 accumulators (a GEMM epilogue): T(silu(T(a0)) * T(a1)) with the narrowing
+// of a0 and a1 done by the conversion instruction on the common path.  That instruction differs
+// from the host's narrowing for NaNs only, a NaN gate or up value makes y a NaN, and a NaN y fails
+// the range test: whatever does not pass goes through swiglu_one on the software-narrowed values.
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::store_t swiglu_from_acc(float a0, float a1) {
+    using E = Elem<T>;
+    static_assert(sizeof(typename E::store_t) == 2, "16-bit dtypes only");
+    const float g = E::to_f32(E::from_f32_finite(a0));
+    const float u = E::to_f32(E::from_f32_finite(a1));
+    const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
+    const float y = g * __builtin_amdgcn_rcpf(1.0f + e) * u;
+    const bool ok = narrow_is_safe<T>(y, kSwigluUlps) && (fabsf(g - 26.0f) <= 34.0f);
+    if (__builtin_expect(ok, 1)) return E::from_f32_finite(y);
+    return swiglu_one<T>(E::from_f32(a0), E::from_f32(a1));
+}
+
 // ---- SwiGLU backward -----------------------------------------------------------
 // Host definition (csrc/ops/fused_ops.cpp:218-226), in fp64:
 //   s = 1/(1+exp(-g));  dup = (dy*g)*s;  dgate = (dy*u) * (s * (1 + g*(1-s)))
