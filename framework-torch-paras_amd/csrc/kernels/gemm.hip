@@ -123,7 +123,9 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
         const int nrows = static_cast<int>(rows_left < S::kBM ? rows_left : S::kBM) - (wm * 64 + 4 * lh);
         const int ncols = static_cast<int>(cols_left < G * kBN ? cols_left : G * kBN) - (wn * 64 + lr);
         const unsigned ldc2 = static_cast<unsigned>(p.ldc) * 2u;
-        const unsigned lane_b = static_cast<unsigned>(wm * 64 + 4 * lh) * ldc2 + static_cast<unsigned>(wn * 64 + lr) * 2u;
+        unsigned lane_b = static_cast<unsigned>(wm * 64 + 4 * lh) * ldc2 + static_cast<unsigned>(wn * 64 + lr) * 2u;
+        asm volatile("" : "+v"(lane_b));       // one add per store from here on (not a 64-bit multiply-add per element)
+        const bool full = rows_left >= S::kBM && cols_left >= G * kBN;    // uniform
 #pragma unroll
         for (int g = 0; g < G; ++g)
 #pragma unroll
@@ -132,23 +134,10 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
                 for (int ni = 0; ni < 2; ++ni) {
                     if (g * kBN + ni * 32 >= ncols) continue;
                     std::uint16_t o[16];
-                    float probe = 0.0f;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        o[r] = El::from_f32_finite(acc[g][mi][ni][r]);
-                        probe += acc[g][mi][ni][r];
-                    }
-                    if (__builtin_amdgcn_ballot_w64(probe != probe) != 0) {
-                        asm volatile("" ::: "memory");
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) o[r] = El::from_f32(acc[g][mi][ni][r]);
-                    }
+                    narrow_block<T>(acc[g][mi][ni], o);
                     char* blk = reinterpret_cast<char*>(cb) + (g * kBN + ni * 32) * 2;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
-                        if (ro < nrows) *reinterpret_cast<std::uint16_t*>(blk + (lane_b + static_cast<unsigned>(ro) * ldc2)) = o[r];
-                    }
+                    if (full) store_block<true>(blk, lane_b, ldc2, mi, nrows, o);
+                    else      store_block<false>(blk, lane_b, ldc2, mi, nrows, o);
                 }
         return;
     }

@@ -315,6 +315,36 @@ __device__ __forceinline__ void short_tile_mainloop(const std::uint16_t* a_base,
 
 }  // namespace wide
 
+// ---- epilogue helpers.  A lane (column lr, half lh) of a 32 x 32 accumulator block holds rows
+// (r/4)*8 + 4*lh + r%4, r = 0..15.  Stores go to `blk` (the block's first column in the tile's first
+// row: the same address in every lane, so it stays in scalar registers) plus a 32-bit byte offset:
+// `lane_b` (this lane's first row and column) plus a row offset that is again the same in every lane.
+// kFull: the whole tile lies inside the matrix, no row is tested.
+template <bool kFull>
+__device__ __forceinline__ void store_block(char* blk, unsigned lane_b, unsigned ld2, int mi, int nrows, const std::uint16_t (&o)[16]) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
+        if (kFull || ro < nrows) *reinterpret_cast<std::uint16_t*>(blk + (lane_b + static_cast<unsigned>(ro) * ld2)) = o[r];
+    }
+}
+// Narrows a block of plain results: the conversion instruction, and once more in software (which
+// writes NaNs as the host's types do) if a NaN turns up anywhere in the wave's block.
+template <typename T>
+__device__ __forceinline__ void narrow_block(const float16_t& a, std::uint16_t (&o)[16]) {
+    float probe = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        o[r] = Elem<T>::from_f32_finite(a[r]);
+        probe += a[r];
+    }
+    if (__builtin_amdgcn_ballot_w64(probe != probe) != 0) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[r] = Elem<T>::from_f32(a[r]);
+    }
+}
+
 // The two tile shapes as a kernel sees them.
 template <int G>
 struct Tile128G {

@@ -151,42 +151,29 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
         const int nrows = static_cast<int>(rows_left < kBM ? rows_left : kBM) - (wm * 64 + 4 * lh);
         const int ncols = static_cast<int>(cols_left < 2 * kBN ? cols_left : 2 * kBN) - (wn * 64 + lr);
         const unsigned ld2 = static_cast<unsigned>(p.N) * 2u;
-        const unsigned lane_b = static_cast<unsigned>(wm * 64 + 4 * lh) * ld2 + static_cast<unsigned>(wn * 64 + lr) * 2u;
+        unsigned lane_b = static_cast<unsigned>(wm * 64 + 4 * lh) * ld2 + static_cast<unsigned>(wn * 64 + lr) * 2u;
+        asm volatile("" : "+v"(lane_b));       // one add per store from here on
+        const bool full = rows_left >= kBM && cols_left >= (kSwiglu ? kBN : 2 * kBN);    // uniform
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni) {
                 if (kSwiglu) {
                     if (ni * 32 >= ncols) continue;
+                    std::uint16_t o[16];
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
-                        if (ro < nrows)
-                            *reinterpret_cast<std::uint16_t*>(cb + ni * 64 + (lane_b + static_cast<unsigned>(ro) * ld2)) =
-                                swiglu_from_acc<T>(acc[0][mi][ni][r], acc[1][mi][ni][r]);
-                    }
+                    for (int r = 0; r < 16; ++r) o[r] = swiglu_from_acc<T>(acc[0][mi][ni][r], acc[1][mi][ni][r]);
+                    if (full) store_block<true>(cb + ni * 64, lane_b, ld2, mi, nrows, o);
+                    else      store_block<false>(cb + ni * 64, lane_b, ld2, mi, nrows, o);
                 } else {
 #pragma unroll
                     for (int g = 0; g < 2; ++g) {
                         if (g * kBN + ni * 32 >= ncols) continue;
                         std::uint16_t o[16];
-                        float probe = 0.0f;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            o[r] = El::from_f32_finite(acc[g][mi][ni][r]);
-                            probe += acc[g][mi][ni][r];
-                        }
-                        if (__builtin_amdgcn_ballot_w64(probe != probe) != 0) {
-                            asm volatile("" ::: "memory");
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) o[r] = El::from_f32(acc[g][mi][ni][r]);
-                        }
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int ro = mi * 32 + (r >> 2) * 8 + (r & 3);
-                            if (ro < nrows)
-                                *reinterpret_cast<std::uint16_t*>(cb + (g * kBN + ni * 32) * 2 + (lane_b + static_cast<unsigned>(ro) * ld2)) = o[r];
-                        }
+                        narrow_block<T>(acc[g][mi][ni], o);
+                        char* blk = cb + (g * kBN + ni * 32) * 2;
+                        if (full) store_block<true>(blk, lane_b, ld2, mi, nrows, o);
+                        else      store_block<false>(blk, lane_b, ld2, mi, nrows, o);
                     }
                 }
             }
