@@ -49,7 +49,18 @@ struct FfnGemmParams {
     int mt_total;               // upper bound on m-tiles
     int n_units;                // column units (128 output columns for GEMM 1, 256 for GEMM 2)
     int ngt;                    // column units an XCD sweeps together
+    unsigned div_m;             // flat (token, slot) index / k as a multiplication: (x * div_m) >> div_s
+    int div_s;                  // for every x < 2^30 (a 64-bit division per gathered row is ~150 instructions)
 };
+
+// Multiplier and shift with floor(x / d) == (x * m) >> s for all 0 <= x < 2^30, 1 <= d < 2^30:
+// s = 30 + ceil(log2 d), m = ceil(2^s / d) < 2^31; the error x * (m d - 2^s) stays below 2^s.
+inline void division_by(unsigned d, unsigned* m, int* s) {
+    int lg = 0;
+    while ((1ull << lg) < d) ++lg;
+    *s = 30 + lg;
+    *m = static_cast<unsigned>(((1ull << *s) + d - 1) / d);
+}
 
 template <typename T, bool kSwiglu, typename S>
 __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnGemmParams p) {
@@ -102,7 +113,7 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
         const int c = tid + i * S::kThreads;
         long prow = row0 + (c >> 3);
         if (prow >= row_end) prow = row_end - 1;  // clamp: result rows beyond the expert are not stored
-        const long src = p.order ? p.order[prow] / p.k : prow;
+        const long src = p.order ? static_cast<long>((static_cast<unsigned long long>(static_cast<unsigned>(p.order[prow])) * p.div_m) >> p.div_s) : prow;
         a_off[i] = static_cast<unsigned>(src * p.K + (c & 7) * 8);
     }
     // weights of this expert: a uniform base per column group, rows as 32-bit offsets
@@ -316,6 +327,7 @@ int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const voi
     g1.offsets = offsets;
     g1.K = H; g1.N = I; g1.Nw = I; g1.R = R; g1.E = E; g1.k = k;
     g1.mt_total = mt_total;
+    division_by(static_cast<unsigned>(k), &g1.div_m, &g1.div_s);
     g1.n_units = static_cast<int>((I + kBN - 1) / kBN);
     // Column units an XCD sweeps together: up to 2 (one expert's weight panel for them is
     // 4 MB at K = 4096, the size of an XCD's L2; 4 units measured 8 % slower), fewer when
