@@ -162,6 +162,30 @@ def test_rms_norm_backward_one_pass_kernel(shape, dtype):
     assert_bit_exact(gw, wgw, "rms_norm grad_weight")
 
 
+def test_rms_norm_forward_and_backward_random_shapes():
+    """Forty random (rows, H) pairs over every row-length path of both directions (several rows per
+    wave, one workgroup per row, walking workgroups, one or two vectors per thread, the scalar
+    kernels for rows that are not whole 16-byte vectors), both 16-bit dtypes: bit-exact."""
+    gen = torch.Generator().manual_seed(2024)
+    widths = [8, 24, 64, 120, 128, 136, 256, 384, 512, 520, 1000, 1024, 1536, 2048, 2880, 3072, 4096, 4104, 5120, 6144, 7168, 8192,
+              8200, 9216, 12288, 16384, 16392, 20480, 100, 130, 4097]
+    for trial in range(40):
+        H = widths[int(torch.randint(len(widths), (1,), generator=gen))]
+        rows = int(torch.randint(1, max(2, min(3000, 600000 // H)), (1,), generator=gen))
+        dtype = (torch.bfloat16, torch.float16)[trial % 2]
+        x = torch.randn(rows, H, generator=gen).to(dtype)
+        w = (1 + 0.1 * torch.randn(H, generator=gen)).to(dtype)
+        go = torch.randn(rows, H, generator=gen).to(dtype)
+        out, rstd = capi.rms_norm(dev(x), dev(w), 1e-6)
+        wout, wrstd = O.rms_norm(x, w, 1e-6)
+        assert_bit_exact(out, wout, f"rms_norm out {rows}x{H} {dtype}")
+        assert_bit_exact(rstd, wrstd, f"rms_norm rstd {rows}x{H} {dtype}")
+        gx, gw = capi.rms_norm_backward(dev(go), dev(x), dev(w), dev(wrstd))
+        wgx, wgw = O.rms_norm_backward(go, x, w, wrstd)
+        assert_bit_exact(gx, wgx, f"rms_norm grad_input {rows}x{H} {dtype}")
+        assert_bit_exact(gw, wgw, f"rms_norm grad_weight {rows}x{H} {dtype}")
+
+
 def test_rms_norm_backward_many_rows_are_dealt_round_robin():
     """The one-pass kernel runs at most two workgroups per compute unit; with more rows than that
     times 16 every workgroup takes rows b, b + G, b + 2G, ...: row counts around the switch, with
