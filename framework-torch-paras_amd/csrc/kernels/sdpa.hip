@@ -12,7 +12,7 @@
 namespace paras {
 namespace {
 
-enum class SdpaKernel { Flash, Decode, Weights, Padded, Generic };
+enum class SdpaKernel { Flash, Decode, Weights, Padded, Composed, Generic };
 
 int validate(const paras_sdpa_args* a) {
     PARAS_REQUIRE(a != nullptr, "paras sdpa: null argument block");
@@ -78,6 +78,7 @@ SdpaKernel choose(const paras_sdpa_args& a) {
     if (flash_supported(a)) return SdpaKernel::Flash;
     if (weights_supported(a)) return SdpaKernel::Weights;
     if (plan_padded(a, nullptr)) return SdpaKernel::Padded;
+    if (composed_supported(a)) return SdpaKernel::Composed;
     return SdpaKernel::Generic;
 }
 
@@ -122,6 +123,7 @@ const char* paras_sdpa_kernel_name(const paras_sdpa_args* args) {
         case SdpaKernel::Decode: return "decode_split";
         case SdpaKernel::Weights: return "math_mfma";
         case SdpaKernel::Padded: return "padded_mfma";
+        case SdpaKernel::Composed: return "composed";
         default:                 return "generic";
     }
 }
@@ -132,6 +134,7 @@ size_t paras_sdpa_workspace(const paras_sdpa_args* args) {
     switch (choose(*args)) {
         case SdpaKernel::Decode:  return decode_workspace(*args);
         case SdpaKernel::Generic: return generic_workspace(*args);
+        case SdpaKernel::Composed: return composed_workspace(*args);
         case SdpaKernel::Padded: {
             PaddedPlan pl;
             return plan_padded(*args, &pl) ? pl.total : 0;
@@ -162,6 +165,7 @@ int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream) {
         case SdpaKernel::Flash: return launch_flash(a, s);
         case SdpaKernel::Weights: return launch_weights(a, s);
         case SdpaKernel::Padded: return launch_padded(a, workspace, stream, s);
+        case SdpaKernel::Composed: return launch_composed(a, workspace, stream, s);
         case SdpaKernel::Decode:
             PARAS_REQUIRE(workspace != nullptr || decode_workspace(a) == 0, "paras sdpa: workspace is null");
             return launch_decode(a, workspace, s);

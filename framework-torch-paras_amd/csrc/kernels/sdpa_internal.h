@@ -24,6 +24,13 @@ int    launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s);
 bool weights_supported(const paras_sdpa_args& a);
 int  launch_weights(const paras_sdpa_args& a, hipStream_t s);
 
+// The reference's composition run step by step with the library's own batched products and one
+// row kernel (fp32 / fp64 tensors, head sizes and layouts the fused kernels do not take), for
+// problems big enough that the general kernel would take milliseconds.
+bool   composed_supported(const paras_sdpa_args& a);
+size_t composed_workspace(const paras_sdpa_args& a);
+int    launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hipStream_t s);
+
 // Everything else (fp32/fp64, any head size, other layouts).
 size_t generic_workspace(const paras_sdpa_args& a);
 int    launch_generic(const paras_sdpa_args& a, void* workspace, hipStream_t s);

@@ -239,7 +239,11 @@ PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void*
  * "math_mfma" (bf16 / f16 with the weights returned), "padded_mfma" (bf16 / f16
  * head sizes below 128 other than 64: q, k, v copied into the workspace with
  * zero columns up to 64 or 128, then flash_mfma / decode_split; the workspace
- * must be 256-byte aligned) or "generic". */
+ * must be 256-byte aligned), "composed" (what none of these takes, from about
+ * 5e8 multiply-adds on: the reference's own composition,
+ * csrc/ops/attention_ops.cpp:101-135, run as two batched paras_gemm_nt products
+ * around one scale / mask / softmax row kernel, scores in `attn` or in the
+ * 256-byte aligned workspace, a bounded piece at a time) or "generic". */
 PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 
 /* ------------------------------------------------------------------------- */

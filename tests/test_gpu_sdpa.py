@@ -531,3 +531,73 @@ def test_head_sizes_between_the_mfma_kernels_are_padded_inside_the_library(case_
     assert name == "padded_mfma" and out.shape == (B, Hq, Lq, D)
     assert max_abs(out, want) <= ABS_16BIT
     assert bool(torch.isfinite(lse).all())
+
+
+# ---- the composed route: batched products + one row kernel, for large problems no fused kernel takes ----
+
+def _composed_case(dtype, B, Hq, Hkv, Lq, Lk, D, Dv=None, **kw):
+    Dv = Dv or D
+    q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, Dv).to(dtype)
+    return q, k, v
+
+
+def test_composed_route_fp32_causal_with_weights_and_lse():
+    """fp32 at a size where the general kernel would take tens of milliseconds: the reference's
+    composition run with the library's own products; outputs, weights and log-sum-exp."""
+    torch.manual_seed(3)
+    q, k, v = _composed_case(torch.float32, 2, 8, 8, 1024, 1024, 64)
+    out, attn, lse, name = run(q, k, v, is_causal=True, want_attn=True, want_lse=True)
+    assert name == "composed"
+    want, wattn = O.sdpa_math(q, k, v, is_causal=True, gemm="aten")
+    assert rel_err(out, want) <= REL_F32 and rel_err(attn, wattn) <= REL_F32
+    assert float(attn.cpu().triu(1).abs().max()) == 0.0
+    ref_lse = torch.logsumexp((q @ k.transpose(-1, -2) * 0.125).masked_fill(~torch.ones(1024, 1024).tril().bool(), -math.inf), -1)
+    assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-5, atol=1e-5)
+    out2, _, _, _ = run(q, k, v, is_causal=True)              # scores in the workspace instead of the weights tensor
+    assert torch.equal(out2.cpu(), out.cpu())
+
+
+@pytest.mark.parametrize("cap", [None, 3 * 512 * 1024, 100 * 1024])
+def test_composed_route_gqa_masks_and_pieces(cap, monkeypatch):
+    """Grouped heads (the q heads of a kv head share its keys), a broadcast bool mask and an
+    additive one, Lq != Lk, Dv != D; with the score bound lowered the same problem runs a few heads
+    at a time and in blocks of query rows."""
+    if cap is not None:
+        monkeypatch.setenv("PARAS_SDPA_SCORE_CAP", str(cap))
+    torch.manual_seed(4)
+    q, k, v = _composed_case(torch.float32, 2, 8, 2, 512, 1024, 64, Dv=96)
+    mask = torch.rand(2, 1, 512, 1024) > 0.3
+    mask[0, 0, 7] = False                                     # a query that sees no key: NaN like the reference
+    out, attn, _, name = run(q, k, v, mask=mask, want_attn=True)
+    assert name == "composed"
+    want, wattn = O.sdpa_math(q, k, v, attn_mask=mask, enable_gqa=True, gemm="aten")
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(out.cpu()), nan) and bool(nan[0, :, 7].all())
+    assert rel_err(torch.nan_to_num(out.cpu()), torch.nan_to_num(want)) <= REL_F32
+    assert rel_err(torch.nan_to_num(attn.cpu()), torch.nan_to_num(wattn)) <= REL_F32
+    bias = torch.randn(1, 8, 512, 1024)
+    out, _, _, name = run(q, k, v, mask=bias)
+    assert name == "composed"
+    want, _ = O.sdpa_math(q, k, v, attn_mask=bias, enable_gqa=True, gemm="aten")
+    assert rel_err(out, want) <= REL_F32
+    # one q head per kv head: several heads per piece
+    q1, k1, v1 = _composed_case(torch.float32, 2, 6, 6, 640, 768, 80)
+    out, _, _, name = run(q1, k1, v1, is_causal=True)
+    assert name == "composed"
+    want, _ = O.sdpa_math(q1, k1, v1, is_causal=True, gemm="aten")
+    assert rel_err(out, want) <= REL_F32
+
+
+def test_composed_route_fp64_and_wide_16_bit_heads():
+    torch.manual_seed(5)
+    q, k, v = _composed_case(torch.float64, 1, 4, 4, 2048, 2048, 32)
+    out, _, _, name = run(q, k, v)
+    assert name == "composed"
+    want, _ = O.sdpa_math(q, k, v, gemm="aten")
+    assert rel_err(out, want) <= 1e-12
+    # bf16 with a head size no MFMA attention kernel has: the products still run on the matrix cores
+    q, k, v = _composed_case(torch.bfloat16, 1, 4, 4, 1024, 1024, 256)
+    out, attn, _, name = run(q, k, v, is_causal=True, want_attn=True)
+    assert name == "composed"
+    want, wattn = O.sdpa_math(q, k, v, is_causal=True, gemm="aten")
+    assert max_abs(out, want) <= ABS_16BIT and max_abs(attn, wattn) <= ABS_16BIT
