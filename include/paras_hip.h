@@ -329,9 +329,11 @@ PARAS_API int paras_moe_ffn(const void* x, const void* w_gate, const void* w_up,
 /* elements (0 = shared).  addend may be NULL; ld_add = 0 broadcasts one row   */
 /* (a bias) over the M rows.  All four float dtypes.  bf16 / f16 with K a       */
 /* multiple of 64 and 16-byte aligned operand rows run on the MFMA kernels     */
-/* (fp32 accumulation, one rounding); everything else -- fp32 / fp64 tensors,  */
-/* other K, other alignments -- on a general kernel (fp32 accumulation, fp64   */
-/* for fp64 tensors), so no product needs a host path.                         */
+/* (fp32 accumulation, one rounding); fp32 tensors with at least 32 tiles of   */
+/* 128 x 128 outputs on the fp32 MFMA kernel (full fp32 multiplies, any K and  */
+/* alignment); everything else -- fp64 tensors, small fp32 products, 16-bit    */
+/* ones with other K or alignments -- on a general kernel (fp32 accumulation,  */
+/* fp64 for fp64 tensors), so no product needs a host path.                    */
 /* ------------------------------------------------------------------------- */
 PARAS_API int paras_gemm_nt(const void* a, const void* b, const void* addend, void* c,
                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,

@@ -110,6 +110,31 @@ def test_gemm_nt_general_kernel(dtype):
         assert_gemm_close(capi.gemm_nt(a, b), O.matmul_nt(a.cpu(), b.cpu()), dtype)
 
 
+def test_gemm_nt_fp32_on_the_matrix_cores():
+    """fp32 products with enough outputs for 128 x 128 tiles run on v_mfma_f32_32x32x2_f32 (full
+    fp32 multiplies): ragged M, N, K, rows that are not 16-byte aligned (scalar staging), a batch
+    with a shared weight, alpha / beta with a bias and with a full addend; 1e-5 against fp64."""
+    torch.manual_seed(21)
+    def close(got, want):
+        scale = want.abs().max().item()
+        assert (got.double().cpu() - want).abs().max().item() <= 1e-5 * scale
+    for (M, N, K) in [(1024, 1024, 512), (1000, 777, 333), (130, 4100, 17), (4096, 640, 2048)]:
+        a, b = torch.randn(M, K), torch.randn(N, K) / math.sqrt(K)
+        close(capi.gemm_nt(a.cuda(), b.cuda()), a.double() @ b.double().t())
+    a, b = torch.randn(700, 259), torch.randn(900, 259)                       # K odd: no 16-byte loads
+    bias, full = torch.randn(900), torch.randn(700, 900)
+    close(capi.gemm_nt(a.cuda(), b.cuda(), bias.cuda(), alpha=0.5, beta=2.0), 0.5 * (a.double() @ b.double().t()) + 2.0 * bias.double())
+    close(capi.gemm_nt(a.cuda(), b.cuda(), full.cuda(), alpha=-1.25, beta=0.75), -1.25 * (a.double() @ b.double().t()) + 0.75 * full.double())
+    buf = torch.randn(512 * 260 + 1).cuda()                                    # rows 4 bytes off 16-byte alignment
+    av = buf[1:].view(512, 260)[:, :256]
+    bw = torch.randn(640, 256)
+    close(capi.gemm_nt(av, bw.cuda()), av.cpu().double() @ bw.double().t())
+    a3, b2 = torch.randn(6, 300, 128), torch.randn(512, 128)                   # batched activations, one weight
+    close(capi.gemm_nt(a3.cuda(), b2.cuda()), a3.double() @ b2.double().t())
+    a3, b3 = torch.randn(5, 256, 96), torch.randn(5, 384, 96)                  # a weight per batch entry
+    close(capi.gemm_nt(a3.cuda(), b3.cuda()), a3.double() @ b3.double().transpose(1, 2))
+
+
 def test_gemm_nt_linearity_at_projection_size():
     """Size-independent property at a transformer projection shape: (2 a) W^T == 2 (a W^T) bit for
     bit, since scaling by a power of two commutes with every rounding; plus sampled rows vs the oracle."""
