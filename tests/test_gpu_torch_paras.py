@@ -75,6 +75,20 @@ def test_sdpa_causal(device):
                  F.scaled_dot_product_attention(q, k, v, is_causal=True), "causal")
 
 
+def test_sdpa_fp32_at_a_size_that_runs_composed(device):
+    """fp32 (the reference's default dtype) at a thousand tokens: batched products and one row kernel
+    inside the library, workspace from the device pool; also through the math op with its weights."""
+    q, k, v, dq, dk, dv = _qkv(device, B=1, H=8, Lq=1024, Lk=1024, E=64)
+    assert_close(F.scaled_dot_product_attention(dq, dk, dv, is_causal=True),
+                 F.scaled_dot_product_attention(q, k, v, is_causal=True), "fp32 causal, 1024 tokens")
+    out, attn = torch.ops.aten._scaled_dot_product_attention_math(dq, dk, dv, is_causal=True)
+    want, wattn = torch.ops.aten._scaled_dot_product_attention_math(q, k, v, is_causal=True)
+    assert_close(out, want, "math op out")
+    assert_close(attn, wattn, "math op weights")
+    x, w = torch.randn(1024, 768), torch.randn(1536, 768) / 28.0          # an fp32 projection on the matrix cores
+    assert_close(F.linear(x.to(device), w.to(device)), F.linear(x, w), "fp32 linear")
+
+
 def test_sdpa_causal_unequal_lengths(device):
     q, k, v, dq, dk, dv = _qkv(device, Lq=4, Lk=8)
     assert_close(F.scaled_dot_product_attention(dq, dk, dv, is_causal=True),
