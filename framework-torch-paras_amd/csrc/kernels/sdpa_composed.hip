@@ -96,9 +96,10 @@ __global__ __launch_bounds__(kBlock) void scale_mask_softmax_rows_kernel(const R
     __shared__ double slots[kWaves];
     for (long r = blockIdx.x; r < p.heads * p.rows; r += gridDim.x) {
         const long hh = r / p.rows, ri = r % p.rows;
-        const long h = p.h0 + hh, i = p.i0 + ri;
+        const long hg = p.h0 + hh, i = p.i0 + ri;                    // hg counts on through the batches when they are taken together
+        const long b = p.b + hg / p.Hq, h = hg % p.Hq;
         S* row = static_cast<S*>(p.scores) + hh * p.head_stride + ri * p.Lk;
-        const long mrow = p.b * p.ms[0] + h * p.ms[1] + i * p.ms[2];
+        const long mrow = b * p.ms[0] + h * p.ms[1] + i * p.ms[2];
         auto value = [&](long j) -> double {
             double s = E::to_f64(E::from_f64(E::to_f64(row[j]) * p.scale));
             if (p.is_causal) {
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(kBlock) void scale_mask_softmax_rows_kernel(const R
         for (long j = threadIdx.x; j < p.Lk; j += kBlock) sum += exp(value(j) - m);
         sum = block_reduce(sum, slots, false);
         for (long j = threadIdx.x; j < p.Lk; j += kBlock) row[j] = E::from_f64(exp(value(j) - m) / sum);
-        if (p.lse && threadIdx.x == 0) p.lse[(p.b * p.Hq + h) * p.Lq + i] = static_cast<float>(m + log(sum));
+        if (p.lse && threadIdx.x == 0) p.lse[(b * p.Hq + h) * p.Lq + i] = static_cast<float>(m + log(sum));
         __syncthreads();     // slots are reused by the next row
     }
 }
@@ -128,13 +129,20 @@ struct Plan {
     size_t vt_bytes, score_bytes;
 };
 
+// One q head per kv head and batches that sit a whole number of heads apart: batch and head form
+// one run of heads, and a piece may span batches (fewer, larger library calls).
+bool heads_run_on(const paras_sdpa_args& a) {
+    return a.Hq == a.Hkv && a.q_strides[0] == a.Hq * a.q_strides[1] && a.k_strides[0] == a.Hkv * a.k_strides[1];
+}
+
 Plan make_plan(const paras_sdpa_args& a) {
     const long rep = a.Hq / a.Hkv;
     const long per_head = a.Lq * a.Lk;
+    const long head_run = heads_run_on(a) ? a.B * a.Hq : a.Hq;
     Plan pl{};
     if (per_head * rep <= score_cap()) {
         pl.rows = a.Lq;
-        pl.heads = rep == 1 ? std::min<long>(a.Hq, std::max<long>(1, score_cap() / per_head)) : rep;
+        pl.heads = rep == 1 ? std::min<long>(head_run, std::max<long>(1, score_cap() / per_head)) : rep;
     } else {
         pl.heads = rep;
         pl.rows = std::max<long>(1, score_cap() / (a.Lk * rep));
@@ -147,13 +155,13 @@ Plan make_plan(const paras_sdpa_args& a) {
 
 }  // namespace
 
-// Large enough that three library calls per piece cost less than the general kernel's scalar
-// fp64 dot products (which it forms three times per score), and addressable by the products
-// (32-bit element offsets inside one operand).
+// Large enough that a handful of library calls cost less than the general kernel's scalar fp64 dot
+// products (which it forms three times per score), and addressable by the products (32-bit element
+// offsets inside one operand).
 bool composed_supported(const paras_sdpa_args& a) {
     if (a.Lq < 64 || a.Lk < 64 || a.D < 1 || a.Dv < 1) return false;
     const double macs = static_cast<double>(a.B) * a.Hq * a.Lq * a.Lk * (a.D + a.Dv);
-    if (macs < static_cast<double>(1L << 29)) return false;
+    if (macs < static_cast<double>(1L << 25)) return false;          // measured: level with the general kernel at 1.7e7, 2.6x faster at 6.7e7
     const long rep = a.Hq / a.Hkv;
     if (a.Lk * rep > score_cap()) return false;                        // not even one row block fits
     if (a.Lq * a.Lk >= (1L << 31) || a.Lk * a.Dv >= (1L << 31)) return false;
@@ -188,9 +196,11 @@ int launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hip
         PARAS_HIP_TRY(hipGetLastError());
     }
 
-    for (long b = 0; b < a.B; ++b)
-        for (long h0 = 0; h0 < a.Hq; h0 += pl.heads) {
-            const long nh = std::min<long>(pl.heads, a.Hq - h0);
+    const bool run_on = heads_run_on(a);
+    const long n_batches = run_on ? 1 : a.B, n_heads = run_on ? a.B * a.Hq : a.Hq;
+    for (long b = 0; b < n_batches; ++b)
+        for (long h0 = 0; h0 < n_heads; h0 += pl.heads) {
+            const long nh = std::min<long>(pl.heads, n_heads - h0);
             const long hkv0 = h0 / rep;
             for (long i0 = 0; i0 < a.Lq; i0 += pl.rows) {
                 const long nr = std::min<long>(pl.rows, a.Lq - i0);

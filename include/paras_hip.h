@@ -240,7 +240,7 @@ PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void*
  * head sizes below 128 other than 64: q, k, v copied into the workspace with
  * zero columns up to 64 or 128, then flash_mfma / decode_split; the workspace
  * must be 256-byte aligned), "composed" (what none of these takes, from about
- * 5e8 multiply-adds on: the reference's own composition,
+ * 3e7 multiply-adds and 64 queries and keys on: the reference's own composition,
  * csrc/ops/attention_ops.cpp:101-135, run as two batched paras_gemm_nt products
  * around one scale / mask / softmax row kernel, scores in `attn` or in the
  * 256-byte aligned workspace, a bounded piece at a time) or "generic". */
