@@ -165,6 +165,8 @@ bool composed_supported(const paras_sdpa_args& a) {
     const long rep = a.Hq / a.Hkv;
     if (a.Lk * rep > score_cap()) return false;                        // not even one row block fits
     if (a.Lq * a.Lk >= (1L << 31) || a.Lk * a.Dv >= (1L << 31)) return false;
+    if (a.q_strides[2] < a.D || a.k_strides[2] < a.D) return false;   // rows the products cannot take (expanded or overlapping views)
+    if (a.B * a.Hkv > 65535 || (a.Dv + 31) / 32 > 65535 || a.B * a.Hq > 65535) return false;   // grid limits of the transpose and the batched products
     return true;
 }
 
@@ -185,7 +187,6 @@ int launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hip
     // v transposed once: the second product reads it along the keys
     {
         const dim3 grid(static_cast<unsigned>((a.Lk + 31) / 32), static_cast<unsigned>((a.Dv + 31) / 32), static_cast<unsigned>(a.B * a.Hkv));
-        PARAS_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "paras sdpa: too many heads or too wide a head for the composed route");
 #define PARAS_TRANSPOSE_V(S_)                                                                                                   \
     hipLaunchKernelGGL((transpose_v_kernel<S_>), grid, dim3(kBlock), 0, s, static_cast<const S_*>(a.v), reinterpret_cast<S_*>(vt), \
                        (long)a.Hkv, (long)a.Lk, (long)a.Dv, (long)a.v_strides[0], (long)a.v_strides[1], (long)a.v_strides[2])
