@@ -87,7 +87,8 @@ def test_ffn_golden():
 
 
 @pytest.mark.parametrize("shape", [(64, 4, 2, 128, 256), (300, 8, 2, 256, 512), (100, 8, 2, 128, 192), (257, 3, 1, 64, 64),
-                                   (500, 8, 4, 320, 448)])
+                                   (500, 8, 4, 320, 448), (333, 8, 3, 128, 128), (200, 16, 5, 64, 192), (150, 8, 7, 128, 64),
+                                   (90, 12, 6, 192, 128)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_ffn_matches_oracle(shape, dtype):
     T, E, k, H, I = shape
