@@ -74,87 +74,15 @@
 #include "core/device_context.h"
 #include "core/device_math.h"
 #include "core/status.h"
+#include "kernels/sdpa_flash_common.h"
 #include "kernels/sdpa_internal.h"
 
 namespace paras {
 namespace {
 
-constexpr int kBN = 64;    // keys per tile
+using namespace flash;
+
 constexpr int kBM = 128;   // queries per workgroup: 4 waves x 32
-
-typedef short i16x8 __attribute__((ext_vector_type(8)));
-typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
-
-struct FlashParams {
-    const std::uint16_t* q;
-    const std::uint16_t* k;
-    const std::uint16_t* v;
-    std::uint16_t*       out;
-    float*               lse;
-    long qs_b, qs_h, qs_l;  // element strides
-    long ks_b, ks_h, ks_l;
-    long vs_b, vs_h, vs_l;
-    int  B, Hq, Hkv, Lq, Lk;
-    int  n_qblocks;
-    float scale_log2;  // scale * log2(e)
-    float scale;
-    // optional mask over [B, Hq, Lq, Lk] (element strides; 0 = broadcast): bytes (nonzero = attend)
-    // or additive values of the tensor dtype
-    const unsigned char* mask;
-    long ms_b, ms_h, ms_q, ms_k;
-    float inv_scale;   // the scores are kept unscaled: an additive mask value m enters as m / scale
-};
-
-template <typename T> struct Mma;
-template <> struct Mma<bf16_t> {
-    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ std::uint32_t pack2(float lo, float hi) {
-        typedef float f32x2 __attribute__((ext_vector_type(2)));
-        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        const f32x2 v = {lo, hi};
-        return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, bf16x2));
-    }
-};
-template <> struct Mma<f16_t> {
-    __device__ static __forceinline__ float16_t run(i16x8 a, i16x8 b, float16_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ std::uint32_t pack2(float lo, float hi) {
-        typedef float f32x2 __attribute__((ext_vector_type(2)));
-        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-        const f32x2 v = {lo, hi};
-        return __builtin_bit_cast(std::uint32_t, __builtin_convertvector(v, f16x2));
-    }
-};
-
-// Exchange between the two half-waves that share a query: v_permlane32_swap
-// swaps lanes 32..63 of its first register with lanes 0..31 of its second.
-// Fed the same value twice it leaves the lower half's value in every lane of
-// the first register and the upper half's value in every lane of the second.
-// Written as inline asm because the compiler's builtin for it returns the
-// first result twice (seen with ROCm 7.2's hipcc); the s_nop pairs cover the
-// VALU-write -> permlane-read and permlane-write -> VALU-read wait states the
-// hazard recognizer cannot see inside an asm block.
-__device__ __forceinline__ void half_swap(float x, float& lo, float& hi) {
-    float a = x, b = x;
-    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    lo = a;
-    hi = b;
-}
-__device__ __forceinline__ float half_swap_max(float x) {
-    float lo, hi;
-    half_swap(x, lo, hi);
-    return fmaxf(lo, hi);
-}
-__device__ __forceinline__ float half_swap_sum(float x) {
-    float lo, hi;
-    half_swap(x, lo, hi);
-    return lo + hi;
-}
 
 // kMask: 0 none, 1 bytes (nonzero = attend), 2 additive values of type T.
 template <typename T, int D, bool kCausal, int kMask>
@@ -682,6 +610,7 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     p.inv_scale = static_cast<float>(1.0 / a.scale);
     const bool causal = a.is_causal != 0;
     const int mk = a.mask_kind;
+    if (wide_supported(p, static_cast<int>(a.D), mk)) return launch_flash_wide(p, causal, a.dtype == PARAS_BF16, s);
     if (a.dtype == PARAS_BF16)
         return a.D == 128 ? launch_t<bf16_t, 128>(p, causal, mk, s) : launch_t<bf16_t, 64>(p, causal, mk, s);
     return a.D == 128 ? launch_t<f16_t, 128>(p, causal, mk, s) : launch_t<f16_t, 64>(p, causal, mk, s);

@@ -1,0 +1,457 @@
+// Flash-attention forward for gfx950, head size 128, 64 queries per wavefront.
+//
+// Same mathematics and the same lane layout as sdpa_flash.hip (S^T = K Q^T and
+// O^T = V^T P^T on v_mfma_f32_32x32x16, a lane owns one query column, online
+// softmax with a lazily raised reference point; the reference materialises the
+// scores instead: csrc/ops/attention_ops.cpp:101,128).  What differs is the shape
+// of a wavefront's work:
+//
+//   The LDS delivers 128 bytes per clock per CU, and a 32x32x16 MFMA whose K or V
+//   operand comes from LDS needs 1 KB of it: four SIMDs issuing one MFMA every 32
+//   clocks ask for exactly the LDS's peak.  With 32 queries per wavefront the
+//   operand reads are the bound.  Here a wavefront owns TWO 32-query blocks, so
+//   every K / V fragment read from LDS feeds two MFMAs, and a workgroup of four
+//   wavefronts covers 256 queries, so a staged tile is shared by twice the
+//   queries as well.
+//
+//   64 queries x 128 columns of fp32 output are 128 registers per lane, the query
+//   fragments another 64: the kernel runs one wavefront per SIMD with the 512
+//   registers of the unified file.  Outputs and queries live in the accumulation
+//   half (AGPRs), which only the MFMAs touch; scores, probabilities and operand
+//   fragments live in VGPRs.  The compiler does not make that split by itself (it
+//   keeps copying between the halves), so the MFMAs of this kernel are inline
+//   assembly with the register file of each operand spelled out.  What the
+//   compiler cannot see inside them is covered by hand: a VALU read of an MFMA
+//   result is kept at least a dozen MFMAs behind it by the schedule, or behind
+//   explicit s_nop where it is not (first scores, rescale branch, epilogue).
+//
+// With nothing else on the SIMD to fill a stall, the schedule inside a block (32
+// keys x 64 queries = 32 MFMAs) is flat: one MFMA, then a few VALU instructions
+// of the softmax of the block before, then the next MFMA,
+//
+//   u = 0..15   S(j+1) = K(j+1) Q^T   (k-step u/2, query block u%2)
+//   u = 16..31  O^T += V(j)^T P(j)^T  ((query block, key half) = (0,0) (1,0) (0,1) (1,1), four column blocks each)
+//   the 16 exp pairs of S(j) sit before MFMA 7e/4, each ahead of the first PV MFMA that needs it;
+//   the row maxima of S(j+1) are reduced in u = 27..30
+//
+// and every operand is requested from LDS at least eight MFMAs before its use:
+// the V fragments of block j during its score MFMAs, the K fragments of block
+// j+1's score MFMAs (keys of block j+2) during block j's PV MFMAs.  Those keys
+// belong to the next K tile, so during tile t a wavefront reads K tile t+1 and V
+// tile t while K tile t+2 and V tile t+1 stream in: two buffers each, one
+// barrier per tile, and no operand request ever waits for a barrier.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdlib>
+#include <type_traits>
+#include <utility>
+
+#include "core/device_context.h"
+#include "core/device_math.h"
+#include "core/status.h"
+#include "kernels/sdpa_flash_common.h"
+
+namespace paras {
+namespace flash {
+namespace {
+
+#ifndef WIDE_KO
+#define WIDE_KO 0
+#endif
+constexpr int D      = 128;
+constexpr int QB     = 2;            // 32-query blocks per wavefront
+constexpr int NW     = 4;
+constexpr int WQ     = 32 * QB;
+constexpr int KSTEPS = D / 16;       // 8
+constexpr int DBLK   = D / 32;       // 4
+constexpr int CHUNKS = D / 8;        // 16-byte chunks per row
+constexpr int RPI    = 64 / CHUNKS;  // rows one wavefront stages per instruction
+constexpr int NI     = kBN / (RPI * NW);
+static_assert(kWideBM == NW * WQ, "workgroup shape");
+
+// f(integral_constant<int, I>) for I = 0 .. N-1: loop indices the front end sees as constants.
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
+}
+
+template <typename T, bool kCausal>
+__global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p) {
+    auto ksw = [](int row) { return row & 15; };
+    auto vsw = [](int row) { return (row & 3) << 2; };
+
+    // Four separate arrays: an LDS read waits for every direct-to-LDS load in flight unless the
+    // variables involved prove them disjoint, so the main loop names its buffers at compile time.
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds0[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds1[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds0[kBN * D];
+    __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds1[kBN * D];
+    using Par0 = std::integral_constant<int, 0>;
+    using Par1 = std::integral_constant<int, 1>;
+    struct AnyPar { int value; };
+    auto kbuf = [&](auto par, bool flip) -> std::uint16_t* {
+        if constexpr (std::is_same<decltype(par), AnyPar>::value) return ((par.value ^ (flip ? 1 : 0)) & 1) ? k_lds1 : k_lds0;
+        else return (decltype(par)::value != 0) != flip ? k_lds1 : k_lds0;
+    };
+    auto vbuf = [&](auto par, bool flip) -> std::uint16_t* {
+        if constexpr (std::is_same<decltype(par), AnyPar>::value) return ((par.value ^ (flip ? 1 : 0)) & 1) ? v_lds1 : v_lds0;
+        else return (decltype(par)::value != 0) != flip ? v_lds1 : v_lds0;
+    };
+
+    const int nq = p.n_qblocks;
+    int bh, qblock;
+    map_workgroup(blockIdx.x, p.B * p.Hq, nq, bh, qblock);
+    const int b = bh / p.Hq, hq = bh % p.Hq;
+    const int hkv = hq / (p.Hq / p.Hkv);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lq = lane & 31, lh = lane >> 5;
+    const int q0 = qblock * kWideBM + wave * WQ;   // query block qb of this wavefront starts at q0 + 32 qb
+
+    i16x8 qreg[QB][KSTEPS];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int my_q = q0 + 32 * qb + lq;
+        const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
+        const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) qreg[qb][ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
+    }
+
+    const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
+    const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
+
+    int n_tiles = (p.Lk + kBN - 1) / kBN;
+    if (kCausal) {
+        const int last_q = min(qblock * kWideBM + kWideBM, p.Lq) - 1;
+        n_tiles = (min(last_q + 1, p.Lk) + kBN - 1) / kBN;
+    }
+    const int wave_tiles = kCausal ? min(n_tiles, (q0 + WQ - 1) / kBN + 1) : n_tiles;
+
+    // ---- staging: global rows straight into LDS with buffer loads; the descriptor spans rows
+    // [0, Lk) of this (batch, kv head), so rows past the end arrive as zeros without a branch.
+    const int srow = wave * RPI + lane / CHUNKS;
+    const int slot = lane % CHUNKS;
+    const int k_row_bytes = static_cast<int>(p.ks_l) * 2, v_row_bytes = static_cast<int>(p.vs_l) * 2;
+    const int k_lane = srow * k_row_bytes + ((slot ^ ksw(srow)) * 16);
+    const int v_lane = srow * v_row_bytes + ((slot ^ vsw(srow)) * 16);
+    typedef __attribute__((address_space(3))) void* lptr_t;
+    auto make_rsrc = [&](const std::uint16_t* base, int row_bytes) {
+        const int bytes = (p.Lk - 1) * row_bytes + D * 2;           // < 2^31: checked by flash_supported
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<std::uint16_t*>(base), 0, bytes, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(kbase, k_row_bytes);
+    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(vbase, v_row_bytes);
+    auto stage_one = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile, int i) {
+        if constexpr ((WIDE_KO & 2) != 0) { if (first > kBN) return; }
+        const int r0 = i * RPI * NW;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)(tile + (r0 + wave * RPI) * D), 16,
+                                                 lane_off + (first + r0) * row_bytes, 0, 0, 0);
+    };
+    auto stage_rows = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) stage_one(rsrc, lane_off, row_bytes, first, tile, i);
+    };
+    // What tile t's successor needs beyond what tile t already reads: K tile t+2 (into the buffer
+    // of K tile t, which nobody reads any more) and V tile t+1.
+    auto stage_pair = [&](int t, auto par) {
+        stage_rows(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN, kbuf(par, false));
+        stage_rows(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true));
+    };
+    auto publish = [&]() {
+        if constexpr ((WIDE_KO & 8) == 0) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tiles has landed
+        if constexpr ((WIDE_KO & 1) == 0) __syncthreads();
+    };
+
+    float16_t oacc[QB][DBLK];
+    float m_run[QB], l_run[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.f;
+#pragma unroll
+        for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[qb][i][r] = 0.f;
+    }
+
+    stage_rows(k_rsrc, k_lane, k_row_bytes, 0, k_lds0);
+    stage_rows(k_rsrc, k_lane, k_row_bytes, kBN, k_lds1);
+    stage_rows(v_rsrc, v_lane, v_row_bytes, 0, v_lds0);
+    publish();
+
+    const int grp = lane >> 4, m16 = lane & 15;
+    int k_rd[KSTEPS], v_rd[DBLK];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) k_rd[ks] = lq * D + (((2 * ks + lh) ^ ksw(lq)) * 8);
+    {
+        const int vrow = 4 * lh + (m16 >> 2);
+#pragma unroll
+        for (int db = 0; db < DBLK; ++db)
+            v_rd[db] = vrow * D + (((4 * db + 2 * (grp & 1) + ((m16 & 3) >> 1)) ^ vsw(vrow)) * 8) + 4 * (m16 & 1);
+    }
+    const float lazy_margin = 8.0f / p.scale_log2;
+
+    // Block j of query block qb needs masking from its diagonal block on (j * 32 + 31 > first query)
+    // and where it reaches past the end of K (j * 32 + 32 > Lk): j >= first_masked[qb].
+    int first_masked[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) first_masked[qb] = kCausal ? min((q0 + 32 * qb) >> 5, p.Lk >> 5) : (p.Lk >> 5);
+    auto needs_mask = [&](int j, int qb) { return j >= first_masked[qb]; };
+    auto apply_mask = [&](int j, int qb, float16_t& sc) {
+        const int my_q = q0 + 32 * qb + lq;
+        const int last_visible = kCausal ? min(my_q, p.Lk - 1) : p.Lk - 1;
+        const int rel = last_visible - j * 32 - 4 * lh;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if ((r >> 2) * 8 + (r & 3) > rel) sc[r] = -INFINITY;
+    };
+    auto lane_max = [](const float16_t& sc) {
+        float mx = sc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+        return mx;
+    };
+    // Raise the running maxima where a block max (this lane's half of the keys) asks for it; the
+    // two halves of a query only meet inside this rarely taken branch.
+    auto wants_raise = [&](const float (&mx)[QB]) {
+        bool grow = false;
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) grow = grow || (mx[qb] > m_run[qb] + lazy_margin);
+        return __builtin_amdgcn_ballot_w64(grow) != 0;   // wave-uniform, rare after block 0
+    };
+    auto raise_max = [&](const float (&mx)[QB]) {
+        // (pins the outputs in AGPRs up to here: without it their 128 copies to VGPRs are
+        // hoisted out of this branch into every block)
+        asm volatile("" : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]),
+                          "+a"(oacc[1][0]), "+a"(oacc[1][1]), "+a"(oacc[1][2]), "+a"(oacc[1][3]));
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            const float m_new = fmaxf(m_run[qb], half_swap_max(mx[qb]));
+            // (equal covers -inf on both sides: a query that has seen no key yet keeps its zeros)
+            const float alpha = m_run[qb] == m_new ? 1.f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.scale_log2);
+            m_run[qb] = m_new;
+            l_run[qb] *= alpha;
+#pragma unroll
+            for (int i = 0; i < DBLK; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[qb][i][r] *= alpha;
+        }
+        asm volatile("" : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]),
+                          "+a"(oacc[1][0]), "+a"(oacc[1][1]), "+a"(oacc[1][2]), "+a"(oacc[1][3]));
+    };
+    // Scores of block j are complete in `sc`, their in-lane maxima in `mx`, and `raise` says whether
+    // those maxima ask for a higher reference point.  Blocks on the diagonal or at the end of K are
+    // masked first and their maxima taken again.
+    auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB], bool raise) {
+        if (needs_mask(j, 0)) {                 // first_masked[0] <= first_masked[1]: one test on the common path
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                if (needs_mask(j, qb)) {
+                    apply_mask(j, qb, sc[qb]);
+                    mx[qb] = lane_max(sc[qb]);
+                }
+            }
+            raise = wants_raise(mx);
+        }
+        if (raise) raise_max(mx);
+    };
+
+    // Operand fragments: kf = the K rows of the block whose scores come next, vf = the V rows of
+    // the block whose probabilities are applied now.
+    i16x8 kf[KSTEPS], vf[2 * DBLK];
+    auto fetch_k = [&](const std::uint16_t* rows, int ks) { if constexpr ((WIDE_KO & 4) != 0) { if (rows != k_lds0) return; } kf[ks] = *reinterpret_cast<const i16x8*>(rows + k_rd[ks]); };
+    auto fetch_v = [&](const std::uint16_t* rows, int f) {     // f = 4 * (16-key half) + column block
+        if constexpr ((WIDE_KO & 4) != 0) { if (rows != v_lds0) return; }
+        const std::uint16_t* vp = rows + v_rd[f % DBLK] + 16 * (f / DBLK) * D;
+        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
+        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
+        vf[f] = i16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    // One block j of 32 keys: exponentials of `cur` = S(j), PV(j) and the score MFMAs of S(j+1)
+    // into `nxt`.  `par` is the parity of block j's tile: V(j) lives in the V buffer of that
+    // parity, the keys of block j+2 (requested here for block j+1's score MFMAs) in the K buffer
+    // of the other one.  On entry kf holds the keys of block j+1.
+    //
+    // The softmax of S(j) is a list of 128 VALU instructions, dealt four to each of the 32 MFMAs
+    // so that neither pipe waits for the other: the 16 exp pairs two at a time (the four fma, the
+    // four exp, cvt and add of both, the two sum updates: 14 instructions, no exponential next to
+    // its producer or its consumer, so no hazard nop), in
+    // the order the PV MFMAs need them -- pair e is finished before MFMA 7(e|1)/4 + 4, ahead of
+    // MFMA 16 / 20 / 24 / 28 for the four (query block, key half) groups -- then the 16
+    // instructions of the row maxima of S(j+1) under the last four MFMAs.
+    auto block = [&](int j, float16_t (&cur)[QB], float16_t (&nxt)[QB], auto par, auto stage_tag) {
+        constexpr bool kStage = decltype(stage_tag)::value;
+        const std::uint16_t* vrows = vbuf(par, false) + (j & 1) * 32 * D;
+        const std::uint16_t* krows = kbuf(par, true) + (j & 1) * 32 * D;
+        float mc[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) mc[qb] = m_run[qb] * p.scale_log2;
+        u32x4 pw[QB][2];
+        float mx[QB], t3[QB][7], ex[16][2], sm[16];
+        bool raise = false;
+        auto valu_op = [&](auto O) {
+            constexpr int o = decltype(O)::value;
+            if constexpr (o < 112) {
+                constexpr int k = o / 14, r = o % 14;
+                // r: 0-3 fma (a0 a1 b0 b1), 4-7 exp (a0 a1 b0 b1), 8 cvt a, 9 add a, 10 cvt b, 11 add b, 12 sum a, 13 sum b
+                constexpr int e = 2 * k + (r < 8 ? ((r & 3) >> 1) : (r < 12 ? ((r - 8) >> 1) : r - 12));   // exp pair 0..15
+                constexpr int qb = (e >> 2) & 1, i = (e & 3) + 4 * (e >> 3);       // elements 2i, 2i+1 of cur[qb]
+                constexpr int w = r < 8 ? (r & 1) + 2 * (r >> 2) : (r < 12 ? (r & 1) : 2);   // <8: 0,1 fma 2,3 exp; else 0 cvt 1 add 2 sum
+                if constexpr (r < 8) {
+                    if constexpr (w < 2) ex[e][w] = fmaf(cur[qb][2 * i + w], p.scale_log2, -mc[qb]);
+                    else if constexpr ((WIDE_KO & 16) == 0) ex[e][w - 2] = __builtin_amdgcn_exp2f(ex[e][w - 2]);
+                    asm volatile("" : "+v"(ex[e][w & 1]));
+                } else if constexpr (w == 0) {
+                    std::uint32_t pk = Mma<T>::pack2(ex[e][0], ex[e][1]);
+                    asm volatile("" : "+v"(pk));
+                    pw[qb][i / 4][i % 4] = pk;
+                } else if constexpr (w == 1) {
+                    sm[e] = ex[e][0] + ex[e][1];
+                    asm volatile("" : "+v"(sm[e]));
+                } else {
+                    l_run[qb] += sm[e];
+                    asm volatile("" : "+v"(l_run[qb]));
+                }
+            } else {
+                constexpr int qb = (o - 112) / 8, r = (o - 112) % 8;
+                const float16_t& sv = nxt[qb];
+                if constexpr (r < 5)       t3[qb][r] = fmaxf(fmaxf(sv[3 * r], sv[3 * r + 1]), sv[3 * r + 2]);
+                else if constexpr (r == 5) t3[qb][5] = fmaxf(fmaxf(t3[qb][0], t3[qb][1]), t3[qb][2]);
+                else if constexpr (r == 6) t3[qb][6] = fmaxf(fmaxf(t3[qb][3], t3[qb][4]), sv[15]);
+                else                       mx[qb] = fmaxf(t3[qb][5], t3[qb][6]);
+                if constexpr (r < 7) asm volatile("" : "+v"(t3[qb][r]));
+                else                 asm volatile("" : "+v"(mx[qb]));
+            }
+        };
+        static_for<32>([&](auto U) {
+            constexpr int u = decltype(U)::value;
+            if constexpr ((WIDE_KO & 32) == 0 || u >= 28)
+                static_for<4>([&](auto I) {
+                    constexpr int o = 4 * u + decltype(I)::value;
+                    if constexpr ((WIDE_KO & 64) == 0 || (o % 14 != 9 && o % 14 != 10 && o % 14 != 12 && o % 14 != 13) || o >= 112) valu_op(std::integral_constant<int, o>{});
+                });
+            if constexpr (u == 31) raise = wants_raise(mx);          // decided under the last MFMA, acted on after it
+            // Two waits per block instead of one per MFMA (an instruction of any kind costs this
+            // lone wavefront an issue slot): every request waited for here is eight MFMAs old.
+            if constexpr (u == 0 || u == 16) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
+            if constexpr (u < 16) {
+                constexpr int c = u >> 1, qb = u & 1;
+                if constexpr (c == 0) Mma<T>::score_first(nxt[qb], kf[0], qreg[qb][0]);
+                else                  Mma<T>::score_acc(nxt[qb], kf[c], qreg[qb][c]);
+                if constexpr (u < 2 * DBLK) fetch_v(vrows, u);
+            } else {
+                constexpr int g = (u - 16) >> 2, qb = g & 1, s2 = g >> 1, db = (u - 16) & 3;
+                oacc[qb][db] = Mma<T>::run(vf[s2 * DBLK + db], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
+                if constexpr (u < 16 + KSTEPS) fetch_k(krows, u - 16);
+            }
+            if constexpr (kStage && u % 4 == 1) {
+                // the next tile pair (K tile t+2, V tile t+1), one request every fourth MFMA
+                constexpr int i = u / 4;
+                const int t = j >> 1;
+                if constexpr (i < NI) stage_one(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN, kbuf(par, false), i);
+                else                  stage_one(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true), i - NI);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        finish_scores(j + 1, nxt, mx, raise);
+    };
+    using Yes = std::true_type;
+    using No  = std::false_type;
+
+    float16_t s_a[QB], s_b[QB];
+    {
+        // S(0) from the first half of K tile 0, then the keys of block 1 for block 0's score MFMAs
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) fetch_k(k_lds0, ks);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                if (ks == 0) Mma<T>::score_first(s_a[qb], kf[0], qreg[qb][0]);
+                else         Mma<T>::score_acc(s_a[qb], kf[ks], qreg[qb][ks]);
+            }
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s_a[0]), "+v"(s_a[1]));
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) fetch_k(k_lds0 + 32 * D, ks);
+        float mx[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) mx[qb] = lane_max(s_a[qb]);
+        finish_scores(0, s_a, mx, wants_raise(mx));
+    }
+    // Every tile runs the same two blocks, the last one included: its second block then forms
+    // scores nobody uses (of keys past the end of K or past the diagonal; whatever the LDS rows
+    // hold, they are masked to -inf before anything reads them), and a block that lies wholly past
+    // the end of K contributes zeros.  One instance of the block code instead of a handful keeps
+    // the register assignment of the loop the one that was checked.
+    auto tile = [&](int t, auto par) {
+        block(2 * t, s_a, s_b, par, Yes{});
+        block(2 * t + 1, s_b, s_a, par, No{});
+        publish();
+    };
+    for (int t = 0; t < wave_tiles; t += 2) {
+        tile(t, Par0{});
+        if (t + 1 >= wave_tiles) break;
+        tile(t + 1, Par1{});
+    }
+    for (int t = wave_tiles; t < n_tiles; ++t) {           // done early (causal): keep staging for the other wavefronts
+        stage_pair(t, AnyPar{t});
+        publish();
+    }
+
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int my_q = q0 + 32 * qb + lq;
+        const float l_tot = half_swap_sum(l_run[qb]);
+        const float inv_l = 1.0f / l_tot;
+        if (my_q < p.Lq) {
+            std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
+#pragma unroll
+            for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d = db * 32 + g * 8 + 4 * lh;
+                    u32x2 w;
+                    w[0] = Mma<T>::pack2(oacc[qb][db][4 * g + 0] * inv_l, oacc[qb][db][4 * g + 1] * inv_l);
+                    w[1] = Mma<T>::pack2(oacc[qb][db][4 * g + 2] * inv_l, oacc[qb][db][4 * g + 3] * inv_l);
+                    *reinterpret_cast<u32x2*>(op + d) = w;
+                }
+            if (p.lse != nullptr && lh == 0)
+                p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run[qb] * p.scale + logf(l_tot);
+        }
+    }
+}
+
+template <typename T>
+int launch_t(FlashParams p, bool causal, hipStream_t s) {
+    p.n_qblocks = (p.Lq + kWideBM - 1) / kWideBM;
+    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
+    const dim3 grid(static_cast<unsigned>(blocks)), wg(256);
+    if (causal) hipLaunchKernelGGL((flash_wide_kernel<T, true>), grid, wg, 0, s, p);
+    else        hipLaunchKernelGGL((flash_wide_kernel<T, false>), grid, wg, 0, s, p);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
+}  // namespace
+
+bool wide_supported(const FlashParams& p, int head, int mask_kind) {
+    static const int forced = [] { const char* e = std::getenv("PARAS_FLASH_WIDE"); return e ? std::atoi(e) : -1; }();
+    if (head != D || mask_kind != 0) return false;
+    if (forced >= 0) return forced != 0;
+    return false;   // opt-in (PARAS_FLASH_WIDE=1) until it wins on the causal shapes too
+}
+
+int launch_flash_wide(FlashParams p, bool causal, bool is_bf16, hipStream_t s) {
+    return is_bf16 ? launch_t<bf16_t>(p, causal, s) : launch_t<f16_t>(p, causal, s);
+}
+
+}  // namespace flash
+}  // namespace paras
