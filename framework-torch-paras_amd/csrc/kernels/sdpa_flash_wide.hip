@@ -91,6 +91,12 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     __shared__ __attribute__((aligned(1024))) std::uint16_t k_lds1[kBN * D];
     __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds0[kBN * D];
     __shared__ __attribute__((aligned(1024))) std::uint16_t v_lds1[kBN * D];
+    // A wavefront's 64 x 128 outputs pass through LDS on their way out (16 KB each, its own region:
+    // no barrier), so that the global stores write whole rows.
+    constexpr int OROW = D + 8;   // row pitch of that region in elements: 16 bytes of padding spread the rows over the banks
+    __shared__ __attribute__((aligned(1024))) std::uint16_t o_lds[kWideBM * OROW];
+    using Yes = std::true_type;
+    using No  = std::false_type;
     using Par0 = std::integral_constant<int, 0>;
     using Par1 = std::integral_constant<int, 1>;
     struct AnyPar { int value; };
@@ -103,51 +109,83 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
         else return (decltype(par)::value != 0) != flip ? v_lds1 : v_lds0;
     };
 
-    const int nq = p.n_qblocks;
-    int bh, qblock;
-    map_workgroup(blockIdx.x, p.B * p.Hq, nq, bh, qblock);
-    const int b = bh / p.Hq, hq = bh % p.Hq;
-    const int hkv = hq / (p.Hq / p.Hkv);
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lq = lane & 31, lh = lane >> 5;
-    const int q0 = qblock * kWideBM + wave * WQ;   // query block qb of this wavefront starts at q0 + 32 qb
 
+    // ---- work items.  The grid is one workgroup per CU and every workgroup walks a list of
+    // (batch * head, query tile) items of its own: a new workgroup could only start once the one
+    // before it had drained (64 KB of LDS and all 512 registers allow one per CU), which left the
+    // CU idle for 11 us per item -- launch, first loads, first scores.  Walking the list inside
+    // the kernel, the loads of the next item are in flight while the outputs of this one are
+    // normalised and stored.
+    //   Workgroup w runs on XCD w % 8 (round-robin dispatch), so with a head count that divides
+    // by 8 the heads are dealt to the XCDs and the workgroups of an XCD share the K / V of few
+    // heads at a time in its L2.  Within such a pool the items are numbered head by head, longest
+    // query tile first under the causal rule, and dealt in rounds of one item per workgroup, every
+    // other round in reverse order, which evens out the triangle (tile i then tile n-1-i).
+    const int nq = p.n_qblocks;
+    const int BH = p.B * p.Hq;
+    const int n_wg = static_cast<int>(gridDim.x), wg_id = static_cast<int>(blockIdx.x);
+    const bool by_xcd = BH % 8 == 0 && n_wg % 8 == 0;
+    const int pool_wgs = by_xcd ? n_wg >> 3 : n_wg;
+    const int pool_pos = by_xcd ? wg_id >> 3 : wg_id;
+    const int pool_items = (by_xcd ? BH >> 3 : BH) * nq;
+    auto item_at = [&](int round, int& bh, int& qblock) {
+        const int i = round * pool_wgs + ((round & 1) ? pool_wgs - 1 - pool_pos : pool_pos);
+        if (i >= pool_items) return false;
+        const int head = i / nq, pos = i - head * nq;
+        bh = by_xcd ? head * 8 + (wg_id & 7) : head;
+        qblock = kCausal ? nq - 1 - pos : pos;
+        return true;
+    };
+
+    // ---- the item at hand
+    int b, hq, q0, n_tiles, wave_tiles, first_masked[QB];
+    __amdgpu_buffer_rsrc_t k_rsrc, v_rsrc;
     i16x8 qreg[QB][KSTEPS];
+    const int k_row_bytes = static_cast<int>(p.ks_l) * 2, v_row_bytes = static_cast<int>(p.vs_l) * 2;
+    auto make_rsrc = [&](const std::uint16_t* base, int row_bytes) {
+        const int bytes = (p.Lk - 1) * row_bytes + D * 2;           // < 2^31: checked by flash_supported
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<std::uint16_t*>(base), 0, bytes, 0x00020000);
+    };
+    auto load_queries = [&]() {
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        const int my_q = q0 + 32 * qb + lq;
-        const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
-        const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
+        for (int qb = 0; qb < QB; ++qb) {
+            const int my_q = q0 + 32 * qb + lq;
+            const int qrow = my_q < p.Lq ? my_q : p.Lq - 1;
+            const std::uint16_t* qp = p.q + b * p.qs_b + hq * p.qs_h + static_cast<long>(qrow) * p.qs_l;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) qreg[qb][ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
-    }
-
-    const std::uint16_t* kbase = p.k + b * p.ks_b + hkv * p.ks_h;
-    const std::uint16_t* vbase = p.v + b * p.vs_b + hkv * p.vs_h;
-
-    int n_tiles = (p.Lk + kBN - 1) / kBN;
-    if (kCausal) {
-        const int last_q = min(qblock * kWideBM + kWideBM, p.Lq) - 1;
-        n_tiles = (min(last_q + 1, p.Lk) + kBN - 1) / kBN;
-    }
-    const int wave_tiles = kCausal ? min(n_tiles, (q0 + WQ - 1) / kBN + 1) : n_tiles;
+            for (int ks = 0; ks < KSTEPS; ++ks) qreg[qb][ks] = *reinterpret_cast<const i16x8*>(qp + ks * 16 + lh * 8);
+        }
+    };
+    // Everything that depends on the item.
+    auto enter_item = [&](int bh, int qblock) {
+        b = bh / p.Hq;
+        hq = bh - b * p.Hq;
+        const int hkv = hq / (p.Hq / p.Hkv);
+        q0 = qblock * kWideBM + wave * WQ;   // query block qb of this wavefront starts at q0 + 32 qb
+        k_rsrc = make_rsrc(p.k + b * p.ks_b + hkv * p.ks_h, k_row_bytes);
+        v_rsrc = make_rsrc(p.v + b * p.vs_b + hkv * p.vs_h, v_row_bytes);
+        n_tiles = (p.Lk + kBN - 1) / kBN;
+        if (kCausal) {
+            const int last_q = min(qblock * kWideBM + kWideBM, p.Lq) - 1;
+            n_tiles = (min(last_q + 1, p.Lk) + kBN - 1) / kBN;
+        }
+        wave_tiles = kCausal ? min(n_tiles, (q0 + WQ - 1) / kBN + 1) : n_tiles;
+        // Block j of query block qb needs masking from its diagonal block on (j * 32 + 31 > first
+        // query) and where it reaches past the end of K (j * 32 + 32 > Lk): j >= first_masked[qb].
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) first_masked[qb] = kCausal ? min((q0 + 32 * qb) >> 5, p.Lk >> 5) : (p.Lk >> 5);
+    };
 
     // ---- staging: global rows straight into LDS with buffer loads; the descriptor spans rows
     // [0, Lk) of this (batch, kv head), so rows past the end arrive as zeros without a branch.
     const int srow = wave * RPI + lane / CHUNKS;
     const int slot = lane % CHUNKS;
-    const int k_row_bytes = static_cast<int>(p.ks_l) * 2, v_row_bytes = static_cast<int>(p.vs_l) * 2;
     const int k_lane = srow * k_row_bytes + ((slot ^ ksw(srow)) * 16);
     const int v_lane = srow * v_row_bytes + ((slot ^ vsw(srow)) * 16);
     typedef __attribute__((address_space(3))) void* lptr_t;
-    auto make_rsrc = [&](const std::uint16_t* base, int row_bytes) {
-        const int bytes = (p.Lk - 1) * row_bytes + D * 2;           // < 2^31: checked by flash_supported
-        return __builtin_amdgcn_make_buffer_rsrc(const_cast<std::uint16_t*>(base), 0, bytes, 0x00020000);
-    };
-    const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(kbase, k_row_bytes);
-    const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(vbase, v_row_bytes);
     auto stage_one = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile, int i) {
         if constexpr ((WIDE_KO & 2) != 0) { if (first > kBN) return; }
         const int r0 = i * RPI * NW;
@@ -171,20 +209,12 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
 
     float16_t oacc[QB][DBLK];
     float m_run[QB], l_run[QB];
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        m_run[qb] = -INFINITY;
-        l_run[qb] = 0.f;
-#pragma unroll
-        for (int i = 0; i < DBLK; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[qb][i][r] = 0.f;
-    }
-
-    stage_rows(k_rsrc, k_lane, k_row_bytes, 0, k_lds0);
-    stage_rows(k_rsrc, k_lane, k_row_bytes, kBN, k_lds1);
-    stage_rows(v_rsrc, v_lane, v_row_bytes, 0, v_lds0);
-    publish();
+    // The first tiles of an item: K tiles 0 and 1, V tile 0 (the loop stages the rest).
+    auto stage_first = [&]() {
+        stage_rows(k_rsrc, k_lane, k_row_bytes, 0, k_lds0);
+        stage_rows(k_rsrc, k_lane, k_row_bytes, kBN, k_lds1);
+        stage_rows(v_rsrc, v_lane, v_row_bytes, 0, v_lds0);
+    };
 
     const int grp = lane >> 4, m16 = lane & 15;
     int k_rd[KSTEPS], v_rd[DBLK];
@@ -198,11 +228,6 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     }
     const float lazy_margin = 8.0f / p.scale_log2;
 
-    // Block j of query block qb needs masking from its diagonal block on (j * 32 + 31 > first query)
-    // and where it reaches past the end of K (j * 32 + 32 > Lk): j >= first_masked[qb].
-    int first_masked[QB];
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb) first_masked[qb] = kCausal ? min((q0 + 32 * qb) >> 5, p.Lk >> 5) : (p.Lk >> 5);
     auto needs_mask = [&](int j, int qb) { return j >= first_masked[qb]; };
     auto apply_mask = [&](int j, int qb, float16_t& sc) {
         const int my_q = q0 + 32 * qb + lq;
@@ -297,47 +322,59 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
         u32x4 pw[QB][2];
         float mx[QB], t3[QB][7], ex[16][2], sm[16];
         bool raise = false;
-        auto valu_op = [&](auto O) {
+        // v_max3_f32 as written (fmaxf would canonicalise operands that come out of inline assembly)
+        auto max3 = [](float a, float b, float c) {
+            float r;
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+            return r;
+        };
+        // Instruction o of the list, and (separately, one instruction later: an inline-assembly
+        // operand written by the instruction just before costs a hazard nop) the empty asm that
+        // pins its result, i.e. keeps the instruction in its slot.
+        auto valu_op = [&](auto O, auto PinOnly) {
             constexpr int o = decltype(O)::value;
-            if constexpr (o < 112) {
+            constexpr bool pin = decltype(PinOnly)::value;
+            if constexpr (o < 0 || o >= 128) {
+            } else if constexpr (o < 112) {
                 constexpr int k = o / 14, r = o % 14;
                 // r: 0-3 fma (a0 a1 b0 b1), 4-7 exp (a0 a1 b0 b1), 8 cvt a, 9 add a, 10 cvt b, 11 add b, 12 sum a, 13 sum b
                 constexpr int e = 2 * k + (r < 8 ? ((r & 3) >> 1) : (r < 12 ? ((r - 8) >> 1) : r - 12));   // exp pair 0..15
                 constexpr int qb = (e >> 2) & 1, i = (e & 3) + 4 * (e >> 3);       // elements 2i, 2i+1 of cur[qb]
                 constexpr int w = r < 8 ? (r & 1) + 2 * (r >> 2) : (r < 12 ? (r & 1) : 2);   // <8: 0,1 fma 2,3 exp; else 0 cvt 1 add 2 sum
                 if constexpr (r < 8) {
-                    if constexpr (w < 2) ex[e][w] = fmaf(cur[qb][2 * i + w], p.scale_log2, -mc[qb]);
+                    if constexpr (pin) asm volatile("" :: "v"(ex[e][w & 1]));
+                    else if constexpr (w < 2) ex[e][w] = fmaf(cur[qb][2 * i + w], p.scale_log2, -mc[qb]);
                     else if constexpr ((WIDE_KO & 16) == 0) ex[e][w - 2] = __builtin_amdgcn_exp2f(ex[e][w - 2]);
-                    asm volatile("" : "+v"(ex[e][w & 1]));
                 } else if constexpr (w == 0) {
-                    std::uint32_t pk = Mma<T>::pack2(ex[e][0], ex[e][1]);
-                    asm volatile("" : "+v"(pk));
-                    pw[qb][i / 4][i % 4] = pk;
+                    if constexpr (pin) asm volatile("" :: "v"(pw[qb][i / 4][i % 4]));
+                    else pw[qb][i / 4][i % 4] = Mma<T>::pack2(ex[e][0], ex[e][1]);
                 } else if constexpr (w == 1) {
-                    sm[e] = ex[e][0] + ex[e][1];
-                    asm volatile("" : "+v"(sm[e]));
+                    if constexpr (pin) asm volatile("" :: "v"(sm[e]));
+                    else sm[e] = ex[e][0] + ex[e][1];
                 } else {
-                    l_run[qb] += sm[e];
-                    asm volatile("" : "+v"(l_run[qb]));
+                    if constexpr (pin) asm volatile("" :: "v"(l_run[qb]));
+                    else l_run[qb] += sm[e];
                 }
             } else {
                 constexpr int qb = (o - 112) / 8, r = (o - 112) % 8;
                 const float16_t& sv = nxt[qb];
-                if constexpr (r < 5)       t3[qb][r] = fmaxf(fmaxf(sv[3 * r], sv[3 * r + 1]), sv[3 * r + 2]);
-                else if constexpr (r == 5) t3[qb][5] = fmaxf(fmaxf(t3[qb][0], t3[qb][1]), t3[qb][2]);
-                else if constexpr (r == 6) t3[qb][6] = fmaxf(fmaxf(t3[qb][3], t3[qb][4]), sv[15]);
-                else                       mx[qb] = fmaxf(t3[qb][5], t3[qb][6]);
-                if constexpr (r < 7) asm volatile("" : "+v"(t3[qb][r]));
-                else                 asm volatile("" : "+v"(mx[qb]));
+                if constexpr (pin) {
+                    if constexpr (r < 7) asm volatile("" :: "v"(t3[qb][r]));
+                    else                 asm volatile("" :: "v"(mx[qb]));
+                } else if constexpr (r < 5)  t3[qb][r] = max3(sv[3 * r], sv[3 * r + 1], sv[3 * r + 2]);
+                else if constexpr (r == 5)   t3[qb][5] = max3(t3[qb][0], t3[qb][1], t3[qb][2]);
+                else if constexpr (r == 6)   t3[qb][6] = max3(t3[qb][3], t3[qb][4], sv[15]);
+                else                         mx[qb] = fmaxf(t3[qb][5], t3[qb][6]);
             }
         };
         static_for<32>([&](auto U) {
             constexpr int u = decltype(U)::value;
-            if constexpr ((WIDE_KO & 32) == 0 || u >= 28)
-                static_for<4>([&](auto I) {
-                    constexpr int o = 4 * u + decltype(I)::value;
-                    if constexpr ((WIDE_KO & 64) == 0 || (o % 14 != 9 && o % 14 != 10 && o % 14 != 12 && o % 14 != 13) || o >= 112) valu_op(std::integral_constant<int, o>{});
-                });
+            static_for<4>([&](auto I) {
+                constexpr int o = 4 * u + decltype(I)::value;
+                valu_op(std::integral_constant<int, o>{}, No{});
+                valu_op(std::integral_constant<int, o - 1>{}, Yes{});
+            });
+            if constexpr (u == 31) valu_op(std::integral_constant<int, 127>{}, Yes{});
             if constexpr (u == 31) raise = wants_raise(mx);          // decided under the last MFMA, acted on after it
             // Two waits per block instead of one per MFMA (an instruction of any kind costs this
             // lone wavefront an issue slot): every request waited for here is eight MFMAs old.
@@ -350,7 +387,7 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
             } else {
                 constexpr int g = (u - 16) >> 2, qb = g & 1, s2 = g >> 1, db = (u - 16) & 3;
                 oacc[qb][db] = Mma<T>::run(vf[s2 * DBLK + db], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
-                if constexpr (u < 16 + KSTEPS) fetch_k(krows, u - 16);
+                if constexpr (u >= 32 - KSTEPS) fetch_k(krows, u - (32 - KSTEPS));   // (the first V fragments are dead by now: their registers take these)
             }
             if constexpr (kStage && u % 4 == 1) {
                 // the next tile pair (K tile t+2, V tile t+1), one request every fourth MFMA
@@ -363,29 +400,44 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
         });
         finish_scores(j + 1, nxt, mx, raise);
     };
-    using Yes = std::true_type;
-    using No  = std::false_type;
+    // Outputs of the item at hand: out = O / l, and the log-sum-exp if asked for.  A lane holds
+    // four consecutive columns of its query per accumulator group, i.e. 8-byte pieces of 32
+    // different rows per store: they are written to LDS instead (rows padded by 16 bytes, so one
+    // address register and immediate offsets do) and read back a row at a time, 16 bytes per
+    // lane, four rows per store instruction.
+    auto outputs_to_lds = [&](int ob, int ohq, int oq0) {
+        std::uint16_t* mine = o_lds + wave * WQ * OROW;
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            const float l_tot = half_swap_sum(l_run[qb]);
+            const float inv_l = 1.0f / l_tot;
+            const int row = 32 * qb + lq;
+#pragma unroll
+            for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = Mma<T>::pack2(oacc[qb][db][4 * g + 0] * inv_l, oacc[qb][db][4 * g + 1] * inv_l);
+                    w[1] = Mma<T>::pack2(oacc[qb][db][4 * g + 2] * inv_l, oacc[qb][db][4 * g + 3] * inv_l);
+                    *reinterpret_cast<u32x2*>(mine + row * OROW + (4 * db + g) * 8 + 4 * lh) = w;
+                }
+            const int my_q = oq0 + row;
+            if (p.lse != nullptr && lh == 0 && my_q < p.Lq)
+                p.lse[(static_cast<long>(ob) * p.Hq + ohq) * p.Lq + my_q] = m_run[qb] * p.scale + logf(l_tot);
+        }
+    };
+    auto outputs_to_memory = [&](int ob, int ohq, int oq0) {
+        const std::uint16_t* mine = o_lds + wave * WQ * OROW;
+        std::uint16_t* orow = p.out + ((static_cast<long>(ob) * p.Hq + ohq) * p.Lq + oq0) * D;
+#pragma unroll
+        for (int i = 0; i < WQ / 4; ++i) {
+            const int row = 4 * i + (lane >> 4), chunk = lane & 15;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(mine + row * OROW + chunk * 8);
+            if (oq0 + row < p.Lq) *reinterpret_cast<u32x4*>(orow + row * D + chunk * 8) = v;
+        }
+    };
 
     float16_t s_a[QB], s_b[QB];
-    {
-        // S(0) from the first half of K tile 0, then the keys of block 1 for block 0's score MFMAs
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) fetch_k(k_lds0, ks);
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) {
-                if (ks == 0) Mma<T>::score_first(s_a[qb], kf[0], qreg[qb][0]);
-                else         Mma<T>::score_acc(s_a[qb], kf[ks], qreg[qb][ks]);
-            }
-        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s_a[0]), "+v"(s_a[1]));
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) fetch_k(k_lds0 + 32 * D, ks);
-        float mx[QB];
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) mx[qb] = lane_max(s_a[qb]);
-        finish_scores(0, s_a, mx, wants_raise(mx));
-    }
     // Every tile runs the same two blocks, the last one included: its second block then forms
     // scores nobody uses (of keys past the end of K or past the diagonal; whatever the LDS rows
     // hold, they are masked to -inf before anything reads them), and a block that lies wholly past
@@ -396,43 +448,95 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
         block(2 * t + 1, s_b, s_a, par, No{});
         publish();
     };
-    for (int t = 0; t < wave_tiles; t += 2) {
-        tile(t, Par0{});
-        if (t + 1 >= wave_tiles) break;
-        tile(t + 1, Par1{});
-    }
-    for (int t = wave_tiles; t < n_tiles; ++t) {           // done early (causal): keep staging for the other wavefronts
-        stage_pair(t, AnyPar{t});
-        publish();
-    }
 
+    int round = 0;
+    {
+        int bh, qblock;
+        item_at(0, bh, qblock);          // the grid is never larger than the item count
+        enter_item(bh, qblock);
+        stage_first();
+        load_queries();
+    }
+    for (;;) {
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-        const int my_q = q0 + 32 * qb + lq;
-        const float l_tot = half_swap_sum(l_run[qb]);
-        const float inv_l = 1.0f / l_tot;
-        if (my_q < p.Lq) {
-            std::uint16_t* op = p.out + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q) * D;
+        for (int qb = 0; qb < QB; ++qb) {
+            l_run[qb] = 0.f;
 #pragma unroll
-            for (int db = 0; db < DBLK; ++db)
+            for (int i = 0; i < DBLK; ++i)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int d = db * 32 + g * 8 + 4 * lh;
-                    u32x2 w;
-                    w[0] = Mma<T>::pack2(oacc[qb][db][4 * g + 0] * inv_l, oacc[qb][db][4 * g + 1] * inv_l);
-                    w[1] = Mma<T>::pack2(oacc[qb][db][4 * g + 2] * inv_l, oacc[qb][db][4 * g + 3] * inv_l);
-                    *reinterpret_cast<u32x2*>(op + d) = w;
-                }
-            if (p.lse != nullptr && lh == 0)
-                p.lse[(static_cast<long>(b) * p.Hq + hq) * p.Lq + my_q] = m_run[qb] * p.scale + logf(l_tot);
+                for (int r = 0; r < 16; ++r) oacc[qb][i][r] = 0.f;
         }
+        publish();
+        {
+            // S(0) from the first half of K tile 0, then the keys of block 1 for block 0's score MFMAs
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) fetch_k(k_lds0, ks);
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                    if (ks == 0) Mma<T>::score_first(s_a[qb], kf[0], qreg[qb][0]);
+                    else         Mma<T>::score_acc(s_a[qb], kf[ks], qreg[qb][ks]);
+                }
+            asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s_a[0]), "+v"(s_a[1]));   // MFMA results the compiler cannot see coming
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) fetch_k(k_lds0 + 32 * D, ks);
+            // The first reference point is the maximum of block 0 itself: nothing to rescale yet.
+            // (Every query sees key 0, so the maximum is finite.)
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                if (needs_mask(0, qb)) apply_mask(0, qb, s_a[qb]);
+                m_run[qb] = half_swap_max(lane_max(s_a[qb]));
+            }
+        }
+        for (int t = 0; t < wave_tiles; t += 2) {
+            tile(t, Par0{});
+            if (t + 1 >= wave_tiles) break;
+            tile(t + 1, Par1{});
+        }
+        // A wavefront that is done before the others (causal: its diagonal comes first) sends its
+        // rows off now, under their MFMAs, and then keeps staging tiles for them.
+        const bool early = wave_tiles < n_tiles;
+        const int ob = b, ohq = hq, oq0 = q0;
+        if ((WIDE_KO & 128) == 0 && early) {
+            outputs_to_lds(ob, ohq, oq0);
+            outputs_to_memory(ob, ohq, oq0);
+        }
+        for (int t = wave_tiles; t < n_tiles; ++t) {
+            stage_pair(t, AnyPar{t});
+            publish();
+        }
+        // Nobody reads the tiles of this item any more: ask for the next item's first tiles and
+        // queries, and let them travel while the outputs of this one are normalised and stored.
+        int bh, qblock;
+        const bool more = item_at(++round, bh, qblock);
+        if (more) {
+            enter_item(bh, qblock);
+            if constexpr ((WIDE_KO & 512) == 0) stage_first();
+            if constexpr ((WIDE_KO & 256) == 0) load_queries();
+        }
+        if ((WIDE_KO & 128) == 0 && !early) {
+            outputs_to_lds(ob, ohq, oq0);
+            outputs_to_memory(ob, ohq, oq0);
+        }
+        if (!more) break;
+        // (the queries belong in AGPRs from here on: say so, or the allocator keeps half of them in VGPRs
+        // and copies four registers in front of every score MFMA)
+        asm volatile("" : "+a"(qreg[0][0]), "+a"(qreg[0][1]), "+a"(qreg[0][2]), "+a"(qreg[0][3]), "+a"(qreg[0][4]), "+a"(qreg[0][5]), "+a"(qreg[0][6]), "+a"(qreg[0][7]),
+                          "+a"(qreg[1][0]), "+a"(qreg[1][1]), "+a"(qreg[1][2]), "+a"(qreg[1][3]), "+a"(qreg[1][4]), "+a"(qreg[1][5]), "+a"(qreg[1][6]), "+a"(qreg[1][7]));
     }
 }
 
 template <typename T>
 int launch_t(FlashParams p, bool causal, hipStream_t s) {
     p.n_qblocks = (p.Lq + kWideBM - 1) / kWideBM;
-    const long blocks = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
+    const long items = static_cast<long>(p.B) * p.Hq * p.n_qblocks;
+    // one workgroup per CU (that is all its LDS and registers hold), each walking its share of the items
+    int dev = 0, cus = 0;
+    PARAS_HIP_TRY(hipGetDevice(&dev));
+    PARAS_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    long blocks = items < cus ? items : cus;
+    if (blocks >= 8 && (static_cast<long>(p.B) * p.Hq) % 8 == 0) blocks -= blocks % 8;
     const dim3 grid(static_cast<unsigned>(blocks)), wg(256);
     if (causal) hipLaunchKernelGGL((flash_wide_kernel<T, true>), grid, wg, 0, s, p);
     else        hipLaunchKernelGGL((flash_wide_kernel<T, false>), grid, wg, 0, s, p);
