@@ -164,7 +164,7 @@ def main() -> int:
         q, k, v = qc.to(dev), kc.to(dev), vc.to(dev)
         out = torch.empty_like(q)
         a = capi.sdpa_args(q, k, v, out, is_causal=True)
-        assert L.paras_sdpa_kernel_name(C.byref(a)) == b"flash_mfma"
+        assert L.paras_sdpa_kernel_name(C.byref(a)).startswith(b"flash_mfma")
         ms, wall = timer.run(lambda i: must(L.paras_sdpa_fwd(C.byref(a), None, st)), steps, warmup, SETTLE_MFMA_MS)
         flops = 4 * B * H * S * S * D / 2          # causal-halved
         tf = flops / ms / 1e9

@@ -119,7 +119,7 @@ const char* paras_sdpa_kernel_name(const paras_sdpa_args* args) {
     using namespace paras;
     if (validate(args) != PARAS_OK) return "invalid";
     switch (choose(*args)) {
-        case SdpaKernel::Flash:  return "flash_mfma";
+        case SdpaKernel::Flash:  return flash_uses_wide(*args) ? "flash_mfma_wide" : "flash_mfma";
         case SdpaKernel::Decode: return "decode_split";
         case SdpaKernel::Weights: return "math_mfma";
         case SdpaKernel::Padded: return "padded_mfma";

@@ -590,6 +590,10 @@ bool flash_supported(const paras_sdpa_args& a) {
     return true;
 }
 
+bool flash_uses_wide(const paras_sdpa_args& a) {
+    return flash::wide_supported(a.B, a.Hq, a.Lq, a.Lk, static_cast<int>(a.D), a.mask_kind, a.is_causal != 0);
+}
+
 int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     FlashParams p;
     p.q = static_cast<const std::uint16_t*>(a.q);
@@ -610,7 +614,7 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     p.inv_scale = static_cast<float>(1.0 / a.scale);
     const bool causal = a.is_causal != 0;
     const int mk = a.mask_kind;
-    if (wide_supported(p, static_cast<int>(a.D), mk)) return launch_flash_wide(p, causal, a.dtype == PARAS_BF16, s);
+    if (flash_uses_wide(a)) return launch_flash_wide(p, causal, a.dtype == PARAS_BF16, s);
     if (a.dtype == PARAS_BF16)
         return a.D == 128 ? launch_t<bf16_t, 128>(p, causal, mk, s) : launch_t<bf16_t, 64>(p, causal, mk, s);
     return a.D == 128 ? launch_t<f16_t, 128>(p, causal, mk, s) : launch_t<f16_t, 64>(p, causal, mk, s);

@@ -35,6 +35,7 @@ struct FlashParams {
     const unsigned char* mask;
     long ms_b, ms_h, ms_q, ms_k;
     float inv_scale;   // the scores are kept unscaled: an additive mask value m enters as m / scale
+    unsigned magic_nq, magic_hq, magic_rep;   // ceil(2^32 / d) for d = n_qblocks, Hq, Hq / Hkv (set by the wide kernel's launcher)
 };
 
 template <typename T> struct Mma;
@@ -131,7 +132,7 @@ __device__ __forceinline__ void map_workgroup(int idx, int BH, int nq, int& bh, 
 
 // 64 queries per wavefront (sdpa_flash_wide.hip): head size 128, causal or unmasked.
 constexpr int kWideBM = 256;   // queries per workgroup of that kernel
-bool wide_supported(const FlashParams& p, int D, int mask_kind);
+bool wide_supported(long B, long Hq, long Lq, long Lk, int D, int mask_kind, bool causal);
 int  launch_flash_wide(FlashParams p, bool causal, bool is_bf16, hipStream_t s);
 
 }  // namespace flash

@@ -56,9 +56,6 @@ namespace paras {
 namespace flash {
 namespace {
 
-#ifndef WIDE_KO
-#define WIDE_KO 0
-#endif
 constexpr int D      = 128;
 constexpr int QB     = 2;            // 32-query blocks per wavefront
 constexpr int NW     = 4;
@@ -131,10 +128,12 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     const int pool_wgs = by_xcd ? n_wg >> 3 : n_wg;
     const int pool_pos = by_xcd ? wg_id >> 3 : wg_id;
     const int pool_items = (by_xcd ? BH >> 3 : BH) * nq;
+    // (x / d as a multiply-high by ceil(2^32 / d): exact while x * d < 2^32, which the launcher checks)
+    auto fast_div = [](int x, unsigned magic) { return static_cast<int>(__umulhi(static_cast<unsigned>(x), magic)); };
     auto item_at = [&](int round, int& bh, int& qblock) {
         const int i = round * pool_wgs + ((round & 1) ? pool_wgs - 1 - pool_pos : pool_pos);
         if (i >= pool_items) return false;
-        const int head = i / nq, pos = i - head * nq;
+        const int head = nq == 1 ? i : fast_div(i, p.magic_nq), pos = i - head * nq;
         bh = by_xcd ? head * 8 + (wg_id & 7) : head;
         qblock = kCausal ? nq - 1 - pos : pos;
         return true;
@@ -161,9 +160,9 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     };
     // Everything that depends on the item.
     auto enter_item = [&](int bh, int qblock) {
-        b = bh / p.Hq;
+        b = p.Hq == 1 ? bh : fast_div(bh, p.magic_hq);
         hq = bh - b * p.Hq;
-        const int hkv = hq / (p.Hq / p.Hkv);
+        const int hkv = p.Hq == p.Hkv ? hq : fast_div(hq, p.magic_rep);
         q0 = qblock * kWideBM + wave * WQ;   // query block qb of this wavefront starts at q0 + 32 qb
         k_rsrc = make_rsrc(p.k + b * p.ks_b + hkv * p.ks_h, k_row_bytes);
         v_rsrc = make_rsrc(p.v + b * p.vs_b + hkv * p.vs_h, v_row_bytes);
@@ -187,7 +186,6 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     const int v_lane = srow * v_row_bytes + ((slot ^ vsw(srow)) * 16);
     typedef __attribute__((address_space(3))) void* lptr_t;
     auto stage_one = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile, int i) {
-        if constexpr ((WIDE_KO & 2) != 0) { if (first > kBN) return; }
         const int r0 = i * RPI * NW;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)(tile + (r0 + wave * RPI) * D), 16,
                                                  lane_off + (first + r0) * row_bytes, 0, 0, 0);
@@ -203,8 +201,8 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
         stage_rows(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true));
     };
     auto publish = [&]() {
-        if constexpr ((WIDE_KO & 8) == 0) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tiles has landed
-        if constexpr ((WIDE_KO & 1) == 0) __syncthreads();
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's part of the tiles has landed
+        __syncthreads();
     };
 
     float16_t oacc[QB][DBLK];
@@ -291,9 +289,8 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     // Operand fragments: kf = the K rows of the block whose scores come next, vf = the V rows of
     // the block whose probabilities are applied now.
     i16x8 kf[KSTEPS], vf[2 * DBLK];
-    auto fetch_k = [&](const std::uint16_t* rows, int ks) { if constexpr ((WIDE_KO & 4) != 0) { if (rows != k_lds0) return; } kf[ks] = *reinterpret_cast<const i16x8*>(rows + k_rd[ks]); };
+    auto fetch_k = [&](const std::uint16_t* rows, int ks) { kf[ks] = *reinterpret_cast<const i16x8*>(rows + k_rd[ks]); };
     auto fetch_v = [&](const std::uint16_t* rows, int f) {     // f = 4 * (16-key half) + column block
-        if constexpr ((WIDE_KO & 4) != 0) { if (rows != v_lds0) return; }
         const std::uint16_t* vp = rows + v_rd[f % DBLK] + 16 * (f / DBLK) * D;
         const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp));
         const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(vp + 8 * D));
@@ -344,7 +341,7 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
                 if constexpr (r < 8) {
                     if constexpr (pin) asm volatile("" :: "v"(ex[e][w & 1]));
                     else if constexpr (w < 2) ex[e][w] = fmaf(cur[qb][2 * i + w], p.scale_log2, -mc[qb]);
-                    else if constexpr ((WIDE_KO & 16) == 0) ex[e][w - 2] = __builtin_amdgcn_exp2f(ex[e][w - 2]);
+                    else ex[e][w - 2] = __builtin_amdgcn_exp2f(ex[e][w - 2]);
                 } else if constexpr (w == 0) {
                     if constexpr (pin) asm volatile("" :: "v"(pw[qb][i / 4][i % 4]));
                     else pw[qb][i / 4][i % 4] = Mma<T>::pack2(ex[e][0], ex[e][1]);
@@ -498,7 +495,7 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
         // rows off now, under their MFMAs, and then keeps staging tiles for them.
         const bool early = wave_tiles < n_tiles;
         const int ob = b, ohq = hq, oq0 = q0;
-        if ((WIDE_KO & 128) == 0 && early) {
+        if (early) {
             outputs_to_lds(ob, ohq, oq0);
             outputs_to_memory(ob, ohq, oq0);
         }
@@ -506,18 +503,23 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
             stage_pair(t, AnyPar{t});
             publish();
         }
-        // Nobody reads the tiles of this item any more: ask for the next item's first tiles and
-        // queries, and let them travel while the outputs of this one are normalised and stored.
+        // Nobody reads the tiles of this item any more.
+        // Order of the hand-over: the next queries are requested first (registers, the longest
+        // latency), then this item's outputs go through the wavefront's own LDS region (an LDS read
+        // issued while a dozen direct-to-LDS loads are in flight would wait for them), and only then
+        // the next item's first tiles are requested.
         int bh, qblock;
         const bool more = item_at(++round, bh, qblock);
         if (more) {
             enter_item(bh, qblock);
-            if constexpr ((WIDE_KO & 512) == 0) stage_first();
-            if constexpr ((WIDE_KO & 256) == 0) load_queries();
+            load_queries();
         }
-        if ((WIDE_KO & 128) == 0 && !early) {
+        if (!early) {
             outputs_to_lds(ob, ohq, oq0);
             outputs_to_memory(ob, ohq, oq0);
+        }
+        if (more) {
+            stage_first();
         }
         if (!more) break;
         // (the queries belong in AGPRs from here on: say so, or the allocator keeps half of them in VGPRs
@@ -535,6 +537,10 @@ int launch_t(FlashParams p, bool causal, hipStream_t s) {
     int dev = 0, cus = 0;
     PARAS_HIP_TRY(hipGetDevice(&dev));
     PARAS_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    auto magic = [](long d) { return static_cast<unsigned>(((1ull << 32) + static_cast<unsigned long long>(d) - 1) / static_cast<unsigned long long>(d)); };
+    p.magic_nq = magic(p.n_qblocks);
+    p.magic_hq = magic(p.Hq);
+    p.magic_rep = magic(p.Hq / p.Hkv);
     long blocks = items < cus ? items : cus;
     if (blocks >= 8 && (static_cast<long>(p.B) * p.Hq) % 8 == 0) blocks -= blocks % 8;
     const dim3 grid(static_cast<unsigned>(blocks)), wg(256);
@@ -546,11 +552,21 @@ int launch_t(FlashParams p, bool causal, hipStream_t s) {
 
 }  // namespace
 
-bool wide_supported(const FlashParams& p, int head, int mask_kind) {
+bool wide_supported(long B, long Hq, long Lq, long Lk, int head, int mask_kind, bool causal) {
     static const int forced = [] { const char* e = std::getenv("PARAS_FLASH_WIDE"); return e ? std::atoi(e) : -1; }();
     if (head != D || mask_kind != 0) return false;
+    // the item arithmetic divides by multiply-high: exact while dividend * divisor < 2^32
+    const unsigned long long nq = (static_cast<unsigned long long>(Lq) + kWideBM - 1) / kWideBM;
+    const unsigned long long bh = static_cast<unsigned long long>(B) * static_cast<unsigned long long>(Hq);
+    if (bh * nq * nq >= (1ull << 32) || bh * static_cast<unsigned long long>(Hq) >= (1ull << 32)) return false;
     if (forced >= 0) return forced != 0;
-    return false;   // opt-in (PARAS_FLASH_WIDE=1) until it wins on the causal shapes too
+    // One workgroup per CU and 256 queries per item: it needs a few items per CU to keep them all
+    // busy and, under the causal rule, long rows for the items' fixed cost to pay off (measured
+    // against the 32-queries-per-wavefront kernel: ahead from 4096 causal / 1024 unmasked queries on).
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return false;
+    if (bh * nq < 2ull * static_cast<unsigned long long>(cus)) return false;
+    return causal ? (Lq >= 4096 && Lk >= 4096) : (Lq >= 1024 && Lk >= 1024);
 }
 
 int launch_flash_wide(FlashParams p, bool causal, bool is_bf16, hipStream_t s) {

@@ -12,6 +12,9 @@ namespace paras {
 // (causal or none), no attention weights returned.
 bool flash_supported(const paras_sdpa_args& a);
 int  launch_flash(const paras_sdpa_args& a, hipStream_t s);
+// Whether launch_flash takes its 64-queries-per-wavefront form (head size 128, no mask, enough
+// long rows to fill the chip with one workgroup per CU); only meaningful when flash_supported.
+bool flash_uses_wide(const paras_sdpa_args& a);
 
 // Split-KV decode: short query (Lq * Hq/Hkv <= 16), long K/V, bf16/f16,
 // D == Dv in {64, 128}, optional bool / additive mask, not causal.

@@ -235,7 +235,9 @@ typedef struct paras_sdpa_args {
 PARAS_API size_t paras_sdpa_workspace(const paras_sdpa_args* args);
 /* `workspace` may be NULL when paras_sdpa_workspace() returned 0. */
 PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void* stream);
-/* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma", "decode_split",
+/* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma" ("flash_mfma_wide"
+ * where its 64-queries-per-wavefront form runs: head size 128, no mask, at least
+ * two 256-query tiles per CU, rows of 4096 causal / 1024 unmasked on), "decode_split",
  * "math_mfma" (bf16 / f16 with the weights returned), "padded_mfma" (bf16 / f16
  * head sizes below 128 other than 64: q, k, v copied into the workspace with
  * zero columns up to 64 or 128, then flash_mfma / decode_split; the workspace

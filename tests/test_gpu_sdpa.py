@@ -76,9 +76,9 @@ def test_golden_vectors_generic_kernel(tag):
 def test_golden_vectors_mfma_kernels(tag):
     c = case(f"sdpa_d128_{tag}")
     out, _, _, kern = run(c["q"], c["k"], c["v"], is_causal=True)
-    assert kern == "flash_mfma" and max_abs(out, c["out_causal"]) <= ABS_16BIT
+    assert kern.startswith("flash_mfma") and max_abs(out, c["out_causal"]) <= ABS_16BIT
     out, _, _, kern = run(c["q"], c["k"], c["v"])
-    assert kern == "flash_mfma" and max_abs(out, c["out_plain"]) <= ABS_16BIT
+    assert kern.startswith("flash_mfma") and max_abs(out, c["out_plain"]) <= ABS_16BIT
     d = case(f"sdpa_decode_{tag}")
     out, _, _, kern = run(d["q"], c["k"], c["v"])
     assert kern == "decode_split" and max_abs(out, d["out"]) <= ABS_16BIT
@@ -109,7 +109,7 @@ def test_flash_matches_oracle(dtype, shape):
     q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
     out, _, lse, kern = run(q, k, v, is_causal=causal, want_lse=True)
     want, _ = O.sdpa_math(q, k, v, is_causal=causal, enable_gqa=True, gemm="aten")
-    assert kern == "flash_mfma"
+    assert kern.startswith("flash_mfma")
     assert max_abs(out, want) <= ABS_16BIT, f"{shape} {dtype}"
     rep = Hq // Hkv
     s = (q.float() @ k.float().repeat_interleave(rep, 1).transpose(-1, -2)) / math.sqrt(D)
@@ -134,7 +134,7 @@ def test_flash_accuracy_with_large_scores(dtype):
         v = torch.randn(B, H, S, D).to(dtype)
         for causal in (True, False):
             out, _, lse, kern = run(q, k, v, is_causal=causal, want_lse=True)
-            assert kern == "flash_mfma"
+            assert kern.startswith("flash_mfma")
             s = (q.double() @ k.double().transpose(-1, -2)) / math.sqrt(D)
             if causal:
                 s = s.masked_fill(~torch.ones(S, S).tril().bool(), -math.inf)
@@ -154,7 +154,7 @@ def test_flash_strided_inputs_and_explicit_scale():
     dqv, dkv, dvv = (dq[:, :, i].permute(0, 2, 1, 3) for i in range(3))
     out, _, _, kern = capi.sdpa(dqv, dkv, dvv, is_causal=True, scale=0.05)
     want, _ = O.sdpa_math(q.contiguous(), k.contiguous(), v.contiguous(), is_causal=True, scale=0.05, gemm="aten")
-    assert kern == "flash_mfma" and max_abs(out, want) <= ABS_16BIT
+    assert kern.startswith("flash_mfma") and max_abs(out, want) <= ABS_16BIT
 
 
 @pytest.mark.parametrize("Lk", [77, 191, 300])
@@ -170,7 +170,7 @@ def test_flash_never_reads_past_the_last_key(Lk):
     for causal in (False, True):
         out, _, _, kern = capi.sdpa(q.cuda(), kbuf[:, :, :Lk], vbuf[:, :, :Lk], is_causal=causal)
         want, _ = O.sdpa_math(q, k, v, is_causal=causal, gemm="aten")
-        assert kern == "flash_mfma"
+        assert kern.startswith("flash_mfma")
         assert bool(torch.isfinite(out).all()) and max_abs(out, want) <= ABS_16BIT
 
 
@@ -181,7 +181,7 @@ def test_flash_broadcast_key_rows():
     k1, v1 = torch.randn(B, H, 1, D).half(), torch.randn(B, H, 1, D).half()
     out, _, _, kern = capi.sdpa(q.cuda(), k1.cuda().expand(B, H, Lk, D), v1.cuda().expand(B, H, Lk, D), is_causal=False)
     want, _ = O.sdpa_math(q, k1.expand(B, H, Lk, D).contiguous(), v1.expand(B, H, Lk, D).contiguous(), gemm="aten")
-    assert kern == "flash_mfma" and max_abs(out, want) <= ABS_16BIT
+    assert kern.startswith("flash_mfma") and max_abs(out, want) <= ABS_16BIT
 
 
 def test_flash_random_shapes_layouts_and_padding():
@@ -218,7 +218,7 @@ def test_flash_random_shapes_layouts_and_padding():
             s = s.masked_fill(~torch.ones(Lq, Lk, device="cuda").tril().bool(), -math.inf)
         want = torch.softmax(s, -1) @ v.float().repeat_interleave(rep, 1)
         case_id = f"B={B} Hq={Hq} Hkv={Hkv} Lq={Lq} Lk={Lk} D={D} {dt} causal={causal} {layout} scale={scale}"
-        assert kern in ("flash_mfma", "decode_split"), case_id     # a handful of queries goes to the decode kernel
+        assert kern in ("flash_mfma", "flash_mfma_wide", "decode_split"), case_id     # a handful of queries goes to the decode kernel
         assert bool(torch.isfinite(out).all()) and float((out.float() - want).abs().max()) <= ABS_16BIT, case_id
 
 
@@ -252,7 +252,7 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
         mask = (torch.randn(mshape) * 0.5).masked_fill(~keep, -math.inf).to(dtype)
     out, _, _, kern = run(q, k, v, mask=mask)
     want, _ = O.sdpa_math(q, k, v, attn_mask=mask, enable_gqa=True, gemm="aten")
-    assert kern == "flash_mfma"
+    assert kern.startswith("flash_mfma")
     if dead_row is not None:
         assert bool(out[:, :, dead_row].isnan().all()) and bool(want[:, :, dead_row].isnan().all())
         rows = [i for i in range(Lq) if i != dead_row]
@@ -468,7 +468,7 @@ def test_config3_shape_properties_and_slice():
     q, k, v = torch.randn(B, H, S, D).bfloat16(), torch.randn(B, H, S, D).bfloat16(), torch.randn(B, H, S, D).bfloat16()
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     out, _, lse, kern = capi.sdpa(qd, kd, vd, is_causal=True, want_lse=True)
-    assert kern == "flash_mfma"
+    assert kern == "flash_mfma_wide"        # 2048 tiles of 256 queries for 256 CUs
     want, _ = O.sdpa_math(q[:1, :2], k[:1, :2], v[:1, :2], is_causal=True, gemm="aten")
     assert max_abs(out[:1, :2], want) <= ABS_16BIT
     # rows 3000..3063 of the last head: causal == an explicit lower-triangular mask on those rows
@@ -484,6 +484,40 @@ def test_config3_shape_properties_and_slice():
     o2, _, _, _ = capi.sdpa(qd, kd, v2, is_causal=True)
     o12, _, _, _ = capi.sdpa(qd, kd, (vd.float() + v2.float()).bfloat16(), is_causal=True)
     assert (o12.float() - (out.float() + o2.float())).abs().max().item() <= 6e-2
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Lq,Lk,causal,dtype", [
+    (4, 32, 8, 1024, 1024, False, torch.bfloat16),      # grouped heads, two tiles per CU
+    (4, 32, 32, 1100, 1300, False, torch.bfloat16),     # neither length a multiple of the tile sizes
+    (5, 27, 27, 1024, 2000, False, torch.float16),      # a head count that does not divide by 8
+    (1, 32, 8, 4096, 4096, True, torch.bfloat16),       # causal, two items per workgroup
+    (2, 16, 4, 4100, 4200, True, torch.float16),        # causal, ragged last tile, Lq != Lk
+])
+def test_flash_wide_kernel_matches_oracle(B, Hq, Hkv, Lq, Lk, causal, dtype):
+    """The 64-queries-per-wavefront form of the flash kernel (one workgroup per CU walking a
+    list of 256-query items) at shapes where paras_sdpa_fwd picks it: sampled heads against the
+    oracle, the log-sum-exp against fp64, strided inputs against contiguous ones."""
+    torch.manual_seed(Lq + Lk)
+    q, k, v = torch.randn(B, Hq, Lq, 128).to(dtype), torch.randn(B, Hkv, Lk, 128).to(dtype), torch.randn(B, Hkv, Lk, 128).to(dtype)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    out, _, lse, kern = capi.sdpa(qd, kd, vd, is_causal=causal, want_lse=True)
+    assert kern == "flash_mfma_wide"
+    assert not bool(out.isnan().any())
+    rep = Hq // Hkv
+    for b, h in ((0, 0), (B - 1, Hq - 1), (B // 2, Hq // 2 + 1)):
+        hk = h // rep
+        want, _ = O.sdpa_math(q[b:b + 1, h:h + 1], k[b:b + 1, hk:hk + 1], v[b:b + 1, hk:hk + 1], is_causal=causal, gemm="aten")
+        assert max_abs(out[b:b + 1, h:h + 1], want) <= ABS_16BIT, (b, h)
+        s = (q[b, h].double() @ k[b, hk].double().T) / math.sqrt(128)
+        if causal:
+            s = s.masked_fill(~torch.ones(Lq, Lk).tril().bool(), -math.inf)
+        assert torch.allclose(lse[b, h].double().cpu(), torch.logsumexp(s, -1), rtol=0, atol=5e-4), (b, h)
+    # the same call on inputs with padded rows and a transposed batch / head order
+    qs = torch.empty(Hq, B, Lq, 160, dtype=dtype, device="cuda").permute(1, 0, 2, 3)[..., :128]
+    ks = torch.empty(B, Hkv, Lk, 136, dtype=dtype, device="cuda")[..., :128]
+    qs.copy_(qd); ks.copy_(kd)
+    out2, _, _, kern2 = capi.sdpa(qs, ks, vd, is_causal=causal)
+    assert kern2 == "flash_mfma_wide" and torch.equal(out2, out)
 
 
 def test_config4_shape_slice_and_gqa_equivalence():
