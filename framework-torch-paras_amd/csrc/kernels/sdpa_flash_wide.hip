@@ -449,7 +449,7 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     int round = 0;
     {
         int bh, qblock;
-        item_at(0, bh, qblock);          // the grid is never larger than the item count
+        if (!item_at(0, bh, qblock)) return;   // (the grid is never larger than the item count: not expected)
         enter_item(bh, qblock);
         stage_first();
         load_queries();
