@@ -42,7 +42,7 @@ import time
 from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
-for p in (ROOT / "tests", ROOT / "oracle"):
+for p in (ROOT / "framework-torch-paras_amd", ROOT / "oracle"):
     if str(p) not in sys.path:
         sys.path.insert(0, str(p))
 
@@ -120,7 +120,7 @@ def main() -> int:
         return 2
 
     import torch
-    import capi
+    import paras_capi as capi
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)

@@ -185,8 +185,17 @@ __global__ __launch_bounds__(kBlock) void route_scatter_kernel(const long* __res
 constexpr int  kScratchHeader   = 256;
 constexpr int  kFusedMaxBlocks  = 256;          // 256-thread workgroups: all resident on 256 CUs
 constexpr long kFusedMaxTokens  = static_cast<long>(kFusedMaxBlocks) * kBlock;
-constexpr int  kSpinLimit       = 1 << 15;      // polls of a word, each a round trip to memory: tens of milliseconds, then the workgroup counts for itself
+// How long a workgroup waits for the others' counts before it counts for itself: by the clock
+// (wall_clock64 ticks at 100 MHz), about what the recount costs, so that a grid kept off the chip
+// by other work turns a 9 us call into a few hundred microseconds, not tens of milliseconds.
+// PARAS_ROUTE_SPIN_LIMIT (a number of polls) is a test hook that forces the recount.
+constexpr unsigned kWaitTicks   = 30000;        // 300 us
+constexpr int  kSpinLimit       = 1 << 30;
 constexpr int  kEpochShift      = 16;           // a workgroup's count is at most kBlock
+
+// Workgroups that stopped waiting and counted for themselves, since the module was loaded
+// (read through paras_moe_route_give_ups: a number that grows says the chip is oversubscribed).
+static __device__ unsigned long long route_give_ups = 0;
 
 __global__ __launch_bounds__(kBlock) void route_clear_kernel(unsigned long long* __restrict__ words, long n) {
     const long i = static_cast<long>(blockIdx.x) * kBlock + threadIdx.x;
@@ -198,7 +207,7 @@ template <typename T, bool kSmall>
 __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     const typename Elem<T>::store_t* __restrict__ logits, long T_, int E, int k, long* __restrict__ topi,
     float* __restrict__ topw, long* __restrict__ order, long* __restrict__ inv_order, long* __restrict__ counts,
-    long* __restrict__ offsets, unsigned char* __restrict__ scratch, unsigned long long epoch, int spin_limit) {
+    long* __restrict__ offsets, unsigned char* __restrict__ scratch, unsigned long long epoch, int spin_limit, unsigned wait_ticks) {
     using El = Elem<T>;
     __shared__ int wave_cnt[kWavesPerBlock][kMaxExperts];
     __shared__ long tot[kMaxExperts + 1];     // after the meeting: exclusive expert offsets
@@ -338,12 +347,13 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     {
         bool ran_out = false;
         const long n_words = static_cast<long>(nblk) * E;
+        const unsigned long long t_start = wall_clock64();
         for (long i = tid; i < n_words; i += kBlock) {
             const unsigned long long* wp = &words[i];
             unsigned long long w = __hip_atomic_load(wp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             int polls = 1;
             while ((w >> kEpochShift) != epoch) {
-                if (polls >= spin_limit) {
+                if (polls >= spin_limit || wall_clock64() - t_start > wait_ticks) {
                     ran_out = true;
                     break;
                 }
@@ -360,6 +370,7 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
         if (ran_out) gave_up = 1;
     }
     __syncthreads();
+    if (gave_up && tid == 0) atomicAdd(&route_give_ups, 1ull);
 
     // ---- totals (expert offsets) and the share of the workgroups before this one ---------
     if (gave_up) {
@@ -452,7 +463,7 @@ void launch_fused(const void* logits, long T_, int E, int k, long* topi, float* 
     const dim3 grid(static_cast<unsigned>(nblk)), block(kBlock);
     // PARAS_ROUTE_SPIN_LIMIT: polls before a workgroup stops waiting for the others (tests set 1 to
     // drive the workgroups through the path that counts for itself)
-    const char* env = std::getenv("PARAS_ROUTE_SPIN_LIMIT");
+    const char* env = std::getenv("PARAS_ROUTE_SPIN_LIMIT");   // (looked up per call: the tests switch it between calls)
     const int spin = env != nullptr && std::atoi(env) > 0 ? std::atoi(env) : kSpinLimit;
     if (epoch == 0) {
         const long n_words = nblk * E;
@@ -462,10 +473,10 @@ void launch_fused(const void* logits, long T_, int E, int k, long* topi, float* 
     }
     if (E <= 8 && k <= 8)
         hipLaunchKernelGGL((route_fused_kernel<T, true>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, epoch, spin);
+                           topw, order, inv_order, counts, offsets, scratch, epoch, spin, kWaitTicks);
     else
         hipLaunchKernelGGL((route_fused_kernel<T, false>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, epoch, spin);
+                           topw, order, inv_order, counts, offsets, scratch, epoch, spin, kWaitTicks);
 }
 
 // Shared by the entry points: routes on `scratch` (device memory of route_scratch_bytes(T, E)).
@@ -519,19 +530,23 @@ int static_scratch_for(unsigned char** out) {
 
 // ---------------------------------------------------------------------------------------
 // The library's own scratch for paras_moe_route: kEpochSlots areas per GPU that only
-// route_fused_kernel ever writes (zero when the module is loaded), handed out in turn so that
-// calls running side by side on different streams rarely share one.  If two launches do share
-// an area, each sees the other's epoch in some words, waits its polls out and counts for itself:
-// slow, never wrong.  As for `scratch`, host code uses the per-device address only.
-constexpr int kEpochSlots = 4;
+// route_fused_kernel ever writes (zero when the module is loaded), one per stream by a hash of the
+// stream handle: calls on one stream run one after the other anyway, calls on different streams
+// rarely share an area.  If two launches do share one, each sees the other's epoch in some words,
+// waits its time out and counts for itself: slower, never wrong.  As for `scratch`, host code
+// uses the per-device address only.
+constexpr int kEpochSlots = 8;
 static __device__ __align__(256) unsigned char epoch_scratch[kEpochSlots * kStaticScratchBytes];
 unsigned char* g_epoch_scratch_ptr[kMaxGpus] = {};
 std::atomic<unsigned long long> g_epoch{2};        // 0: "clear first", 1: the epoch of a cleared area
-std::atomic<unsigned> g_epoch_slot{0};
 
-int epoch_scratch_for(unsigned char** out) {
+int epoch_scratch_for(hipStream_t s, unsigned char** out) {
     int dev = -1;
-    PARAS_HIP_TRY(hipGetDevice(&dev));
+    // the device the launch goes to: the stream's, or the current one for the null stream
+    if (s == nullptr || hipStreamGetDevice(s, &dev) != hipSuccess) {
+        (void)hipGetLastError();
+        PARAS_HIP_TRY(hipGetDevice(&dev));
+    }
     if (dev < 0 || dev >= kMaxGpus) {
         *out = nullptr;          // beyond the table: the caller's workspace serves
         return PARAS_OK;
@@ -543,12 +558,16 @@ int epoch_scratch_for(unsigned char** out) {
         if (ptr == nullptr) return fail(PARAS_ERR_HIP, "paras_moe_route: no device address for the routing scratch");
         g_epoch_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
     }
-    *out = g_epoch_scratch_ptr[dev];
+    const uintptr_t h = reinterpret_cast<uintptr_t>(s);
+    const size_t slot = static_cast<size_t>(((h >> 4) * 0x9E3779B97F4A7C15ull) >> 61);   // top three bits: kEpochSlots == 8
+    static_assert(kEpochSlots == 8, "the hash above yields three bits");
+    *out = g_epoch_scratch_ptr[dev] + slot * kStaticScratchBytes;
     return PARAS_OK;
 }
 
 // True when work queued on `s` now is being recorded into a graph (or that cannot be told).
 bool stream_is_capturing(hipStream_t s) {
+    if (s == nullptr) return false;   // the null stream cannot be captured, and asking would disturb a capture elsewhere
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(s, &status) != hipSuccess) {
         (void)hipGetLastError();
@@ -561,6 +580,15 @@ bool stream_is_capturing(hipStream_t s) {
 }  // namespace paras
 
 extern "C" {
+
+int paras_moe_route_give_ups(uint64_t* count) {
+    using namespace paras;
+    PARAS_REQUIRE(count != nullptr, "paras_moe_route_give_ups: null pointer");
+    unsigned long long n = 0;
+    PARAS_HIP_TRY(hipMemcpyFromSymbol(&n, HIP_SYMBOL(route_give_ups), sizeof(n)));
+    *count = n;
+    return PARAS_OK;
+}
 
 size_t paras_moe_route_workspace(int64_t T, int64_t E, int64_t k) {
     (void)k;
@@ -600,10 +628,10 @@ int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dty
         const char* own = std::getenv("PARAS_ROUTE_OWN_SCRATCH");
         if ((own == nullptr || std::atoi(own) != 0) && !stream_is_capturing(s)) {
             unsigned char* base = nullptr;
-            rc = epoch_scratch_for(&base);
+            rc = epoch_scratch_for(s, &base);
             if (rc != PARAS_OK) return rc;
             if (base != nullptr) {
-                area = base + static_cast<size_t>(g_epoch_slot.fetch_add(1, std::memory_order_relaxed) % kEpochSlots) * kStaticScratchBytes;
+                area = base;
                 epoch = g_epoch.fetch_add(1, std::memory_order_relaxed);
             }
         }

@@ -27,16 +27,18 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / kWave;
-constexpr long kScoreCapDefault = 1L << 28;      // score elements held at a time (1 GiB of fp32)
-// PARAS_SDPA_SCORE_CAP (elements) lowers the bound, so that tests reach the piecewise forms at small sizes.
-long score_cap() {
-    const char* v = getenv("PARAS_SDPA_SCORE_CAP");
-    const long n = v ? atol(v) : 0;
-    return n > 0 && n < kScoreCapDefault ? n : kScoreCapDefault;
-}
-
+constexpr long kScoreCapBytes = 1L << 30;        // scores held at a time: 1 GiB whatever the element type
 size_t up256(size_t n) { return (n + 255) / 256 * 256; }
 int elem_size(int dtype) { return dtype == PARAS_F64 ? 8 : dtype == PARAS_F32 ? 4 : 2; }
+// The bound in elements.  PARAS_SDPA_SCORE_CAP (elements) lowers it, so that tests reach the
+// piecewise forms at small sizes (looked up per call: the tests switch it between calls; a caller
+// that changes it between paras_sdpa_workspace and paras_sdpa_fwd gets the workspace check's error).
+long score_cap(int dtype) {
+    const long cap = kScoreCapBytes / elem_size(dtype);
+    const char* v = getenv("PARAS_SDPA_SCORE_CAP");
+    const long n = v ? atol(v) : 0;
+    return n > 0 && n < cap ? n : cap;
+}
 
 // vt[(b*Hkv + h)][d][j] = v[b][h][j][d]
 template <typename S>
@@ -140,12 +142,12 @@ Plan make_plan(const paras_sdpa_args& a) {
     const long per_head = a.Lq * a.Lk;
     const long head_run = heads_run_on(a) ? a.B * a.Hq : a.Hq;
     Plan pl{};
-    if (per_head * rep <= score_cap()) {
+    if (per_head * rep <= score_cap(a.dtype)) {
         pl.rows = a.Lq;
-        pl.heads = rep == 1 ? std::min<long>(head_run, std::max<long>(1, score_cap() / per_head)) : rep;
+        pl.heads = rep == 1 ? std::min<long>(head_run, std::max<long>(1, score_cap(a.dtype) / per_head)) : rep;
     } else {
         pl.heads = rep;
-        pl.rows = std::max<long>(1, score_cap() / (a.Lk * rep));
+        pl.rows = std::max<long>(1, score_cap(a.dtype) / (a.Lk * rep));
     }
     const size_t es = static_cast<size_t>(elem_size(a.dtype));
     pl.vt_bytes = up256(static_cast<size_t>(a.B * a.Hkv * a.Dv * a.Lk) * es);
@@ -163,7 +165,7 @@ bool composed_supported(const paras_sdpa_args& a) {
     const double macs = static_cast<double>(a.B) * a.Hq * a.Lq * a.Lk * (a.D + a.Dv);
     if (macs < static_cast<double>(1L << 25)) return false;          // measured: level with the general kernel at 1.7e7, 2.6x faster at 6.7e7
     const long rep = a.Hq / a.Hkv;
-    if (a.Lk * rep > score_cap()) return false;                        // not even one row block fits
+    if (a.Lk * rep > score_cap(a.dtype)) return false;                        // not even one row block fits
     if (a.Lq * a.Lk >= (1L << 31) || a.Lk * a.Dv >= (1L << 31)) return false;
     if (a.q_strides[2] < a.D || a.k_strides[2] < a.D) return false;   // rows the products cannot take (expanded or overlapping views)
     if (a.B * a.Hkv > 65535 || (a.Dv + 31) / 32 > 65535 || a.B * a.Hq > 65535) return false;   // grid limits of the transpose and the batched products

@@ -29,6 +29,7 @@
 #include <cmath>
 #include <mutex>
 #include <set>
+#include <utility>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
                     for (int g = 0; g < 4; ++g) {
                         const int key = key0 + g * 8 + 4 * lh;
                         if (wide && key + 3 < p.Lk) {
-                            *reinterpret_cast<u32x2*>(arow + key) = u32x2{pw[2 * g], pw[2 * g + 1]};
+                            store8_nt(arow + key, u32x2{pw[2 * g], pw[2 * g + 1]});   // written once, read by nobody here: keep K / V in L2
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
                 if (row >= p.Lq) break;
                 std::uint16_t* zr = p.attn + ((static_cast<long>(b) * p.Hq + hq) * p.Lq + row) * p.Lk;
                 if (rows16) {
-                    for (int key = first + lane * 8; key < p.Lk; key += 64 * 8) store16(zr + key, u32x4{0u, 0u, 0u, 0u});
+                    for (int key = first + lane * 8; key < p.Lk; key += 64 * 8) store16_nt(zr + key, u32x4{0u, 0u, 0u, 0u});
                 } else {
                     for (int key = first + lane; key < p.Lk; key += 64) zr[key] = 0;
                 }
@@ -424,14 +425,16 @@ int launch_t(WeightsParams p, int mode, hipStream_t s) {
     const long blocks = static_cast<long>(p.B) * p.Hq * per_bh;
     const dim3 grid(static_cast<unsigned>(blocks)), wg(512);
     constexpr unsigned kLdsBytes = 4u * kTile * D * 2u;     // K and V, two stages each
-    // More than 64 KB of LDS has to be asked for by name, once per kernel.
+    // More than 64 KB of LDS has to be asked for by name, once per kernel and device.
     auto allow = [&](const void* fn) {
         static std::mutex mu;
-        static std::set<const void*> done;
+        static std::set<std::pair<int, const void*>> done;
+        int dev = 0;
+        if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
         std::lock_guard<std::mutex> g(mu);
-        if (done.count(fn)) return hipSuccess;
+        if (done.count({dev, fn})) return hipSuccess;
         const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBytes));
-        if (e == hipSuccess) done.insert(fn);
+        if (e == hipSuccess) done.insert({dev, fn});
         return e;
     };
     switch (mode) {

@@ -268,16 +268,25 @@ PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 /* 65536 tokens the whole routing is one kernel: its workgroups publish their  */
 /* counts stamped with the call's epoch and poll each other's.  Outside graph  */
 /* capture that kernel is the only launch and the stamped counts live in the   */
-/* library's own device memory (4 areas of 131,328 bytes per GPU, taken in     */
-/* turn; calls that overlap on one area stay exact and turn slow); on a stream */
-/* that is being captured, or with PARAS_ROUTE_OWN_SCRATCH=0, they live in     */
-/* `workspace`, which a fill kernel queued in front clears.                    */
+/* library's own device memory (8 areas of 131,328 bytes per GPU, one per      */
+/* stream by a hash of the handle; calls that overlap on one area stay exact   */
+/* and turn slower: a workgroup waits about 300 us for the others' counts and  */
+/* then counts for itself); on a stream that is being captured, or with        */
+/* PARAS_ROUTE_OWN_SCRATCH=0, they live in `workspace`, which a fill kernel    */
+/* queued in front clears.                                                     */
 /* ------------------------------------------------------------------------- */
 PARAS_API size_t paras_moe_route_workspace(int64_t T, int64_t E, int64_t k);
 PARAS_API int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k,
                               int dtype, int64_t* topi, float* topw, int64_t* order,
                               int64_t* inv_order, int64_t* counts, int64_t* offsets,
                               void* workspace, void* stream);
+/* How many workgroups of paras_moe_route / paras_moe_route_noalloc stopped waiting
+ * for the others and counted for themselves since the library was loaded, on the
+ * current device (a diagnostic with no counterpart in the reference: results are
+ * the same either way; a number that keeps growing says the routing kernel's
+ * workgroups are not resident together, i.e. the chip is oversubscribed).
+ * Synchronous: it copies one word from the device. */
+PARAS_API int paras_moe_route_give_ups(uint64_t* count);
 
 /* paras_moe_route for callers that cannot allocate (code under HIP graph
  * capture, serving loops, harnesses that forbid hipMalloc).  It has no

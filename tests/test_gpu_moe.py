@@ -4,6 +4,8 @@ FFN bar: bf16 / fp16 within 2e-2 absolute of the host-engine oracle, or one
 unit in the last place of the 16-bit result where that is larger (|y| >= 4 for
 bf16: a GEMM whose fp32 summation order differs from ATen's flips the final
 rounding of a few outputs, by exactly one ulp)."""
+import ctypes as C
+
 import pytest
 import torch
 
@@ -235,10 +237,15 @@ def test_route_when_the_workgroups_do_not_wait_for_each_other(shape, monkeypatch
     logits[5] = logits[5, 0]
     want = O.moe_route(logits, k)
     monkeypatch.setenv("PARAS_ROUTE_SPIN_LIMIT", "1")
+    before, after = C.c_uint64(0), C.c_uint64(0)
+    capi.check(capi.lib().paras_moe_route_give_ups(C.byref(before)))
     for _ in range(3):
         got = capi.moe_route(logits.cuda(), k)
         for name, g, w in zip(NAMES, got, want):
             assert_bit_exact(g, w, f"moe_route {name} without waiting")
+    capi.check(capi.lib().paras_moe_route_give_ups(C.byref(after)))
+    if T >= 5000:                                 # (a handful of workgroups may all have arrived by the first poll)
+        assert after.value > before.value, "the give-up counter did not move"
     got = capi.moe_route_noalloc(logits.cuda(), k)
     for name, g, w in zip(NAMES, got, want):
         assert_bit_exact(g, w, f"moe_route_noalloc {name} without waiting")

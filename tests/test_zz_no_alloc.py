@@ -48,12 +48,29 @@ def test_allocates_nothing_and_rejects_what_does_not_fit():
     a0, c0 = C.c_uint64(), C.c_uint64()
     L.paras_memory_stats(0, C.byref(a0), C.byref(c0))
     before = torch.cuda.memory_stats()["num_alloc_retries"], torch.cuda.memory_allocated()
+    free0 = torch.cuda.mem_get_info()[0]          # what the driver itself has left: a direct hipMalloc would show here
     capi.moe_route_noalloc(dl, 2, out=out)
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
     a1, c1 = C.c_uint64(), C.c_uint64()
     L.paras_memory_stats(0, C.byref(a1), C.byref(c1))
     assert (a0.value, c0.value) == (a1.value, c1.value)
     assert before == (torch.cuda.memory_stats()["num_alloc_retries"], torch.cuda.memory_allocated())
+    # under stream capture an allocation (or a free) would fail the capture; replays give the same outputs
+    want = [o.clone() for o in out]
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            capi.moe_route_noalloc(dl, 2, out=out)
+    for _ in range(3):
+        for o in out:
+            o.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        for name, got, w in zip(NAMES, out, want):
+            assert_bit_exact(got, w, f"replayed {name}")
     with pytest.raises(capi.ParasError, match="exceed the static scratch"):
         capi.moe_route_noalloc(torch.zeros(65537, 8, device="cuda"), 2)
     with pytest.raises(capi.ParasError, match="expert count"):
