@@ -288,7 +288,16 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             }
         }
     };
+    // With a mask the scores are narrowed where the host engine narrows them (attention_ops.cpp:101-128:
+    // the product, the scaled product and the sum with an additive mask are tensors of T): a row that
+    // sees few keys is decided by one or two scores, and a 2^-9 step on one of them is several per cent
+    // on its weight.  The scores leave here scaled; the kernel's scale is 1 in these variants.
+    auto round_T = [](float x) { return Elem<T>::to_f32(Elem<T>::from_f32_finite(x)); };
     auto mask_apply = [&](const std::uint32_t (&mr)[MREGS], float16_t& sc) {
+        if constexpr (kMask != 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[r] = round_T(round_T(sc[r]) * p.score_scale);
+        }
         if constexpr (kMask == 1) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -297,7 +306,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const std::uint16_t bits = static_cast<std::uint16_t>(mr[r >> 1] >> (16 * (r & 1)));
-                sc[r] = fmaf(Elem<T>::to_f32(bits), p.inv_scale, sc[r]);
+                sc[r] = round_T(sc[r] + Elem<T>::to_f32(bits));
             }
         }
     };
@@ -611,7 +620,11 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     p.scale_log2 = static_cast<float>(a.scale * 1.4426950408889634);
     p.mask = static_cast<const unsigned char*>(a.mask);
     p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2]; p.ms_k = a.mask_strides[3];
-    p.inv_scale = static_cast<float>(1.0 / a.scale);
+    p.score_scale = static_cast<float>(a.scale);
+    if (a.mask_kind != 0) {          // the masked variants scale the scores themselves, between two narrowings
+        p.scale = 1.0f;
+        p.scale_log2 = 1.4426950408889634f;
+    }
     const bool causal = a.is_causal != 0;
     const int mk = a.mask_kind;
     if (flash_uses_wide(a)) return launch_flash_wide(p, causal, a.dtype == PARAS_BF16, s);

@@ -34,7 +34,7 @@ struct FlashParams {
     // or additive values of the tensor dtype
     const unsigned char* mask;
     long ms_b, ms_h, ms_q, ms_k;
-    float inv_scale;   // the scores are kept unscaled: an additive mask value m enters as m / scale
+    float score_scale; // the caller's scale as given; the masked variants apply it themselves and run with scale = 1
     unsigned magic_nq, magic_hq, magic_rep;   // ceil(2^32 / d) for d = n_qblocks, Hq, Hq / Hkv (set by the wide kernel's launcher)
 };
 

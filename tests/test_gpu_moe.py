@@ -12,32 +12,11 @@ import torch
 import capi
 import oracle as O
 from conftest import assert_bit_exact
+from ffn_bar import assert_ffn_close
 from golden_util import DTYPE_TAGS, case
 
 pytestmark = pytest.mark.gpu
 NAMES = ("topi", "topw", "order", "inv", "counts", "offsets")
-
-
-def ulp16(ref, dtype):
-    mant = 7 if dtype == torch.bfloat16 else 10
-    return 2.0 ** (torch.floor(torch.log2(ref.double().abs().clamp_min(1e-30))) - mant)
-
-
-def assert_ffn_close(out, ref, dtype):
-    """Per element: max(2e-2, one 16-bit ulp of the reference value).  A GEMM
-    whose fp32 summation order differs from ATen's flips the last bit of a few
-    intermediate y values; weighted and re-rounded they reach the output as at
-    most one ulp of the top binade of the outputs, for at most 1 element in
-    1000.  Measured at BASELINE config 5 over all 8192 x 4096 outputs
-    (max |out| 11.25): worst 0.0625, 5472 elements (1.6e-4) beyond 2e-2, 3170
-    (9.4e-5) beyond max(2e-2, 1 ulp), mean error 7.8e-5."""
-    err = (out.double().cpu() - ref.double()).abs()
-    tol = torch.maximum(torch.full_like(err, 2e-2), ulp16(ref, dtype) * 1.001)
-    frac = float((err > tol).double().mean())
-    top = float(ulp16(ref.double().abs().max() * 1.999, dtype))
-    assert frac <= 1e-3, f"{frac:.2e} of elements beyond max(2e-2, 1 ulp); worst {err.max().item():.3e}"
-    assert err.max().item() <= max(2e-2, top) * 1.001, f"worst {err.max().item():.3e} > one ulp of the top binade {top:.3e}"
-    return err
 
 
 @pytest.mark.parametrize("tag", DTYPE_TAGS)

@@ -250,33 +250,24 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
         mask = keep
     else:
         mask = (torch.randn(mshape) * 0.5).masked_fill(~keep, -math.inf).to(dtype)
-    out, _, _, kern = run(q, k, v, mask=mask)
-    want, _ = O.sdpa_math(q, k, v, attn_mask=mask, enable_gqa=True, gemm="aten")
+    scale = O.round_to_dtype(1 / math.sqrt(D), dtype)      # the op layer narrows the scale to the tensor type
+    out, _, _, kern = run(q, k, v, mask=mask, scale=scale)
+    want, _ = O.sdpa_math(q, k, v, attn_mask=mask, enable_gqa=True, gemm="aten", scale=scale)
     assert kern.startswith("flash_mfma")
     if dead_row is not None:
         assert bool(out[:, :, dead_row].isnan().all()) and bool(want[:, :, dead_row].isnan().all())
         rows = [i for i in range(Lq) if i != dead_row]
         out, want = out[:, :, rows], want[:, :, rows]
     assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(want).all())
-    # Two bars.  Against softmax(q k^T s + mask) v evaluated in fp64 from the same 16-bit inputs: 1e-2.
-    # Against the host-engine oracle: 2e-2 for all but 1e-4 of the elements, 3e-2 for those.  The oracle
-    # rounds the scores to 16 bits before the softmax; with part of the keys masked out a row is often
-    # dominated by one or two keys, a 2^-9 relative step on a score of magnitude 4-8 is then several per
-    # cent on the leading weights, and the oracle is itself more than 1e-2 away from the exact value.
-    # Measured over these 16 cases: worst 0.0234 (bf16, bool mask, [2,4,4,200,200,128]: 3 of 204800
-    # elements beyond 2e-2), every other case at most 0.0156, fp16 at most 0.002.
-    rep = Hq // Hkv
-    sc = (q.double() @ k.double().repeat_interleave(rep, 1).transpose(-1, -2)) / math.sqrt(D)
-    full = mask if mask.dim() == 4 else mask.expand(1, 1, *mask.shape[-2:]) if mask.dim() == 2 else mask
-    sc = sc.masked_fill(~full, -math.inf) if kind == "bool" else sc + full.double()
-    exact = torch.softmax(sc, -1) @ v.double().repeat_interleave(rep, 1)
-    if dead_row is not None:
-        exact = exact[:, :, rows]
-    err_exact = (out.double().cpu() - exact).abs()
+    # The host engine narrows the scores to 16 bits three times before the softmax (product, scaled
+    # product, sum with the mask); with part of the keys masked out a row is often decided by one or two
+    # keys, and those roundings move the result by up to 2.4e-2 from softmax(q k^T s + mask) v in fp64
+    # (tests/test_parity_bars_cpu.py).  The masked kernels narrow at the same three places, so they are
+    # held to the host engine, not to the exact value: 1e-2 for bf16 (measured worst 0.0078 = one step
+    # of a result in [1, 2)), 2.5e-3 for fp16 (measured 0.00098).
     err_oracle = (out.double().cpu() - want.double()).abs()
-    assert float(err_exact.max()) <= 1e-2, f"{shape} {dtype} {kind}"
-    assert float((err_oracle > ABS_16BIT).double().mean()) <= 1e-4, f"{shape} {dtype} {kind}: {int((err_oracle > ABS_16BIT).sum())} elements beyond 2e-2"
-    assert float(err_oracle.max()) <= 1.5 * ABS_16BIT, f"{shape} {dtype} {kind}: worst {float(err_oracle.max()):.4f}"
+    bar = 1e-2 if dtype == torch.bfloat16 else 2.5e-3
+    assert float(err_oracle.max()) <= bar, f"{shape} {dtype} {kind}: worst {float(err_oracle.max()):.4f}"
 
 
 def ulps_apart(a, b):
