@@ -63,11 +63,30 @@ def load_traffic() -> dict:
     path = ROOT / "profiles" / "hbm_traffic.txt"
     out = {}
     if path.exists():
+        measured_on = None
         for ln in path.read_text().splitlines():
             f = ln.split()
-            if len(f) == 3 and not ln.startswith("#"):
+            if ln.startswith("# kernel sources "):
+                measured_on = f[3]
+            elif len(f) == 3 and not ln.startswith("#"):
                 out[f[0]] = int(float(f[1]) + float(f[2]))
+        now = kernel_sources_digest()
+        if measured_on != now:
+            log(f"bench.py: profiles/hbm_traffic.txt was measured on kernel sources {measured_on}, the tree holds {now}: "
+                "the `traffic` figures may be stale (measure again with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+            out["_stale"] = True
     return out
+
+
+def kernel_sources_digest() -> str:
+    """Digest of the kernel sources the library is built from; the traffic file records the one it was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted((ROOT / "framework-torch-paras_amd" / "csrc").rglob("*")):
+        if f.suffix in (".hip", ".h", ".cpp"):
+            h.update(f.name.encode())
+            h.update(f.read_bytes())
+    return h.hexdigest()[:16]
 
 
 SETTLE_MS = 40.0        # untimed settling of the short memory-bound launches (see Timer.run)
@@ -164,15 +183,18 @@ def main() -> int:
         q, k, v = qc.to(dev), kc.to(dev), vc.to(dev)
         out = torch.empty_like(q)
         a = capi.sdpa_args(q, k, v, out, is_causal=True)
-        assert L.paras_sdpa_kernel_name(C.byref(a)).startswith(b"flash_mfma")
+        kname = L.paras_sdpa_kernel_name(C.byref(a)).decode()
+        assert kname.startswith("flash_mfma")
+        wide = kname == "flash_mfma_wide"      # 64 queries per wavefront, one workgroup per CU walking a list of items
         ms, wall = timer.run(lambda i: must(L.paras_sdpa_fwd(C.byref(a), None, st)), steps, warmup, SETTLE_MFMA_MS)
         flops = 4 * B * H * S * S * D / 2          # causal-halved
         tf = flops / ms / 1e9
         results["sdpa_prefill"] = {
             "workload": "bf16 causal flash-attention fwd B=4 H=32 S=4096 D=128 (configs[2])",
             "value": round(tf, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall, 4),
-            "kernel": "flash_fwd_kernel<bf16,128,causal>", "algorithmic_flops_per_launch": flops,
-            "roofline": roofline("mfma", tf, "flash_fwd_kernel"),
+            "kernel": "flash_wide_kernel<bf16,causal>" if wide else "flash_fwd_kernel<bf16,128,causal>",
+            "algorithmic_flops_per_launch": flops,
+            "roofline": roofline("mfma", tf, "flash_wide_kernel" if wide else "flash_fwd_kernel"),
         }
         log(f"sdpa_prefill: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s  ({tf / MFMA_BF16_PEAK_TFLOPS:.1%} of dense bf16 peak)")
         got_head = [(b_, h_, out[b_, h_, :256].cpu()) for b_, h_ in ((0, 0), (3, 31))]
@@ -535,6 +557,8 @@ def main() -> int:
         "parity_checked": head.get("parity_checked", False),
         "workloads": results,
     }
+    if traffic.get("_stale"):
+        line["traffic_measured_on_other_sources"] = True
     print(json.dumps(line))
     bad = [n_ for n_, r in results.items() if r.get("parity") and r["parity"].get("ok") is False]
     if bad:

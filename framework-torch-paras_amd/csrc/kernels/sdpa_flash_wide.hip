@@ -426,9 +426,23 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     auto outputs_to_memory = [&](int ob, int ohq, int oq0) {
         const std::uint16_t* mine = o_lds + wave * WQ * OROW;
         std::uint16_t* orow = p.out + ((static_cast<long>(ob) * p.Hq + ohq) * p.Lq + oq0) * D;
+        const int chunk = lane & 15, sub = lane >> 4;
+        if (oq0 + WQ <= p.Lq) {
+            // all of the wavefront's rows exist (wave-uniform): eight reads in flight, then their stores
+            // (a test per row makes sixteen branches, each a read, a wait and a store: 1 % of the kernel)
 #pragma unroll
+            for (int h = 0; h < WQ / 32; ++h) {
+                u32x4 v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4*>(mine + (32 * h + 4 * i + sub) * OROW + chunk * 8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(orow + (32 * h + 4 * i + sub) * D + chunk * 8) = v[i];
+            }
+            return;
+        }
+#pragma unroll 1
         for (int i = 0; i < WQ / 4; ++i) {
-            const int row = 4 * i + (lane >> 4), chunk = lane & 15;
+            const int row = 4 * i + sub;
             const u32x4 v = *reinterpret_cast<const u32x4*>(mine + row * OROW + chunk * 8);
             if (oq0 + row < p.Lq) *reinterpret_cast<u32x4*>(orow + row * D + chunk * 8) = v;
         }
