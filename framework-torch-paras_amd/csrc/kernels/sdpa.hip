@@ -31,7 +31,7 @@ int validate(const paras_sdpa_args* a) {
 
 bool empty_output(const paras_sdpa_args& a) { return a.B == 0 || a.Hq == 0 || a.Lq == 0 || a.Dv == 0; }
 
-// 16-bit head sizes below 128 other than 64: the MFMA kernels exist for 64 and 128, so q, k and v
+// 16-bit head sizes below 256 other than 64 and 128: the MFMA kernels exist for 64, 128 and 256, so q, k and v
 // are copied into the workspace with zero columns appended (q.k and the first D output columns do
 // not change; the scale is the caller's, i.e. that of the real head size) and the first D columns
 // of the padded result are copied out -- instead of the general fp64 kernel, three orders of
@@ -44,9 +44,9 @@ size_t up256(size_t n) { return (n + 255) / 256 * 256; }
 
 bool plan_padded(const paras_sdpa_args& a, PaddedPlan* plan) {
     if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
-    if (a.attn != nullptr || a.D != a.Dv || a.D < 1 || a.D >= 128 || a.D == 64) return false;
+    if (a.attn != nullptr || a.D != a.Dv || a.D < 1 || a.D >= 256 || a.D == 64 || a.D == 128) return false;
     if (a.Lq < 1 || a.Lk < 1) return false;
-    const int64_t Dp = a.D < 64 ? 64 : 128;
+    const int64_t Dp = a.D < 64 ? 64 : a.D < 128 ? 128 : 256;
     PaddedPlan pl{};
     pl.inner = a;
     pl.inner.D = pl.inner.Dv = Dp;

@@ -86,7 +86,7 @@ constexpr int kBM = 128;   // queries per workgroup: 4 waves x 32
 
 // kMask: 0 none, 1 bytes (nonzero = attend), 2 additive values of type T.
 template <typename T, int D, bool kCausal, int kMask>
-__global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) {
+__global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const FlashParams p) {
     static_assert(!(kCausal && kMask != 0), "a mask and the causal rule are mutually exclusive");
     // 32-query blocks per wave.  The code is written for any QB; 2 halves the LDS operand
     // traffic per query but needs one wave per SIMD and measured 30 % slower (nothing hides
@@ -100,8 +100,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     constexpr int CHUNKS = D / 8;
     constexpr int RPI    = 64 / CHUNKS;
     constexpr int NI     = kBN / (RPI * NW);
-    auto ksw = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
-    auto vsw = [](int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
+    auto ksw = [](int row) { return D >= 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto vsw = [](int row) { return D >= 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
 
     // LDS: two tiles each of K and V (4 x 16 KiB per workgroup at D = 128, two workgroups per
     // CU).  They are four separate arrays on purpose: the compiler makes an LDS read wait for
@@ -183,6 +183,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     const int k_row_bytes = static_cast<int>(p.ks_l) * 2, v_row_bytes = static_cast<int>(p.vs_l) * 2;
     const int k_lane = srow * k_row_bytes + ((slot ^ ksw(srow)) * 16);
     const int v_lane = srow * v_row_bytes + ((slot ^ vsw(srow)) * 16);
+    // Request i of a tile fills rows i * RPI * NW + srow.  That is a multiple of 16 rows further on
+    // for heads of up to 128 elements, so the swizzle of the row is the swizzle of srow; with 256
+    // elements a request covers 8 rows and every other one lands 8 rows on: bit 3 of the K swizzle flips.
+    const int k_lane_odd = D > 128 ? srow * k_row_bytes + ((slot ^ ksw(srow + 8)) * 16) : k_lane;
+    static_assert((RPI * NW) % 16 == 0 || (RPI * NW == 8 && D == 256), "the staging swizzle assumes whole groups of 16 (or 8) rows per request");
     typedef __attribute__((address_space(3))) void* lptr_t;
     auto make_rsrc = [&](const std::uint16_t* base, int row_bytes) {
         const int bytes = (p.Lk - 1) * row_bytes + D * 2;           // < 2^31: checked by flash_supported
@@ -190,24 +195,23 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
     };
     const __amdgpu_buffer_rsrc_t k_rsrc = make_rsrc(kbase, k_row_bytes);
     const __amdgpu_buffer_rsrc_t v_rsrc = make_rsrc(vbase, v_row_bytes);
-    auto stage_rows = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile) {
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int r0 = i * RPI * NW;
-            // a negative offset is a huge unsigned one: out of range like the rows past the end
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)(tile + (r0 + wave * RPI) * D), 16,
-                                                     lane_off + (first + r0) * row_bytes, 0, 0, 0);
-        }
-    };
-    auto stage_one = [&](__amdgpu_buffer_rsrc_t rsrc, int lane_off, int row_bytes, int first, std::uint16_t* tile, int i) {
+    struct OfK {}; struct OfV {};
+    auto stage_one = [&](__amdgpu_buffer_rsrc_t rsrc, auto which, int row_bytes, int first, std::uint16_t* tile, int i) {
         const int r0 = i * RPI * NW;
+        constexpr bool is_k = std::is_same<decltype(which), OfK>::value;
+        const int lane_off = is_k ? ((i & 1) ? k_lane_odd : k_lane) : v_lane;      // (i is a constant wherever this is called)
+        // a negative offset is a huge unsigned one: out of range like the rows past the end
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)(tile + (r0 + wave * RPI) * D), 16,
                                                  lane_off + (first + r0) * row_bytes, 0, 0, 0);
     };
+    auto stage_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto which, int row_bytes, int first, std::uint16_t* tile) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) stage_one(rsrc, which, row_bytes, first, tile, i);
+    };
     // Requests the pair tile t's blocks need beyond K tile t: K tile t+1 and V tile t (`par` = parity of t).
     auto stage_pair = [&](int t, auto par) {
-        stage_rows(k_rsrc, k_lane, k_row_bytes, (t + 1) * kBN - 32, kbuf(par, true));
-        stage_rows(v_rsrc, v_lane, v_row_bytes, t * kBN, vbuf(par, false));
+        stage_rows(k_rsrc, OfK{}, k_row_bytes, (t + 1) * kBN - 32, kbuf(par, true));
+        stage_rows(v_rsrc, OfV{}, v_row_bytes, t * kBN, vbuf(par, false));
     };
     // Barrier that publishes every tile requested so far.
     auto publish = [&]() {
@@ -229,7 +233,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
             for (int r = 0; r < 16; ++r) oacc[qb][i][r] = 0.f;
     }
 
-    stage_rows(k_rsrc, k_lane, k_row_bytes, -32, k_lds0);   // K tile 0: keys 0..31 in its upper half
+    stage_rows(k_rsrc, OfK{}, k_row_bytes, -32, k_lds0);   // K tile 0: keys 0..31 in its upper half
     stage_pair(0, Par0{});
     publish();
 
@@ -449,8 +453,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashParams p) 
                 static_assert(2 * (2 * NI - 1) < NS, "the requests fit the block's slots");
                 if (c % 2 == 0 && c / 2 < 2 * NI) {
                     const int i = c / 2, t = j >> 1;
-                    if (i < NI) stage_one(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN - 32, kbuf(par, false), i);
-                    else        stage_one(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true), i - NI);
+                    if (i < NI) stage_one(k_rsrc, OfK{}, k_row_bytes, (t + 2) * kBN - 32, kbuf(par, false), i);
+                    else        stage_one(v_rsrc, OfV{}, v_row_bytes, (t + 1) * kBN, vbuf(par, true), i - NI);
                 }
             }
             if (c + 2 < NS) fetch(j, c + 2, par);
@@ -579,7 +583,7 @@ bool mult8(const int64_t* strides) { return strides[0] % 8 == 0 && strides[1] % 
 
 bool flash_supported(const paras_sdpa_args& a) {
     if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
-    if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
+    if (a.D != a.Dv || (a.D != 64 && a.D != 128 && a.D != 256)) return false;
     if (a.attn != nullptr) return false;                            // the weights are never formed here
     if (a.mask_kind != 0 && (a.mask == nullptr || a.is_causal)) return false;
     if (a.mask_kind < 0 || a.mask_kind > 2) return false;
@@ -629,8 +633,8 @@ int launch_flash(const paras_sdpa_args& a, hipStream_t s) {
     const int mk = a.mask_kind;
     if (flash_uses_wide(a)) return launch_flash_wide(p, causal, a.dtype == PARAS_BF16, s);
     if (a.dtype == PARAS_BF16)
-        return a.D == 128 ? launch_t<bf16_t, 128>(p, causal, mk, s) : launch_t<bf16_t, 64>(p, causal, mk, s);
-    return a.D == 128 ? launch_t<f16_t, 128>(p, causal, mk, s) : launch_t<f16_t, 64>(p, causal, mk, s);
+        return a.D == 256 ? launch_t<bf16_t, 256>(p, causal, mk, s) : a.D == 128 ? launch_t<bf16_t, 128>(p, causal, mk, s) : launch_t<bf16_t, 64>(p, causal, mk, s);
+    return a.D == 256 ? launch_t<f16_t, 256>(p, causal, mk, s) : a.D == 128 ? launch_t<f16_t, 128>(p, causal, mk, s) : launch_t<f16_t, 64>(p, causal, mk, s);
 }
 
 }  // namespace paras

@@ -196,7 +196,7 @@ def test_flash_random_shapes_layouts_and_padding():
         return torch.randn(*shape, device="cuda", generator=g).to(dt)
 
     for _ in range(40):
-        D, dt = rng.choice([64, 128]), rng.choice([torch.bfloat16, torch.float16])
+        D, dt = rng.choice([64, 128, 256]), rng.choice([torch.bfloat16, torch.float16])
         Hkv, rep, B = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 4]), rng.choice([1, 2, 3])
         Hq = Hkv * rep
         Lq = rng.choice([2, 5, 31, 32, 33, 64, 100, 127, 128, 129, 200, 255, 256, 257, 384, 500, 513])
@@ -268,6 +268,55 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
     err_oracle = (out.double().cpu() - want.double()).abs()
     bar = 1e-2 if dtype == torch.bfloat16 else 2.5e-3
     assert float(err_oracle.max()) <= bar, f"{shape} {dtype} {kind}: worst {float(err_oracle.max()):.4f}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case_", [
+    # B, Hq, Hkv, Lq, Lk, causal, mask, layout
+    (1, 2, 2, 128, 128, True, None, "bhld"), (2, 4, 2, 1024, 1024, True, None, "blhd"), (1, 2, 1, 1000, 1000, True, None, "bhld"),
+    (1, 2, 2, 333, 777, False, None, "padded"), (1, 2, 2, 777, 333, True, None, "bhld"), (1, 3, 3, 200, 1500, False, "bool", "bhld"),
+    (1, 2, 2, 130, 191, False, "add", "blhd"), (1, 1, 1, 300, 33, True, None, "bhld"), (1, 1, 1, 1, 31, False, None, "bhld"),
+    (1, 8, 2, 257, 640, False, None, "bhld")])
+def test_flash_head_size_256_matches_oracle(case_, dtype):
+    """Heads of 256 elements on the flash kernel (one workgroup per CU: its four tiles of K and V
+    fill 128 KB of LDS, a wavefront's outputs and queries its registers): causal, masks, GQA,
+    ragged lengths, strided layouts; log-sum-exp against fp64."""
+    B, Hq, Hkv, Lq, Lk, causal, mk, layout = case_
+    D = 256
+    torch.manual_seed(Lq * 7 + Lk)
+    def make(H, L):          # (host tensor, the same values on the device in the layout under test)
+        if layout == "blhd":
+            base = torch.randn(B, L, H, D).to(dtype)
+            return base.transpose(1, 2), base.cuda().transpose(1, 2)
+        if layout == "padded":
+            base = torch.full((B, H, L + 3, D + 16), float("nan")).to(dtype)
+            base[:, :, :L, 8:8 + D] = torch.randn(B, H, L, D).to(dtype)
+            return base[:, :, :L, 8:8 + D], base.cuda()[:, :, :L, 8:8 + D]
+        base = torch.randn(B, H, L, D).to(dtype)
+        return base, base.cuda()
+    (q, dq), (k, dk), (v, dv) = make(Hq, Lq), make(Hkv, Lk), make(Hkv, Lk)
+    mask = None
+    if mk == "bool":
+        mask = torch.rand(B, 1, Lq, Lk) > 0.3
+        mask[..., 0] = True
+    elif mk == "add":
+        mask = (torch.randn(1, Hq, Lq, Lk) * 0.5).to(dtype)
+    scale = O.round_to_dtype(1.0 / math.sqrt(D), dtype)
+    out, _, lse, name = capi.sdpa(dq, dk, dv, is_causal=causal, mask=None if mask is None else mask.cuda(), scale=scale, want_lse=True)
+    want, _ = O.sdpa_math(q.contiguous(), k.contiguous(), v.contiguous(), is_causal=causal, attn_mask=mask, scale=scale, enable_gqa=True, gemm="aten")
+    assert name == "flash_mfma" and out.shape == (B, Hq, Lq, D)
+    assert max_abs(out, want) <= (1e-2 if mk else ABS_16BIT)
+    rep = Hq // Hkv
+    sc = (q.double() @ k.double().repeat_interleave(rep, 1).transpose(-1, -2)) * scale
+    if causal:
+        sc = sc.masked_fill(~torch.ones(Lq, Lk, dtype=torch.bool).tril(), -math.inf)
+    if mk == "bool":
+        sc = sc.masked_fill(~mask, -math.inf)
+    elif mk == "add":
+        sc = sc + mask.double()
+    ref_lse = torch.logsumexp(sc, -1)
+    tol = 5e-4 if mk is None else 2e-2     # (the masked kernels narrow their scores as the host engine does)
+    assert float((lse.double().cpu() - ref_lse).abs().max()) <= tol
 
 
 def ulps_apart(a, b):
@@ -535,9 +584,11 @@ def test_config4_shape_slice_and_gqa_equivalence():
     # B, Hq, Hkv, Lq, Lk, D, causal, mask
     (2, 4, 4, 200, 200, 80, True, None), (1, 8, 2, 130, 130, 96, False, None), (2, 2, 1, 77, 300, 40, False, "bool"),
     (1, 4, 4, 64, 64, 100, True, None), (2, 8, 2, 1, 900, 96, False, None), (1, 4, 1, 2, 700, 48, False, "add"),
-    (1, 2, 2, 50, 50, 1, False, None), (1, 2, 2, 33, 65, 127, True, None)])
+    (1, 2, 2, 50, 50, 1, False, None), (1, 2, 2, 33, 65, 127, True, None),
+    (2, 2, 2, 200, 200, 192, True, None), (1, 4, 2, 300, 500, 160, False, None), (1, 2, 2, 1, 700, 200, False, None),
+    (1, 2, 1, 129, 257, 255, False, "bool"), (1, 2, 2, 70, 130, 129, False, "add")])
 def test_head_sizes_between_the_mfma_kernels_are_padded_inside_the_library(case_, dtype):
-    """16-bit head sizes below 128 other than 64, through the C ABI: the library copies q, k, v into
+    """16-bit head sizes below 256 other than 64 and 128, through the C ABI: the library copies q, k, v into
     its workspace with zero columns appended and runs the flash / decode kernels (prefill and decode
     shapes, GQA, causal, bool and additive masks, strided inputs)."""
     B, Hq, Hkv, Lq, Lk, D, causal, mk = case_
