@@ -164,8 +164,5 @@ __device__ __forceinline__ u32x4 load16_nt(const void* p) {
 __device__ __forceinline__ void store16_nt(void* p, u32x4 v) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
-__device__ __forceinline__ void store8_nt(void* p, u32x2 v) {
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
-}
 
 }  // namespace paras
