@@ -197,6 +197,15 @@ def main() -> int:
             "roofline": roofline("mfma", tf, "flash_wide_kernel" if wide else "flash_fwd_kernel"),
         }
         log(f"sdpa_prefill: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s  ({tf / MFMA_BF16_PEAK_TFLOPS:.1%} of dense bf16 peak)")
+        # What this box sustains on a register-only loop of the same MFMA (random operands): the published
+        # peak assumes 2.4 GHz, under MFMA load the part is power limited.  Reported, not used in `frac`.
+        sustained = {}
+        for label, wps, valu in (("one_wave_per_simd", 1, 0), ("two_waves_per_simd", 2, 0), ("two_waves_per_simd_2_fp32_per_mfma", 2, 2)):
+            rate = C.c_double(0.0)
+            must(L.paras_mfma_rate_probe(wps, valu, C.byref(rate)))
+            sustained[label] = round(rate.value, 1)
+        results["sdpa_prefill"]["mfma_loop_tflops_on_this_box"] = sustained
+        log(f"  register-only MFMA loop on this box: {sustained} TFLOP/s; the flash kernel runs one wavefront per SIMD")
         got_head = [(b_, h_, out[b_, h_, :256].cpu()) for b_, h_ in ((0, 0), (3, 31))]
         got_tail = out[1, 7, S - 64:].cpu()
 

@@ -383,6 +383,20 @@ PARAS_API int paras_softmax_rows(const void* x, void* out, int64_t rows, int64_t
 PARAS_API int paras_topk_rows(const void* x, void* values, int64_t* indices, int64_t rows,
                               int64_t n, int64_t k, int largest, int dtype, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* Measurement aid (no counterpart in the reference): the rate, in TFLOP/s,    */
+/* that the current device sustains on a register-only loop of                 */
+/* v_mfma_f32_32x32x16_bf16 on random operands, with `waves_per_simd` (1 or 2) */
+/* wavefronts per SIMD and `valu_per_mfma` (0 or 2) independent fp32           */
+/* instructions after each MFMA.  The published dense bf16 peak assumes        */
+/* 2.4 GHz; under this load the part is power limited and clocks lower, so     */
+/* bench.py reports this figure beside the attention and GEMM figures of the   */
+/* same process.  Blocks for about 0.2 s (150 ms of untimed load first: a short */
+/* burst runs at a clock the part does not hold); allocates and frees 0.5 MB;  */
+/* runs on the null stream.                                                    */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_mfma_rate_probe(int waves_per_simd, int valu_per_mfma, double* tflops);
+
 #ifdef __cplusplus
 }
 #endif
