@@ -93,7 +93,7 @@ __device__ __forceinline__ float group_sum(float x) {
 
 // kMask: 0 = none, 1 = bool (true = attend), 2 = additive values of dtype T
 template <typename T, int D, int kMask>
-__global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kThreads, (D > 128 ? 1 : 2)) void decode_split_kernel(const DecodeParams p) {
     constexpr int kD = D, kVS = D + 16;
     constexpr int KS = D / 32;           // 32-wide contraction steps of q k^T
     constexpr int DB = D / 16;           // 16-wide output blocks of O^T
@@ -375,7 +375,7 @@ void plan(const paras_sdpa_args& a, int* splits, int* chunk) {
 
 bool decode_supported(const paras_sdpa_args& a) {
     if (a.dtype != PARAS_BF16 && a.dtype != PARAS_F16) return false;
-    if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
+    if (a.D != a.Dv || (a.D != 64 && a.D != 128 && a.D != 256)) return false;
     if (a.attn != nullptr || a.is_causal) return false;
     if (a.mask_kind != 0 && (a.mask == nullptr || a.mask_kind > 2)) return false;
     if (a.Hkv < 1 || a.Hq % a.Hkv != 0) return false;
@@ -433,7 +433,10 @@ int launch_decode(const paras_sdpa_args& a, void* workspace, hipStream_t s) {
             PARAS_HIP_TRY(hipGetLastError());                                                              \
         }                                                                                                  \
     } while (0)
-    if (a.D == 128) {
+    if (a.D == 256) {
+        if (bf) PARAS_DECODE_LAUNCH(bf16_t, 256);
+        else    PARAS_DECODE_LAUNCH(f16_t, 256);
+    } else if (a.D == 128) {
         if (bf) PARAS_DECODE_LAUNCH(bf16_t, 128);
         else    PARAS_DECODE_LAUNCH(f16_t, 128);
     } else {

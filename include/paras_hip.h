@@ -238,7 +238,7 @@ PARAS_API int paras_sdpa_fwd(const paras_sdpa_args* args, void* workspace, void*
 /* Name of the kernel paras_sdpa_fwd would pick: "flash_mfma" (bf16 / f16 heads of
  * 64, 128 or 256 elements; "flash_mfma_wide" where its 64-queries-per-wavefront
  * form runs: head size 128, no mask, at least two 256-query tiles per CU, rows of
- * 4096 causal / 1024 unmasked on), "decode_split" (heads of 64 or 128),
+ * 4096 causal / 1024 unmasked on), "decode_split" (heads of 64, 128 or 256),
  * "math_mfma" (bf16 / f16 with the weights returned), "padded_mfma" (bf16 / f16
  * head sizes below 256 other than 64 and 128: q, k, v copied into the workspace with
  * zero columns up to 64, 128 or 256, then flash_mfma / decode_split; the workspace

@@ -275,7 +275,7 @@ def test_flash_with_masks_matches_oracle(dtype, kind, shape):
     # B, Hq, Hkv, Lq, Lk, causal, mask, layout
     (1, 2, 2, 128, 128, True, None, "bhld"), (2, 4, 2, 1024, 1024, True, None, "blhd"), (1, 2, 1, 1000, 1000, True, None, "bhld"),
     (1, 2, 2, 333, 777, False, None, "padded"), (1, 2, 2, 777, 333, True, None, "bhld"), (1, 3, 3, 200, 1500, False, "bool", "bhld"),
-    (1, 2, 2, 130, 191, False, "add", "blhd"), (1, 1, 1, 300, 33, True, None, "bhld"), (1, 1, 1, 1, 31, False, None, "bhld"),
+    (1, 2, 2, 130, 191, False, "add", "blhd"), (1, 1, 1, 300, 33, True, None, "bhld"), (1, 1, 1, 17, 31, False, None, "bhld"),
     (1, 8, 2, 257, 640, False, None, "bhld")])
 def test_flash_head_size_256_matches_oracle(case_, dtype):
     """Heads of 256 elements on the flash kernel (one workgroup per CU: its four tiles of K and V
@@ -418,16 +418,18 @@ def test_decode_matches_oracle(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [64, 256])
 @pytest.mark.parametrize("shape", [(2, 8, 2, 1, 1000), (1, 16, 1, 1, 4099), (3, 4, 4, 3, 300), (1, 2, 2, 1, 31)])
-def test_decode_head_size_64(dtype, shape):
+def test_decode_head_sizes_64_and_256(dtype, shape, D):
     """The split-KV decode kernel at head size 64 (half as many contraction steps and output blocks
-    per tile), with and without a key-padding mask."""
+    per tile) and 256 (twice as many; one workgroup per CU, its V tiles fill 137 KB of LDS), with
+    and without a key-padding mask."""
     B, Hq, Hkv, Lq, Lk = shape
-    q, k, v = torch.randn(B, Hq, Lq, 64).to(dtype), torch.randn(B, Hkv, Lk, 64).to(dtype), torch.randn(B, Hkv, Lk, 64).to(dtype)
+    q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
     out, _, lse, kern = run(q, k, v, want_lse=True)
     want, _ = O.sdpa_math(q, k, v, enable_gqa=True, gemm="aten")
     assert kern == "decode_split" and max_abs(out, want) <= ABS_16BIT
-    s = (q.float() @ k.float().repeat_interleave(Hq // Hkv, 1).transpose(-1, -2)) / 8.0
+    s = (q.float() @ k.float().repeat_interleave(Hq // Hkv, 1).transpose(-1, -2)) / math.sqrt(D)
     assert torch.allclose(lse.cpu(), torch.logsumexp(s, -1), rtol=1e-3, atol=1e-3)
     keep = torch.ones(B, 1, 1, Lk, dtype=torch.bool)
     keep[0, ..., Lk // 2:] = False
