@@ -281,3 +281,14 @@ def test_gemm_nt_workspace_batched_and_shapes_that_need_none():
     x = torch.randn(8, 256, device="cuda").bfloat16()
     w = torch.randn(64, 256, device="cuda").bfloat16()
     assert torch.equal(capi.gemm_nt(x, w, workspace=True), capi.gemm_nt(x, w))
+
+
+def test_mfma_rate_probe_reports_a_plausible_rate():
+    """The measurement aid bench.py prints beside the attention figure: a register-only MFMA loop
+    cannot beat the published peak and, on a healthy MI355X, does not fall below a fifth of it."""
+    import ctypes as C
+    rate = C.c_double(0.0)
+    capi.check(capi.lib().paras_mfma_rate_probe(1, 0, C.byref(rate)))
+    assert 500.0 < rate.value < 2600.0
+    assert capi.lib().paras_mfma_rate_probe(3, 0, C.byref(rate)) != 0          # only one or two wavefronts per SIMD
+    assert b"wavefronts per SIMD" in capi.lib().paras_last_error()
