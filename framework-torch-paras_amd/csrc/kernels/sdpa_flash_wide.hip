@@ -243,11 +243,14 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     };
     // Raise the running maxima where a block max (this lane's half of the keys) asks for it; the
     // two halves of a query only meet inside this rarely taken branch.
+    // (the compare builtin hands back the wavefront's lane mask as it stands: a bool fed to the
+    // ballot builtin is first turned into 0 / 1 per lane and compared again)
+    float raise_at[QB];      // m_run + lazy_margin, kept beside m_run
     auto wants_raise = [&](const float (&mx)[QB]) {
-        bool grow = false;
+        unsigned long long grow = 0;
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) grow = grow || (mx[qb] > m_run[qb] + lazy_margin);
-        return __builtin_amdgcn_ballot_w64(grow) != 0;   // wave-uniform, rare after block 0
+        for (int qb = 0; qb < QB; ++qb) grow |= __builtin_amdgcn_fcmpf(mx[qb], raise_at[qb], 2 /* ordered greater than */);
+        return grow != 0;   // wave-uniform, rare after block 0
     };
     auto raise_max = [&](const float (&mx)[QB]) {
         // (pins the outputs in AGPRs up to here: without it their 128 copies to VGPRs are
@@ -260,6 +263,7 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
             // (equal covers -inf on both sides: a query that has seen no key yet keeps its zeros)
             const float alpha = m_run[qb] == m_new ? 1.f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * p.scale_log2);
             m_run[qb] = m_new;
+            raise_at[qb] = m_new + lazy_margin;
             l_run[qb] *= alpha;
 #pragma unroll
             for (int i = 0; i < DBLK; ++i)
@@ -273,17 +277,21 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
     // those maxima ask for a higher reference point.  Blocks on the diagonal or at the end of K are
     // masked first and their maxima taken again.
     auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB], bool raise) {
-        if (needs_mask(j, 0)) {                 // first_masked[0] <= first_masked[1]: one test on the common path
+        const bool masked = needs_mask(j, 0);        // first_masked[0] <= first_masked[1]: one test covers both
+        // One test on the common path, which falls through: both cases are rare and wave-uniform.
+        if (__builtin_expect(masked | raise, 0)) {
+            if (masked) {
 #pragma unroll
-            for (int qb = 0; qb < QB; ++qb) {
-                if (needs_mask(j, qb)) {
-                    apply_mask(j, qb, sc[qb]);
-                    mx[qb] = lane_max(sc[qb]);
+                for (int qb = 0; qb < QB; ++qb) {
+                    if (needs_mask(j, qb)) {
+                        apply_mask(j, qb, sc[qb]);
+                        mx[qb] = lane_max(sc[qb]);
+                    }
                 }
+                raise = wants_raise(mx);
             }
-            raise = wants_raise(mx);
+            if (raise) raise_max(mx);
         }
-        if (raise) raise_max(mx);
     };
 
     // Operand fragments: kf = the K rows of the block whose scores come next, vf = the V rows of
@@ -384,11 +392,17 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
             } else {
                 constexpr int g = (u - 16) >> 2, qb = g & 1, s2 = g >> 1, db = (u - 16) & 3;
                 oacc[qb][db] = Mma<T>::run(vf[s2 * DBLK + db], __builtin_bit_cast(i16x8, pw[qb][s2]), oacc[qb][db]);
-                if constexpr (u >= 32 - KSTEPS) fetch_k(krows, u - (32 - KSTEPS));   // (the first V fragments are dead by now: their registers take these)
+                // The next block's K fragments, under the first eight output MFMAs: the wait in front of
+                // the next block's first score MFMA then finds them eight MFMAs old as well (under the last
+                // eight, the youngest was requested one MFMA before that wait).  No more registers: all of
+                // V's fragments are live here either way, as K's and V's are during the score MFMAs.
+                if constexpr (u < 16 + KSTEPS) fetch_k(krows, u - 16);
             }
-            if constexpr (kStage && u % 4 == 1) {
-                // the next tile pair (K tile t+2, V tile t+1), one request every fourth MFMA
-                constexpr int i = u / 4;
+            if constexpr (kStage && u % 2 == 1 && u / 2 < 2 * NI) {
+                // the next tile pair (K tile t+2, V tile t+1), one request every other MFMA of the tile's
+                // first sixteen: the wait at the end of the tile then finds them all at least 48 MFMAs old
+                // (every fourth MFMA, the last one 34 MFMAs old: 1 % slower)
+                constexpr int i = u / 2;
                 const int t = j >> 1;
                 if constexpr (i < NI) stage_one(k_rsrc, k_lane, k_row_bytes, (t + 2) * kBN, kbuf(par, false), i);
                 else                  stage_one(v_rsrc, v_lane, v_row_bytes, (t + 1) * kBN, vbuf(par, true), i - NI);
@@ -498,6 +512,7 @@ __global__ __launch_bounds__(256, 1) void flash_wide_kernel(const FlashParams p)
             for (int qb = 0; qb < QB; ++qb) {
                 if (needs_mask(0, qb)) apply_mask(0, qb, s_a[qb]);
                 m_run[qb] = half_swap_max(lane_max(s_a[qb]));
+                raise_at[qb] = m_run[qb] + lazy_margin;
             }
         }
         for (int t = 0; t < wave_tiles; t += 2) {
