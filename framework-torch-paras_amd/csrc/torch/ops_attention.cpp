@@ -185,8 +185,8 @@ OverrideableResult sdpa_overrideable(const Tensor& query, const Tensor& key, con
     (void)return_debug_mask;
     Prepared p;
     prepare(query, key, value, attn_bias, is_causal, scale, /*enable_gqa=*/true, &p);
-    // (16-bit head sizes below 128 other than 64 run on the MFMA kernels too: the library pads q, k
-    // and v with zero columns inside its workspace.)
+    // (16-bit head sizes below 256 other than 64, 128 and 256 run on the MFMA kernels too: the library
+    // pads q, k and v with zero columns inside its workspace.)
     Tensor out, lse;
     run(&p, &out, nullptr, &lse);
     std::vector<int64_t> lse_shape(p.out_shape.begin(), p.out_shape.end() - 1);

@@ -124,9 +124,9 @@ def test_sdpa_bf16_key_padding_mask_and_bias(device):
     assert float((got.float() - want).abs().max()) <= 2e-2
 
 
-@pytest.mark.parametrize("D", [96, 80, 40])
+@pytest.mark.parametrize("D", [96, 80, 40, 192, 256])
 def test_sdpa_16bit_other_head_sizes_run_zero_padded(device, D):
-    """Head sizes other than 64 / 128 go through the MFMA kernels with zero columns appended
+    """Head sizes other than 64 / 128 / 256 go through the MFMA kernels with zero columns appended
     (the default scale stays 1/sqrt(D) of the real size); results as for any other 16-bit call."""
     B, H, L = 2, 3, 150
     q, k, v = (torch.randn(B, H, L, D).half() for _ in range(3))
