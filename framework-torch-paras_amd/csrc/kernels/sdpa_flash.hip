@@ -324,10 +324,12 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const
     // test runs on each lane's own half of the keys; the two halves of a query are only brought
     // together inside the rare branch.
     auto raise_max = [&](float (&mx)[QB]) {
-        bool grow = false;
+        // (the compare builtin hands back the wavefront's lane mask as it stands; a bool fed to the
+        // ballot builtin is first turned into 0 / 1 per lane and compared again)
+        unsigned long long grow = 0;
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) grow = grow || (mx[qb] > m_run[qb] + lazy_margin);
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {  // wave-uniform, rare after block 0
+        for (int qb = 0; qb < QB; ++qb) grow |= __builtin_amdgcn_fcmpf(mx[qb], m_run[qb] + lazy_margin, 2 /* ordered greater than */);
+        if (__builtin_expect(grow != 0, 0)) {  // wave-uniform, rare after block 0: the common path falls through
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
                 const float m_new = fmaxf(m_run[qb], half_swap_max(mx[qb]));
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
             if constexpr (kMask != 0) mask_apply(mr, sc[qb]);
-            if (needs_mask(j, qb)) apply_mask(j, qb, sc[qb]);
+            if (__builtin_expect(needs_mask(j, qb), 0)) apply_mask(j, qb, sc[qb]);
             if (kMask != 0 || needs_mask(j, qb)) mx[qb] = lane_max(sc[qb]);
         }
         raise_max(mx);
