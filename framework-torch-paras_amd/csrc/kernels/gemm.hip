@@ -40,7 +40,35 @@ struct DenseParams {
     int  splits;                // kPartial kernels: parts of the contraction, one workgroup each per tile
     long k_per_split;           // contraction elements per part (a multiple of 64)
     float* partial;             // [batch][split][M][N] fp32
+    int  xcd_blocks, xcd_blocks_n;   // XCD-blocked tile order: blocks of kXcdBlockM x kXcdBlockN tiles per batch (0: plain order), blocks along n
 };
+
+// Workgroup w runs on XCD w % 8, each with an L2 of its own.  In the plain order (column units
+// innermost) the 32 workgroups an XCD runs at a time are 16 row tiles x 2 column units: 18 operand
+// panels pass through its L2.  Dealing the tiles in blocks of 4 x 8, one block per XCD at a time,
+// makes that 12 panels: a third fewer L2 misses.  The grid is padded to whole blocks and to a
+// multiple of 8 blocks; a workgroup whose tile does not exist returns at once.
+constexpr int kXcdBlockM = 4, kXcdBlockN = 8, kXcdBlockTiles = kXcdBlockM * kXcdBlockN, kXcds = 8;
+__host__ __device__ inline long xcd_order_workgroups(int blocks) { return static_cast<long>((blocks + kXcds - 1) / kXcds) * kXcds * kXcdBlockTiles; }
+// false: no tile for this workgroup
+__device__ __forceinline__ bool tile_of_workgroup(const DenseParams& p, long wg, long& bidx, int& mt, int& nu) {
+    if (p.xcd_blocks == 0) {
+        const long per_batch = static_cast<long>(p.m_tiles) * p.n_units;
+        bidx = wg / per_batch;
+        const long rem = wg % per_batch;
+        mt = static_cast<int>(rem / p.n_units);
+        nu = static_cast<int>(rem % p.n_units);
+        return true;
+    }
+    const long per_batch = xcd_order_workgroups(p.xcd_blocks);
+    bidx = wg / per_batch;
+    const int w = static_cast<int>(wg % per_batch);
+    const int xcd = w % kXcds, j = w / kXcds;
+    const int block = (j / kXcdBlockTiles) * kXcds + xcd, t = j % kXcdBlockTiles;
+    mt = (block / p.xcd_blocks_n) * kXcdBlockM + t / kXcdBlockN;
+    nu = (block % p.xcd_blocks_n) * kXcdBlockN + t % kXcdBlockN;
+    return block < p.xcd_blocks && mt < p.m_tiles && nu < p.n_units;
+}
 
 // S = Tile256 (8 waves, 256 x 256; for problems with at least 144 such tiles), Tile128 (4 waves,
 // 128 x 256) or Tile128x128 (4 waves, one column group; when there would be fewer than 512 tiles of 128 x 256).
@@ -54,13 +82,13 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
 
     // Column units innermost: the workgroups running together share the A row panel
     // (and, across m-tiles, stream the same B panels through L2).
-    const long per_batch = static_cast<long>(p.m_tiles) * p.n_units;
     const long tile_id = kPartial ? blockIdx.x / p.splits : blockIdx.x;
     const long split = kPartial ? blockIdx.x % p.splits : 0;
     const long k_first = kPartial ? split * p.k_per_split : 0;
     const long k_count = kPartial ? (k_first + p.k_per_split < p.K ? p.k_per_split : p.K - k_first) : p.K;
-    const long bidx = tile_id / per_batch, rem = tile_id % per_batch;
-    const int mt = static_cast<int>(rem / p.n_units), nu = static_cast<int>(rem % p.n_units);
+    long bidx;
+    int mt, nu;
+    if (!tile_of_workgroup(p, tile_id, bidx, mt, nu)) return;      // (the whole workgroup: nobody is left at a barrier)
     const long row0 = static_cast<long>(mt) * S::kBM, n0 = static_cast<long>(nu) * S::kGroups * kBN;
     const std::uint16_t* A = p.a + bidx * p.sa + k_first;
     const std::uint16_t* B = p.b + bidx * p.sb + k_first;
@@ -835,7 +863,16 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
         PARAS_HIP_TRY(hipGetLastError());
         return PARAS_OK;
     }
-    const unsigned blocks = static_cast<unsigned>(m_tiles * n_units * batch);
+    unsigned blocks = static_cast<unsigned>(m_tiles * n_units * batch);
+    if (use_wide && m_tiles >= kXcdBlockM && n_units >= kXcdBlockN) {
+        const long xbm = (m_tiles + kXcdBlockM - 1) / kXcdBlockM, xbn = (n_units + kXcdBlockN - 1) / kXcdBlockN;
+        const long wgs = xbm * xbn <= 0x7fffffLL ? xcd_order_workgroups(static_cast<int>(xbm * xbn)) * batch : -1;
+        if (wgs > 0 && wgs <= 0x7fffffffLL) {
+            p.xcd_blocks = static_cast<int>(xbm * xbn);
+            p.xcd_blocks_n = static_cast<int>(xbn);
+            blocks = static_cast<unsigned>(wgs);
+        }
+    }
     if (use_wide) {
         if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile256>(p, blocks, s);
         else                     launch_dense<f16_t, gemm::Tile256>(p, blocks, s);

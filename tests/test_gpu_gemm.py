@@ -188,6 +188,22 @@ def test_gemm_nt_256_row_tiles_agree_with_128_row_tiles():
     assert_gemm_close(whole[3, -3:], ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("shape", [(2, 1100, 2100, 64), (1, 1024, 2048, 128), (3, 2300, 4200, 64), (1, 16384, 4096, 64)])
+def test_gemm_nt_tiles_dealt_to_the_dies_in_blocks_cover_every_element(shape):
+    """From 4 x 8 tiles of 256 x 256 on, the workgroups take their tiles in blocks of 4 x 8 per die,
+    on a grid padded to whole blocks and to eight blocks at a time: every element of every batch
+    entry has to come out, none twice from a wrong tile.  Whole matrix against the oracle (which
+    fits here: one k-tile or two)."""
+    Bt, M, N, K = shape
+    torch.manual_seed(33)
+    a = torch.randn(Bt, M, K, device="cuda").bfloat16()
+    b = (0.1 * torch.randn(Bt, N, K, device="cuda")).bfloat16()
+    out = capi.gemm_nt(a, b)
+    assert out.shape == (Bt, M, N)
+    for i in range(Bt):
+        assert_gemm_close(out[i], O.matmul_nt(a[i].cpu(), b[i].cpu()), torch.bfloat16)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(1, 4096, 4096), (16, 100, 64), (17, 1027, 320), (64, 4096, 1024), (100, 515, 192),
                                    (128, 2050, 4096)])
