@@ -59,7 +59,7 @@
 // sits between a fragment's request and the MFMA that consumes it.
 //
 // An optional mask (bytes, nonzero = attend; or additive values of the tensor type;
-// broadcast over any of batch / head / query, contiguous along the keys) is applied
+// broadcast over any of batch / head / query, any stride along the keys) is applied
 // to the finished scores of a block; the mask bytes of block j+1 are requested when
 // block j starts.  Queries with no visible key so far carry a running maximum of
 // -inf and contribute zeros; a query with no visible key at all ends as 0/0 = NaN,
@@ -268,12 +268,37 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const
         const long qrow = my_q < p.Lq ? my_q : p.Lq - 1;
         mrow = p.mask + (static_cast<long>(b) * p.ms_b + static_cast<long>(hq) * p.ms_h + qrow * p.ms_q) * (kMask == 1 ? 1 : 2);
     }
-    // The mask is contiguous along the keys and Lk >= 4 (flash_supported): a run that hangs over the
-    // end of the row is read from the row's last four elements and shifted down, so no load leaves
-    // the row and no branch is needed; keys >= Lk get zero bits and are masked by the end-of-K rule.
+    // A mask that is contiguous along the keys, with Lk >= 4: a run that hangs over the end of the
+    // row is read from the row's last four elements and shifted down, so no load leaves the row and
+    // no branch is needed; keys >= Lk get zero bits and are masked by the end-of-K rule.  Any other
+    // stride along the keys (0: a view that broadcasts one value per query over the keys; > 1: slices
+    // and transposed views) is read element by element into the same registers -- sixteen small
+    // loads per block instead of four, requested a block ahead like the runs.
+    const bool mask_runs = p.ms_k == 1 && p.Lk >= 4;       // uniform
     auto mask_load = [&](int j, std::uint32_t (&mr)[MREGS]) {
         if constexpr (kMask != 0) {
             typedef std::uint32_t u32_any __attribute__((aligned(1)));
+            if (!mask_runs) {
+                constexpr int ES = kMask == 1 ? 1 : 2;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    std::uint32_t e[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = min(j * 32 + 8 * g + 4 * lh + i, p.Lk - 1);   // (keys past the end: any value, the end-of-K rule masks them)
+                        const unsigned char* at = mrow + static_cast<long>(key) * p.ms_k * ES;
+                        if constexpr (kMask == 1) e[i] = *at;
+                        else                      e[i] = *reinterpret_cast<const std::uint16_t*>(at);
+                    }
+                    if constexpr (kMask == 1) {
+                        mr[g] = e[0] | (e[1] << 8) | (e[2] << 16) | (e[3] << 24);
+                    } else {
+                        mr[2 * g] = e[0] | (e[1] << 16);
+                        mr[2 * g + 1] = e[2] | (e[3] << 16);
+                    }
+                }
+                return;
+            }
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int key = j * 32 + 8 * g + 4 * lh;
@@ -589,7 +614,7 @@ bool flash_supported(const paras_sdpa_args& a) {
     if (a.attn != nullptr) return false;                            // the weights are never formed here
     if (a.mask_kind != 0 && (a.mask == nullptr || a.is_causal)) return false;
     if (a.mask_kind < 0 || a.mask_kind > 2) return false;
-    if (a.mask_kind != 0 && (a.mask_strides[3] != 1 || a.Lk < 4)) return false;   // mask runs are read four keys at a time
+    if (a.mask_kind != 0 && a.mask_strides[3] < 0) return false;
     if (a.Lq < 1 || a.Lk < 1) return false;
     if (!(a.scale > 0.0) || !std::isfinite(a.scale)) return false;  // the running max is taken on raw scores
     if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || !aligned16(a.out)) return false;
