@@ -26,6 +26,8 @@
 // blocks of 32 keys that lie wholly below the diagonal skip the per-key tests.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <cmath>
 #include <mutex>
 #include <set>
@@ -62,7 +64,7 @@ struct WeightsParams {
     double scale;           // multiplies T(q k^T) in double, as the host engine's mul_out does
     int    scale_is_f32;    // the scale is a float: an fp32 multiply gives the same rounded product
     const unsigned char* mask;
-    long ms_b, ms_h, ms_q;  // element strides (0 = broadcast); the key stride is 1
+    long ms_b, ms_h, ms_q, ms_k;  // element strides (0 = broadcast)
 };
 
 template <typename T> struct Mma16;
@@ -213,19 +215,26 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
             }
             const bool edge = key0 + 32 > p.Lk || (kMode == 3 && key0 + 31 > q0);
             if (kMode == 1 || kMode == 2 || edge) {
-                // masks, without a branch per element (reads past the row's end are clamped into it)
+                // masks, without a branch per element (reads past the row's end are clamped into it); a mask
+                // that is not contiguous along the keys (a transposed or sliced view, one value per query
+                // broadcast over the keys) pays a multiply per element for its place
+                auto masked = [&](auto contiguous) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
-                    const int key_in = key < p.Lk ? key : p.Lk - 1;
-                    float s = sc[r];
-                    bool dead = key >= p.Lk;
-                    if constexpr (kMode == 3) dead = dead || key > my_q;
-                    if constexpr (kMode == 1) dead = dead || mrow[key_in] == 0;
-                    if constexpr (kMode == 2)
-                        s = round_T(s + El::to_f32(*reinterpret_cast<const std::uint16_t*>(mrow + 2 * static_cast<long>(key_in))));   // T(s2 + mask)
-                    sc[r] = dead ? -INFINITY : s;
-                }
+                    for (int r = 0; r < 16; ++r) {
+                        const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                        const int key_in = key < p.Lk ? key : p.Lk - 1;
+                        const long at = decltype(contiguous)::value ? static_cast<long>(key_in) : static_cast<long>(key_in) * p.ms_k;
+                        float s = sc[r];
+                        bool dead = key >= p.Lk;
+                        if constexpr (kMode == 3) dead = dead || key > my_q;
+                        if constexpr (kMode == 1) dead = dead || mrow[at] == 0;
+                        if constexpr (kMode == 2)
+                            s = round_T(s + El::to_f32(*reinterpret_cast<const std::uint16_t*>(mrow + 2 * at)));   // T(s2 + mask)
+                        sc[r] = dead ? -INFINITY : s;
+                    }
+                };
+                if ((kMode != 1 && kMode != 2) || p.ms_k == 1) masked(std::true_type{});
+                else                                           masked(std::false_type{});
             }
         };
 
@@ -483,7 +492,7 @@ bool weights_supported(const paras_sdpa_args& a) {
     if (a.D != a.Dv || (a.D != 64 && a.D != 128)) return false;
     if (a.mask_kind != 0 && (a.mask == nullptr || a.is_causal)) return false;
     if (a.mask_kind < 0 || a.mask_kind > 2) return false;
-    if (a.mask_kind != 0 && a.mask_strides[3] != 1 && a.Lk > 1) return false;
+    if (a.mask_kind != 0 && a.mask_strides[3] < 0) return false;
     if (a.Lq < 1 || a.Lk < 1) return false;
     if (!std::isfinite(a.scale)) return false;
     if (!aligned16(a.q) || !aligned16(a.k) || !aligned16(a.v) || (reinterpret_cast<uintptr_t>(a.out) & 7) != 0) return false;
@@ -510,7 +519,7 @@ int launch_weights(const paras_sdpa_args& a, hipStream_t s) {
     p.scale = a.scale;
     p.scale_is_f32 = static_cast<double>(static_cast<float>(a.scale)) == a.scale ? 1 : 0;
     p.mask = static_cast<const unsigned char*>(a.mask);
-    p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2];
+    p.ms_b = a.mask_strides[0]; p.ms_h = a.mask_strides[1]; p.ms_q = a.mask_strides[2]; p.ms_k = a.mask_strides[3];
     const int mode = a.is_causal ? 3 : a.mask_kind;
     if (a.dtype == PARAS_BF16)
         return a.D == 128 ? launch_t<bf16_t, 128>(p, mode, s) : launch_t<bf16_t, 64>(p, mode, s);

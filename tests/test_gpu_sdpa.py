@@ -377,6 +377,43 @@ def test_math_op_weights_on_the_mfma_kernel(dtype, variant, shape):
     assert bool(torch.isfinite(lse.cpu()[live]).all())
 
 
+@pytest.mark.parametrize("kind", ["bool", "additive"])
+@pytest.mark.parametrize("view", ["transposed", "every_other", "per_query"])
+def test_math_op_weights_kernel_with_masks_strided_along_the_keys(kind, view):
+    """The kernel that returns the weights reads its mask element by element, so any stride along
+    the keys stays on it: a transposed view, every other element of a wider tensor, one value per
+    query broadcast over the keys (whole rows of NaN where that value masks)."""
+    B, Hq, Hkv, Lq, Lk, D = 2, 4, 2, 140, 210, 128
+    dtype = torch.bfloat16
+    torch.manual_seed(sum(map(ord, view + kind)))
+    q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
+
+    def values(*shape):
+        keep = torch.rand(*shape) > 0.3
+        return keep if kind == "bool" else (torch.randn(*shape) * 0.5).masked_fill(~keep, -math.inf).to(dtype)
+
+    if view == "transposed":
+        base = values(B, 1, Lk, Lq)
+        host, dev = base.transpose(-1, -2), base.cuda().transpose(-1, -2)
+    elif view == "every_other":
+        base = values(B, Hq, Lq, 2 * Lk)
+        host, dev = base[..., ::2], base.cuda()[..., ::2]
+    else:
+        base = values(B, 1, Lq, 1)
+        host, dev = base.expand(B, 1, Lq, Lk), base.cuda().expand(B, 1, Lq, Lk)
+    assert dev.stride(-1) == {"transposed": Lq, "every_other": 2, "per_query": 0}[view]
+    scale = O.round_to_dtype(1 / math.sqrt(D), dtype)
+    out, attn, _, kern = capi.sdpa(q.cuda(), k.cuda(), v.cuda(), mask=dev, scale=scale, want_attn=True)
+    want, wattn = O.sdpa_math(q, k, v, attn_mask=host.contiguous(), enable_gqa=True, gemm="aten", scale=scale)
+    assert kern == "math_mfma"
+    assert torch.equal(attn.cpu().isnan(), wattn.isnan()) and torch.equal(out.cpu().isnan(), want.isnan())
+    ok = ~wattn.isnan()
+    d = ulps_apart(attn, wattn)[ok]
+    assert float((d > 1).float().mean()) <= 5e-4 and float((d > 0).float().mean()) <= 5e-3
+    assert float((attn.cpu().double() - wattn.double()).abs()[ok].max()) <= ABS_16BIT
+    assert float((out.cpu().double() - want.double()).abs()[~want.isnan()].max()) <= ABS_16BIT
+
+
 def test_math_op_weights_kernel_strided_inputs_and_explicit_scale():
     """Heads sliced out of a fused [B, L, 3, H, D] projection (strided q / k / v) and an explicit
     scale (narrowed to the tensor type, as the op layer hands it over)."""
