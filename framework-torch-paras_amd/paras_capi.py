@@ -63,6 +63,7 @@ SIGNATURES = {
     "paras_moe_route_noalloc": (i32, [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp, vp, vp]),
     "paras_moe_route_give_ups": (i32, [C.POINTER(C.c_uint64)]),
     "paras_mfma_rate_probe": (i32, [i32, i32, C.POINTER(C.c_double)]),
+    "paras_l2_stream_probe": (i32, [i32, i32, C.POINTER(C.c_double)]),
     "paras_moe_ffn_workspace": (sz, [i64, i64, i64, i64, i32]),
     "paras_moe_ffn": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
     "paras_index_select": (i32, [vp, vp, vp, i64, i64, i64, i64, vp]),

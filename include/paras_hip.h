@@ -397,6 +397,20 @@ PARAS_API int paras_topk_rows(const void* x, void* values, int64_t* indices, int
 /* ------------------------------------------------------------------------- */
 PARAS_API int paras_mfma_rate_probe(int waves_per_simd, int valu_per_mfma, double* tflops);
 
+/* ------------------------------------------------------------------------- */
+/* Measurement aid (no counterpart in the reference): bytes per nanosecond and */
+/* CU that one four-wavefront workgroup per CU pulls through the vector cache  */
+/* when it does nothing but stream a region of `region_kib` KiB of its own     */
+/* (a power of two, 8 ... 1024) over and over: with 64 KiB the regions of an   */
+/* XCD's 32 workgroups stay in its 4 MB L2, with 256 KiB and more they come    */
+/* from the last-level cache.  `to_lds` != 0: buffer loads that write LDS      */
+/* directly (what a GEMM's staging would use); 0: loads into registers.  Tells */
+/* whether a kernel's operand traffic is anywhere near what the memory side    */
+/* delivers.  Blocks for a few ms; allocates and frees CUs x region bytes;     */
+/* runs on the null stream.                                                    */
+/* ------------------------------------------------------------------------- */
+PARAS_API int paras_l2_stream_probe(int to_lds, int region_kib, double* bytes_per_ns_per_cu);
+
 #ifdef __cplusplus
 }
 #endif

@@ -308,3 +308,18 @@ def test_mfma_rate_probe_reports_a_plausible_rate():
     assert 500.0 < rate.value < 2600.0
     assert capi.lib().paras_mfma_rate_probe(3, 0, C.byref(rate)) != 0          # only one or two wavefronts per SIMD
     assert b"wavefronts per SIMD" in capi.lib().paras_last_error()
+
+
+def test_l2_stream_probe_reports_plausible_rates():
+    """The streaming probe: regions that stay in L2 come in faster than regions that do not, and
+    both at a rate a CU can plausibly reach (a GEMM tile of 256 x 256 needs about 40 B/ns per CU)."""
+    import ctypes as C
+    rate = C.c_double(0.0)
+    got = {}
+    for to_lds, kib in ((1, 64), (1, 512), (0, 64)):
+        capi.check(capi.lib().paras_l2_stream_probe(to_lds, kib, C.byref(rate)))
+        got[(to_lds, kib)] = rate.value
+    assert 40.0 < got[(1, 64)] < 400.0, got            # measured 116 - 128 B/ns per CU
+    assert 5.0 < got[(1, 512)] < got[(1, 64)], got      # measured 21 - 26 B/ns per CU from the last-level cache
+    assert 10.0 < got[(0, 64)] < 400.0, got             # measured 33 B/ns per CU with eight loads in flight per wavefront
+    assert capi.lib().paras_l2_stream_probe(1, 48, C.byref(rate)) != 0        # not a power of two
