@@ -430,14 +430,16 @@ def test_math_op_weights_kernel_strided_inputs_and_explicit_scale():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("kind", ["bool", "additive"])
-@pytest.mark.parametrize("view", ["transposed", "every_other", "per_query", "three_keys"])
+@pytest.mark.parametrize("view", ["transposed", "every_other", "per_query", "three_keys", "transposed_64", "every_other_256"])
 def test_flash_with_masks_strided_along_the_keys(dtype, kind, view):
     """Masks that are not contiguous along the keys stay on the flash kernel (read element by
     element): a transposed view (key stride Lq), every other element of a wider tensor (stride 2),
     one value per query broadcast over the keys (stride 0), and a contiguous mask over fewer keys
     than a run of four."""
     B, Hq, Hkv, Lq, Lk, D = (2, 4, 2, 150, 3, 128) if view == "three_keys" else (2, 4, 2, 150, 230, 128)
-    torch.manual_seed(sum(map(ord, view + kind)))
+    if "_" in view and view.rsplit("_", 1)[1].isdigit():          # the same views at the other head sizes
+        view, D = view.rsplit("_", 1)[0], int(view.rsplit("_", 1)[1])
+    torch.manual_seed(sum(map(ord, view + kind)) + D)
     q, k, v = torch.randn(B, Hq, Lq, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype), torch.randn(B, Hkv, Lk, D).to(dtype)
 
     def values(*shape):      # what the mask holds, on the host, laid out however the view under test wants it
