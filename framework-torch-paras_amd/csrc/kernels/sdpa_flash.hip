@@ -274,10 +274,28 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const
     // stride along the keys (0: a view that broadcasts one value per query over the keys; > 1: slices
     // and transposed views) is read element by element into the same registers -- sixteen small
     // loads per block instead of four, requested a block ahead like the runs.
+    //   A block that lies wholly inside a contiguous row is not read as four runs per lane (a wavefront's
+    // 64 lanes then touch 64 different places four times over) but as one 16-byte piece per lane of
+    // the block's 32 (bool) or 64 (additive: two pieces) bytes of its query's row: half lh holds keys
+    // 16 lh .. 16 lh + 15 and needs keys 8 g + 4 lh .. + 3, so the two halves of a query swap every
+    // other run when the mask is applied (v_permlane32_swap: lanes l and l + 32).
     const bool mask_runs = p.ms_k == 1 && p.Lk >= 4;       // uniform
+    auto mask_whole_block = [&](int j) { return mask_runs && j * 32 + 32 <= p.Lk; };      // uniform
     auto mask_load = [&](int j, std::uint32_t (&mr)[MREGS]) {
         if constexpr (kMask != 0) {
             typedef std::uint32_t u32_any __attribute__((aligned(1)));
+            typedef u32x4 u32x4_any __attribute__((aligned(1)));
+            if (mask_whole_block(j)) {
+                constexpr int ES = kMask == 1 ? 1 : 2;
+                const unsigned char* at = mrow + (j * 32 + 16 * lh) * ES;
+#pragma unroll
+                for (int h = 0; h < ES; ++h) {
+                    const u32x4 w = *reinterpret_cast<const u32x4_any*>(at + 16 * h);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) mr[4 * h + i] = w[i];
+                }
+                return;
+            }
             if (!mask_runs) {
                 constexpr int ES = kMask == 1 ? 1 : 2;
 #pragma unroll
@@ -322,8 +340,37 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const
     // sees few keys is decided by one or two scores, and a 2^-9 step on one of them is several per cent
     // on its weight.  The scores leave here scaled; the kernel's scale is 1 in these variants.
     auto round_T = [](float x) { return Elem<T>::to_f32(Elem<T>::from_f32_finite(x)); };
-    auto mask_apply = [&](const std::uint32_t (&mr)[MREGS], float16_t& sc) {
+    auto mask_apply = [&](int j, const std::uint32_t (&loaded)[MREGS], float16_t& sc) {
+        std::uint32_t mr[MREGS];
+#pragma unroll
+        for (int i = 0; i < MREGS; ++i) mr[i] = loaded[i];
         if constexpr (kMask != 0) {
+            if (mask_whole_block(j)) {
+                // registers as loaded: the lane's own sixteen keys.  Lower half: keeps its runs 0 and 2 (bool:
+                // one register each; additive: two), gets runs 0 and 2 of the upper half for its runs 1 and 3.
+                auto swap = [&](int x, int y) {       // upper half of register x <-> lower half of register y
+                    const auto r = __builtin_amdgcn_permlane32_swap(mr[x], mr[y], false, false);
+                    mr[x] = r[0];
+                    mr[y] = r[1];
+                };
+                if constexpr (kMask == 1) {
+                    swap(0, 1);
+                    swap(2, 3);
+                    const std::uint32_t t = mr[1];    // runs in order: registers 0, 2, 1, 3
+                    mr[1] = mr[2];
+                    mr[2] = t;
+                } else {
+                    swap(0, 2);
+                    swap(1, 3);
+                    swap(4, 6);
+                    swap(5, 7);
+                    const std::uint32_t t2 = mr[2], t3 = mr[3];     // runs in order: registers (0,1), (4,5), (2,3), (6,7)
+                    mr[2] = mr[4];
+                    mr[3] = mr[5];
+                    mr[4] = t2;
+                    mr[5] = t3;
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) sc[r] = round_T(round_T(sc[r]) * p.score_scale);
         }
@@ -373,7 +420,7 @@ __global__ __launch_bounds__(256, (D > 128 ? 1 : 2)) void flash_fwd_kernel(const
     auto finish_scores = [&](int j, float16_t (&sc)[QB], float (&mx)[QB], const std::uint32_t (&mr)[MREGS]) {
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
-            if constexpr (kMask != 0) mask_apply(mr, sc[qb]);
+            if constexpr (kMask != 0) mask_apply(j, mr, sc[qb]);
             if (__builtin_expect(needs_mask(j, qb), 0)) apply_mask(j, qb, sc[qb]);
             if (kMask != 0 || needs_mask(j, qb)) mx[qb] = lane_max(sc[qb]);
         }
