@@ -198,6 +198,42 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
         // key0 + (r/4)*8 + 4*lh + r%4.  `edge`: the block reaches past the row's end or past the diagonal
         // (wave-uniform); only then the keys are tested one by one.
         auto scores = [&](const std::uint16_t* k_lds, int jb, int key0, float16_t& sc) {
+            // A block that lies wholly inside a contiguous mask row: the lane asks for its half of its
+            // query's 32 keys (16 lh .. + 15) as one 16-byte piece (two for an additive mask) before the
+            // MFMAs, and the halves of a query swap every other run of four keys afterwards
+            // (v_permlane32_swap: lanes l and l + 32), since half lh owns keys 8 g + 4 lh .. + 3.  Sixteen
+            // element loads per block, each touching as many rows as there are queries in the wave, and
+            // waited for on the spot, doubled the kernel's time with a mask.
+            constexpr int MREGS = kMode == 1 ? 4 : (kMode == 2 ? 8 : 1);
+            std::uint32_t mr[MREGS];
+            const bool mask_whole = (kMode == 1 || kMode == 2) && p.ms_k == 1 && key0 + 32 <= p.Lk;     // wave-uniform
+            if constexpr (kMode == 1 || kMode == 2) {
+                if (mask_whole) {
+                    typedef u32x4 u32x4_any __attribute__((aligned(1)));
+                    constexpr int ES = kMode == 1 ? 1 : 2;
+                    const unsigned char* at = mrow + static_cast<long>(key0 + 16 * lh) * ES;
+#pragma unroll
+                    for (int h = 0; h < ES; ++h) {
+                        const u32x4 w = *reinterpret_cast<const u32x4_any*>(at + 16 * h);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) mr[4 * h + i] = w[i];
+                    }
+                }
+            }
+            // Any other block under a mask: its sixteen elements, asked for before the MFMAs as well (reads
+            // past the row's end are clamped into it).
+            std::uint32_t me[(kMode == 1 || kMode == 2) ? 16 : 1];
+            if constexpr (kMode == 1 || kMode == 2) {
+                if (!mask_whole) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                        const long at = static_cast<long>(key < p.Lk ? key : p.Lk - 1) * p.ms_k;
+                        if constexpr (kMode == 1) me[r] = mrow[at];
+                        else                      me[r] = *reinterpret_cast<const std::uint16_t*>(mrow + 2 * at);
+                    }
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
@@ -214,27 +250,47 @@ __global__ __launch_bounds__(512, 2) void weights_fwd_kernel(const WeightsParams
                     sc[r] = round_T(static_cast<float>(static_cast<double>(round_T(sc[r])) * p.scale));
             }
             const bool edge = key0 + 32 > p.Lk || (kMode == 3 && key0 + 31 > q0);
-            if (kMode == 1 || kMode == 2 || edge) {
-                // masks, without a branch per element (reads past the row's end are clamped into it); a mask
-                // that is not contiguous along the keys (a transposed or sliced view, one value per query
-                // broadcast over the keys) pays a multiply per element for its place
-                auto masked = [&](auto contiguous) {
+            if constexpr (kMode == 1 || kMode == 2) {
+                if (mask_whole) {
+                    auto swap = [&](int x, int y) {       // upper half of register x <-> lower half of register y
+                        const auto r2 = __builtin_amdgcn_permlane32_swap(mr[x], mr[y], false, false);
+                        mr[x] = r2[0];
+                        mr[y] = r2[1];
+                    };
+                    if constexpr (kMode == 1) {
+                        swap(0, 1);
+                        swap(2, 3);
+                        constexpr int reg_of_run[4] = {0, 2, 1, 3};
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
-                        const int key_in = key < p.Lk ? key : p.Lk - 1;
-                        const long at = decltype(contiguous)::value ? static_cast<long>(key_in) : static_cast<long>(key_in) * p.ms_k;
-                        float s = sc[r];
-                        bool dead = key >= p.Lk;
-                        if constexpr (kMode == 3) dead = dead || key > my_q;
-                        if constexpr (kMode == 1) dead = dead || mrow[at] == 0;
-                        if constexpr (kMode == 2)
-                            s = round_T(s + El::to_f32(*reinterpret_cast<const std::uint16_t*>(mrow + 2 * at)));   // T(s2 + mask)
-                        sc[r] = dead ? -INFINITY : s;
+                        for (int r = 0; r < 16; ++r)
+                            if (((mr[reg_of_run[r >> 2]] >> (8 * (r & 3))) & 0xffu) == 0) sc[r] = -INFINITY;
+                    } else {
+                        swap(0, 2);
+                        swap(1, 3);
+                        swap(4, 6);
+                        swap(5, 7);
+                        constexpr int reg_of_run[4] = {0, 4, 2, 6};     // first register of each run's pair
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const std::uint16_t bits = static_cast<std::uint16_t>(mr[reg_of_run[r >> 2] + ((r & 3) >> 1)] >> (16 * (r & 1)));
+                            sc[r] = round_T(sc[r] + El::to_f32(bits));        // T(s2 + mask)
+                        }
                     }
-                };
-                if ((kMode != 1 && kMode != 2) || p.ms_k == 1) masked(std::true_type{});
-                else                                           masked(std::false_type{});
+                    return;
+                }
+            }
+            if (kMode == 1 || kMode == 2 || edge) {
+                // without a branch per element
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = key0 + (r >> 2) * 8 + 4 * lh + (r & 3);
+                    float s = sc[r];
+                    bool dead = key >= p.Lk;
+                    if constexpr (kMode == 3) dead = dead || key > my_q;
+                    if constexpr (kMode == 1) dead = dead || me[r] == 0;
+                    if constexpr (kMode == 2) s = round_T(s + El::to_f32(static_cast<std::uint16_t>(me[r])));   // T(s2 + mask)
+                    sc[r] = dead ? -INFINITY : s;
+                }
             }
         };
 
