@@ -40,6 +40,8 @@ struct DenseParams {
     int  splits;                // kPartial kernels: parts of the contraction, one workgroup each per tile
     long k_per_split;           // contraction elements per part (a multiple of 64)
     float* partial;             // [batch][split][M][N] fp32
+    int  swapped;               // few-row kernels only: a and b have changed places (few output COLUMNS, many rows), so a
+                                // result (row of a, row of b) belongs at c[row of b][row of a], and the addend likewise
     int  xcd_blocks, xcd_blocks_n;   // XCD-blocked tile order: blocks of kXcdBlockM x kXcdBlockN tiles per batch (0: plain order), blocks along n
 };
 
@@ -314,6 +316,16 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void skinny_gemm_nt_kernel(const
         const long row = mb * 16 + r16;
         const long col = n0 + nb * 16 + 4 * kg;
         if (row >= p.M) continue;
+        if (p.swapped) {        // `row` is a column of the caller's result and `col + r` a row of it
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (col + r >= p.N) continue;
+                float v = p.alpha * t[r];
+                if (ADD) v = fmaf(p.beta, El::to_f32(ADD[(col + r) * p.ld_add + row]), v);
+                C[(col + r) * p.ldc + row] = El::from_f32(v);
+            }
+            continue;
+        }
         std::uint16_t o16[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -493,14 +505,26 @@ bool few_rows_by_tiles(long M, long N, long batch) {
     return M > 32 && M <= kSkinnyMaxM && (N + gemm::kBN - 1) / gemm::kBN * batch >= 192;
 }
 
+// Few output columns and many rows: the few-row kernels with the operands in each other's place.  Up to
+// 32 columns (every workgroup re-reads the short operand, and from 48 rows of it on the tile kernel with
+// the contraction in parts is faster: M = 16384, N = 128, K = 4096 80 us this way).
+bool swapped_route(long M, long N, long batch) {
+    return N <= 32 && M > kSkinnyMaxM && batch <= 65535 && (M + 15) / 16 <= 0x7fffffffL;
+}
+
 // Parts of the contraction for the 128 x 128 tile kernel with a workspace (0 = it does not apply): 49 to
 // 128 rows and too few tiles to fill the chip; about 384 workgroups in all (measured 128 ... 1024: fewer
 // leave CUs idle, more only add partial tiles for the finishing kernel to read), at least four k-tiles each.
+// More rows than that with at most one tile per CU (a projection over 256 ... 1024 tokens: 64 ... 256
+// tiles, each walking the whole contraction alone on its CU): the same, two parts from 193 tiles on.
 int tile_splitk_plan(long M, long N, long K, long batch, long* k_per_split) {
-    if (M <= 48 || M > kSkinnyMaxM || K % 64 != 0 || N < 128 || few_rows_by_tiles(M, N, batch)) return 0;
-    const long tiles = (N + gemm::kBN - 1) / gemm::kBN * batch;      // one row tile
+    if (M <= 48 || K % 64 != 0 || N < 128) return 0;
+    if (M <= kSkinnyMaxM && few_rows_by_tiles(M, N, batch)) return 0;
+    const long m_tiles = (M + gemm::kBM - 1) / gemm::kBM;
+    const long tiles = m_tiles * ((N + gemm::kBN - 1) / gemm::kBN) * batch;
+    if (m_tiles > 1 && tiles > 256) return 0;
     const long k_tiles = K / 64;
-    long splits = (384 + tiles - 1) / tiles;
+    long splits = (m_tiles > 1 && tiles > 192) ? 2 : (384 + tiles - 1) / tiles;
     if (splits > k_tiles / 4) splits = k_tiles / 4;
     if (splits < 2) return 0;
     const long per = (k_tiles + splits - 1) / splits;
@@ -734,6 +758,7 @@ size_t paras_gemm_nt_workspace(int64_t M, int64_t N, int64_t K, int64_t batch, i
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || (dtype != PARAS_BF16 && dtype != PARAS_F16)) return 0;
     int per = 0;
     long kper = 0;
+    if (K % gemm::kBK == 0 && swapped_route(M, N, batch)) return 0;
     int splits = tile_splitk_plan(M, N, K, batch, &kper);
     if (splits == 0) splits = splitk_plan(M, N, K, batch, &per);
     return static_cast<size_t>(splits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
@@ -802,6 +827,23 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
             default:         return launch_any<f16_t>(p, a, b, addend, c, batch, s);
         }
     }
+    // Few output columns and many rows (a router's logits: tokens x experts): the product is bound by
+    // reading a once, which 128 x 128 tiles on N / 128 of the CUs do badly (M = 16384, K = 4096:
+    // N = 8 in 78 us, N = 128 in 78 us).  The few-row kernels stream a long operand with every CU and
+    // keep the short one in registers, so the operands change places and the results are stored
+    // transposed.
+    if (swapped_route(M, N, batch)) {
+        DenseParams q = p;
+        q.a = p.b; q.b = p.a;
+        q.M = N; q.N = M;
+        q.lda = ldb; q.ldb = lda;
+        q.sa = stride_b; q.sb = stride_a;
+        q.swapped = 1;
+        if (dtype == PARAS_BF16) launch_skinny<bf16_t>(q, batch, s);
+        else                     launch_skinny<f16_t>(q, batch, s);
+        PARAS_HIP_TRY(hipGetLastError());
+        return PARAS_OK;
+    }
     int64_t n_units = (N + 2 * gemm::kBN - 1) / (2 * gemm::kBN);
     const int64_t wide_tiles = (M + gemm::wide::kBM - 1) / gemm::wide::kBM * n_units * batch;
     // measured: faster from a little over half a round of one workgroup per CU upwards (at exactly 128
@@ -819,12 +861,12 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
         const int tsplits = tile_splitk_plan(M, N, K, batch, &kper);
         const size_t tneed = static_cast<size_t>(tsplits) * static_cast<size_t>(batch) * static_cast<size_t>(M) * static_cast<size_t>(N) * sizeof(float);
         if (tsplits >= 2 && workspace_bytes >= tneed && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
-            p.m_tiles = 1;
+            p.m_tiles = static_cast<int>((M + gemm::kBM - 1) / gemm::kBM);
             p.n_units = static_cast<int>((N + gemm::kBN - 1) / gemm::kBN);
             p.splits = tsplits;
             p.k_per_split = kper;
             p.partial = static_cast<float*>(workspace);
-            const unsigned blocks = static_cast<unsigned>(static_cast<long>(p.n_units) * batch * tsplits);
+            const unsigned blocks = static_cast<unsigned>(static_cast<long>(p.m_tiles) * p.n_units * batch * tsplits);
             const bool bf = dtype == PARAS_BF16;
             if (bf) hipLaunchKernelGGL((dense_gemm_nt_kernel<bf16_t, gemm::Tile128x128, true>), dim3(blocks), dim3(gemm::Tile128x128::kThreads), 0, s, p);
             else    hipLaunchKernelGGL((dense_gemm_nt_kernel<f16_t, gemm::Tile128x128, true>), dim3(blocks), dim3(gemm::Tile128x128::kThreads), 0, s, p);

@@ -323,3 +323,36 @@ def test_l2_stream_probe_reports_plausible_rates():
     assert 5.0 < got[(1, 512)] < got[(1, 64)], got      # measured 21 - 26 B/ns per CU from the last-level cache
     assert 10.0 < got[(0, 64)] < 400.0, got             # measured 33 B/ns per CU with eight loads in flight per wavefront
     assert capi.lib().paras_l2_stream_probe(1, 48, C.byref(rate)) != 0        # not a power of two
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(16384, 8, 4096), (5000, 1, 256), (3001, 17, 512), (2048, 32, 1024), (3001, 33, 512), (2048, 128, 1024), (700, 100, 192), (9000, 64, 4096)])
+def test_gemm_nt_few_columns_and_many_rows(shape, dtype):
+    """A router's logits and the like (tokens x experts): the few-row kernels with the operands in each
+    other's place and the results stored transposed; plain, with a bias over the columns, with a full
+    addend and a scale, and batched."""
+    M, N, K = shape
+    torch.manual_seed(M + N)
+    a = torch.randn(M, K).to(dtype)
+    b = (0.1 * torch.randn(N, K)).to(dtype)
+    rows = torch.tensor([0, 1, 15, 16, 127, 128, M // 2, M - 2, M - 1])
+    out = capi.gemm_nt(a.cuda(), b.cuda())
+    assert out.shape == (M, N)
+    assert_gemm_close(out[rows], O.matmul_nt(a[rows], b), dtype)
+    # every element against an fp32 product on the device (nothing left unwritten, nothing misplaced;
+    # that product sums in another order, so small results get an absolute allowance)
+    ref = (a.cuda().float() @ b.cuda().float().t())
+    assert bool(((out.float() - ref).abs() <= 2.0 ** -7 * ref.abs().clamp_min(0.05)).all())
+    bias = torch.randn(N).to(dtype)
+    out2 = capi.gemm_nt(a.cuda(), b.cuda(), bias.cuda())
+    assert_gemm_close(out2[rows], torch.nn.functional.linear(a[rows], b, bias), dtype)
+    full = torch.randn(M, N).to(dtype)
+    out3 = capi.gemm_nt(a.cuda(), b.cuda(), full.cuda(), alpha=0.5, beta=2.0)
+    want3 = (0.5 * (a[rows].double() @ b.double().t()) + 2.0 * full[rows].double())
+    assert_gemm_close(out3[rows], want3, dtype)
+    ab = torch.stack([a[:600], a[600:1200]]) if M >= 1200 else None
+    if ab is not None:
+        bb = torch.stack([b, b.flip(0)])
+        ob = capi.gemm_nt(ab.cuda(), bb.cuda())
+        for i in range(2):
+            assert_gemm_close(ob[i, -3:], O.matmul_nt(ab[i, -3:], bb[i]), dtype)
