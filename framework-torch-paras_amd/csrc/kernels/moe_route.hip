@@ -31,6 +31,8 @@
 //                  hits an expert at most once), plus the start position
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <atomic>
 #include <cmath>
 #include <cstdint>
@@ -47,7 +49,8 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kMaxExperts = 64;
+constexpr int kMaxExperts = 256;          // one thread of a workgroup per expert
+constexpr int kOwnScratchMaxExperts = 64; // what the library's own scratch areas and the allocation-free entry point are sized for
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void route_topk_kernel(
@@ -202,8 +205,12 @@ __global__ __launch_bounds__(kBlock) void route_clear_kernel(unsigned long long*
     if (i < n) words[i] = 0ull;
 }
 
-// kSmall: E <= 8 and k <= 8, the row and the selection live in registers.
-template <typename T, bool kSmall>
+// NR > 0: E <= NR and k <= 8, the row and the selection live in registers -- 8: as doubles (any
+// tensor type); 16, 32, 64: as floats, which hold 16-bit and fp32 logits exactly and compare like
+// them (not for fp64 tensors).  NR = 0: the row is read from memory in every selection pass and
+// the selection back from `topi` for every expert (E x k loads per token, three times over:
+// T = 8192, E = 64, k = 8 took 228 us this way, 12 x the time of E = 8, k = 2).
+template <typename T, int NR>
 __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     const typename Elem<T>::store_t* __restrict__ logits, long T_, int E, int k, long* __restrict__ topi,
     float* __restrict__ topw, long* __restrict__ order, long* __restrict__ inv_order, long* __restrict__ counts,
@@ -227,13 +234,16 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
     }
 
     // ---- top-k of this lane's token ---------------------------------
+    constexpr bool kSmall = NR > 0;
+    using V = typename std::conditional<(NR > 8), float, double>::type;     // what the row is held and compared as
+    static_assert(NR <= 8 || sizeof(typename El::store_t) <= 4, "fp64 logits do not fit floats");
     int sel[kSmall ? 8 : 1];                  // chosen expert per slot (small path)
     double kept[kSmall ? 8 : 1];              // the kept values as fp32 (the softmax input is topv.float())
     double vmax = -INFINITY;
     if (live) {
         const auto* row = logits + t * E;
-        double val[kSmall ? 8 : 1];
-        if constexpr (kSmall) {
+        V val[kSmall ? NR : 1];
+        if constexpr (NR == 8) {
             if (sizeof(typename El::store_t) == 2 && E == 8 && (reinterpret_cast<std::uintptr_t>(logits) & 15) == 0) {     // the row is one aligned 16-byte load
                 const u32x4 w = load16(row);
 #pragma unroll
@@ -243,15 +253,33 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
 #pragma unroll
                 for (int j = 0; j < 8; ++j) val[j] = j < E ? El::to_f64(row[j]) : 0.0;
             }
+        } else if constexpr (NR > 8) {
+            if (sizeof(typename El::store_t) == 2 && E % 8 == 0 && (reinterpret_cast<std::uintptr_t>(logits) & 15) == 0) {  // rows of aligned 16-byte pieces
+#pragma unroll
+                for (int c = 0; c < NR / 8; ++c) {
+                    if (c * 8 < E) {
+                        const u32x4 w = load16(row + c * 8);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            val[c * 8 + j] = static_cast<float>(El::to_f32(static_cast<typename El::store_t>(w[j >> 1] >> (16 * (j & 1)))));
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) val[c * 8 + j] = 0.f;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NR; ++j) val[j] = j < E ? static_cast<float>(El::to_f32(row[j])) : 0.f;
+            }
         }
-        double prev_val = 0.0;
+        V prev_val = 0;
         int prev_idx = -1;
         bool has_prev = false;
         for (int s = 0; s < k; ++s) {
-            double best_val = 0.0;
+            V best_val = 0;
             int best_idx = -1;
             bool has_best = false;
-            auto consider = [&](int j, double v) {
+            auto consider = [&](int j, V v) {
                 const bool within = !has_prev || (v < prev_val) || (v == prev_val && j > prev_idx);
                 const bool better = !has_best || (v > best_val) || (v == best_val && j < best_idx);
                 if (within && better) {
@@ -262,7 +290,7 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
             };
             if constexpr (kSmall) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
+                for (int j = 0; j < NR; ++j)
                     if (j < E) consider(j, val[j]);
             } else {
                 for (int j = 0; j < E; ++j) consider(j, El::to_f64(row[j]));
@@ -419,22 +447,36 @@ __global__ __launch_bounds__(kBlock) void route_fused_kernel(
         }
         __syncthreads();
     }
-    // exclusive scan over the experts by the first wave (E <= 64, totals below 2^31)
+    // exclusive scan over the experts by the first wave: a lane takes kMaxExperts / 64 consecutive
+    // experts (totals below 2^31)
     if (wave == 0) {
-        const int c = lane < E ? all_cnt[lane] : 0;
-        int incl = c;
+        constexpr int kPerLane = kMaxExperts / kWave;
+        int c[kPerLane], mine = 0;
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) {
+            const int e = lane * kPerLane + i;
+            c[i] = e < E ? all_cnt[e] : 0;
+            mine += c[i];
+        }
+        int incl = mine;
 #pragma unroll
         for (int d = 1; d < kWave; d <<= 1) {
             const int up = __shfl_up(incl, d, kWave);
             if (lane >= d) incl += up;
         }
-        if (lane < E) {
-            tot[lane] = incl - c;
-            if (bid == 0) {
-                counts[lane] = c;
-                offsets[lane] = incl - c;
-                if (lane == E - 1) offsets[E] = incl;
+        int run = incl - mine;
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) {
+            const int e = lane * kPerLane + i;
+            if (e < E) {
+                tot[e] = run;
+                if (bid == 0) {
+                    counts[e] = c[i];
+                    offsets[e] = run;
+                    if (e == E - 1) offsets[E] = run + c[i];
+                }
             }
+            run += c[i];
         }
     }
     __syncthreads();
@@ -471,12 +513,16 @@ void launch_fused(const void* logits, long T_, int E, int k, long* topi, float* 
                            reinterpret_cast<unsigned long long*>(scratch + kScratchHeader), n_words);
         epoch = 1;
     }
-    if (E <= 8 && k <= 8)
-        hipLaunchKernelGGL((route_fused_kernel<T, true>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, epoch, spin, kWaitTicks);
-    else
-        hipLaunchKernelGGL((route_fused_kernel<T, false>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi,
-                           topw, order, inv_order, counts, offsets, scratch, epoch, spin, kWaitTicks);
+#define PARAS_ROUTE_FUSED(NR_)                                                                                          \
+    hipLaunchKernelGGL((route_fused_kernel<T, NR_>), grid, block, 0, s, static_cast<const store_t*>(logits), T_, E, k, topi, \
+                       topw, order, inv_order, counts, offsets, scratch, epoch, spin, kWaitTicks)
+    constexpr bool kFloats = sizeof(store_t) <= 4;       // 16-bit and fp32 logits: a row of up to 64 fits registers as floats
+    if (E <= 8 && k <= 8) PARAS_ROUTE_FUSED(8);
+    else if (kFloats && k <= 8 && E <= 16) PARAS_ROUTE_FUSED((kFloats ? 16 : 0));
+    else if (kFloats && k <= 8 && E <= 32) PARAS_ROUTE_FUSED((kFloats ? 32 : 0));
+    else if (kFloats && k <= 8 && E <= 64) PARAS_ROUTE_FUSED((kFloats ? 64 : 0));
+    else PARAS_ROUTE_FUSED(0);
+#undef PARAS_ROUTE_FUSED
 }
 
 // Shared by the entry points: routes on `scratch` (device memory of route_scratch_bytes(T, E)).
@@ -505,7 +551,7 @@ size_t route_scratch_bytes(long T_, long E) {
 // Scratch of the allocation-free entry point: one copy per GPU, held until the process ends.
 // Its name is a host-side stand-in, not a device address: host code only ever uses the
 // per-device address hipGetSymbolAddress returns (static_scratch_for below).
-constexpr size_t kStaticScratchBytes = static_cast<size_t>(kScratchHeader) + static_cast<size_t>(kFusedMaxBlocks) * kMaxExperts * sizeof(unsigned long long);
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(kScratchHeader) + static_cast<size_t>(kFusedMaxBlocks) * kOwnScratchMaxExperts * sizeof(unsigned long long);
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxGpus = 64;
@@ -626,7 +672,7 @@ int paras_moe_route(const void* logits, int64_t T, int64_t E, int64_t k, int dty
         unsigned char* area = static_cast<unsigned char*>(workspace);
         unsigned long long epoch = 0;
         const char* own = std::getenv("PARAS_ROUTE_OWN_SCRATCH");
-        if ((own == nullptr || std::atoi(own) != 0) && !stream_is_capturing(s)) {
+        if ((own == nullptr || std::atoi(own) != 0) && E <= kOwnScratchMaxExperts && !stream_is_capturing(s)) {
             unsigned char* base = nullptr;
             rc = epoch_scratch_for(s, &base);
             if (rc != PARAS_OK) return rc;
@@ -672,7 +718,7 @@ int paras_moe_route_noalloc(const void* logits, int64_t T, int64_t E, int64_t k,
     PARAS_REQUIRE(T >= 1, "paras_moe_route_noalloc: at least one token is required");
     PARAS_REQUIRE(T <= kFusedMaxTokens, "paras_moe_route_noalloc: %lld tokens exceed the static scratch (at most %ld tokens)",
                   static_cast<long long>(T), kFusedMaxTokens);
-    PARAS_REQUIRE(E >= 1 && E <= kMaxExperts, "paras_moe_route_noalloc: expert count must be in [1, %d]", kMaxExperts);
+    PARAS_REQUIRE(E >= 1 && E <= kOwnScratchMaxExperts, "paras_moe_route_noalloc: expert count must be in [1, %d] (the static scratch is sized for that)", kOwnScratchMaxExperts);
     PARAS_REQUIRE(k >= 1 && k <= E, "paras topk: k out of range");
     PARAS_REQUIRE(T * k <= 0x7fffffffL, "paras_moe_route_noalloc: too many routed rows");
     PARAS_REQUIRE(logits && topi && topw && order && counts && offsets, "paras_moe_route_noalloc: null pointer");

@@ -95,7 +95,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor, Tensor> moe_route(const Tenso
     require_same_device("paras moe_route", logits, {});
     Tensor lg = logits.contiguous();
     const int64_t T = lg.size(0), E = lg.size(1);
-    TORCH_CHECK(E >= 1 && E <= 64, "paras moe_route: expert count must be in [1, 64]");
+    TORCH_CHECK(E >= 1 && E <= 256, "paras moe_route: expert count must be in [1, 256]");
     TORCH_CHECK(k >= 1 && k <= E, "paras topk: k out of range");
     const auto i64 = lg.options().dtype(c10::kLong);
     Tensor topi = at::empty({T, k}, i64), topw = at::empty({T, k}, lg.options().dtype(c10::kFloat));

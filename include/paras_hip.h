@@ -263,7 +263,9 @@ PARAS_API const char* paras_sdpa_kernel_name(const paras_sdpa_args* args);
 /* logits: [T, E] dtype `dtype`; topi: [T, k] int64; topw: [T, k] fp32;       */
 /* order: [T*k] int64 (order[p] = t*k + slot of the p-th routed row);         */
 /* inv_order: [T*k] int64 (position of flat slot in `order`; may be NULL);    */
-/* counts: [E] int64; offsets: [E+1] int64.  1 <= k <= E <= 64.               */
+/* counts: [E] int64; offsets: [E+1] int64.  1 <= k <= E <= 256 (up to 64     */
+/* experts and 8 choices a token's logits and choices stay in registers;      */
+/* beyond that they are re-read from memory, several times slower per token). */
 /* `workspace`: paras_moe_route_workspace(T,E,k) bytes of device memory        */
 /* (per-workgroup expert counts; contents on entry do not matter).  Up to      */
 /* 65536 tokens the whole routing is one kernel: its workgroups publish their  */

@@ -28,7 +28,8 @@ def test_route_golden(tag):
 
 
 @pytest.mark.parametrize("shape", [(1, 8, 2), (100, 8, 2), (1000, 8, 2), (777, 16, 4), (300, 64, 8), (5000, 3, 3),
-                                   (8192, 8, 2), (257, 1, 1), (4096, 8, 8)])
+                                   (8192, 8, 2), (257, 1, 1), (4096, 8, 8), (1500, 32, 8), (999, 24, 3), (2100, 60, 7),
+                                   (8192, 64, 8), (1000, 128, 8), (3000, 256, 8), (500, 200, 6), (70000, 128, 4)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_route_matches_oracle(shape, dtype):
     T, E, k = shape
