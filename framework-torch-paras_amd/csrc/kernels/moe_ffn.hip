@@ -25,6 +25,7 @@
 // that the workgroups resident on one XCD cover all m-tiles of a few column
 // tiles: weight tiles are then shared through that XCD's L2.
 #include <hip/hip_runtime.h>
+#include <cstdlib>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
@@ -188,6 +189,139 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
                     }
                 }
             }
+    }
+}
+
+// ---- few rows per expert (decode-time batches): the layer is bound by streaming every active
+// expert's weights once, which 128-row tiles with a handful of live rows do at half the memory
+// rate (and a single token, two active experts, at a fifth of it: its down-projection is 32
+// workgroups).  Here, as in the dense few-row kernel: a workgroup owns 16 weight rows of one expert
+// (for the gate-up GEMM the 16 gate rows and the 16 up rows of the same columns), its eight waves
+// split the contraction in pieces of 64 and feed v_mfma_f32_16x16x32 straight from global memory
+// (weights as the row operand; the expert's few routed rows, from L2, as the other), the eight
+// partial results meet in LDS in wave order.  An expert's rows are taken MB x 16 at a time, so any
+// count works (the weights of a second pass come from L2); experts without rows return at once.
+template <typename T> struct Mma16x16;
+template <> struct Mma16x16<bf16_t> {
+    __device__ static __forceinline__ float4_t run(u32x4 a, u32x4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma16x16<f16_t> {
+    __device__ static __forceinline__ float4_t run(u32x4 a, u32x4 b, float4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+constexpr int kFewWaves = 8;
+
+template <typename T, bool kSwiglu, int MB>
+__global__ __launch_bounds__(kFewWaves * 64) void grouped_few_rows_kernel(const FfnGemmParams p) {
+    using El = Elem<T>;
+    constexpr int NB = kSwiglu ? 2 : 1;                 // weight blocks: gate and up, or one
+    __shared__ float4_t part[kFewWaves][NB * MB][64];
+    const int e = blockIdx.y;
+    const long row_lo = p.offsets[e], row_hi = p.offsets[e + 1];
+    if (row_lo >= row_hi) return;                        // (uniform)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, kg = lane >> 4;
+    const long n0 = static_cast<long>(blockIdx.x) * 16;
+    long wrow = n0 + r16;
+    if (wrow >= p.Nw) wrow = p.Nw - 1;                   // clamped rows are computed but never stored
+    const std::uint16_t* wp[NB];
+    wp[0] = p.b + (static_cast<long>(e) * p.Nw + wrow) * p.K + kg * 16;
+    if constexpr (kSwiglu) wp[1] = p.b2 + (static_cast<long>(e) * p.Nw + wrow) * p.K + kg * 16;
+    const long pieces = p.K / 64;
+    // this wave's pieces of the contraction: wave, wave + 8, ...
+    const long mine = pieces > wave ? (pieces - wave + kFewWaves - 1) / kFewWaves : 0;
+
+    for (long chunk = row_lo; chunk < row_hi; chunk += MB * 16) {
+        const std::uint16_t* xp[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            long prow = chunk + mb * 16 + r16;
+            if (prow >= row_hi) prow = row_hi - 1;
+            const long src = p.order ? static_cast<long>((static_cast<unsigned long long>(static_cast<unsigned>(p.order[prow])) * p.div_m) >> p.div_s) : prow;
+            xp[mb] = p.a + src * p.K + kg * 16;
+        }
+        float4_t acc[NB][MB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+        // two pieces per trip, every load of the trip requested before its first MFMA; lane group kg
+        // supplies elements 16 kg .. + 7 of a piece to the first MFMA and the next eight to the
+        // second (any assignment works as long as both operands use the same one)
+        long t = 0;
+        for (; t + 2 <= mine; t += 2) {
+            u32x4 wv[2][2][NB], xv[2][2][MB];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const long kk = (wave + (t + u) * kFewWaves) * 64 + h * 8;
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) wv[u][h][nb] = load16(wp[nb] + kk);
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) xv[u][h][mb] = load16(xp[mb] + kk);
+                }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16x16<T>::run(wv[u][h][nb], xv[u][h][mb], acc[nb][mb]);
+        }
+        for (; t < mine; ++t) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const long kk = (wave + t * kFewWaves) * 64 + h * 8;
+                u32x4 wv[NB];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) wv[nb] = load16(wp[nb] + kk);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const u32x4 xv = load16(xp[mb] + kk);
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = Mma16x16<T>::run(wv[nb], xv, acc[nb][mb]);
+                }
+            }
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) part[wave][nb * MB + mb][lane] = acc[nb][mb];
+        __syncthreads();
+        // wave w finishes row block w, w + 8, ...: lane l holds routed row l % 16 of the block and the
+        // four weight rows (output columns) 4 (l / 16) .. + 3
+        for (int mb = wave; mb < MB; mb += kFewWaves) {
+            float4_t g = part[0][mb][lane], u = float4_t{0.f, 0.f, 0.f, 0.f};
+            if constexpr (kSwiglu) u = part[0][MB + mb][lane];
+#pragma unroll
+            for (int w = 1; w < kFewWaves; ++w) {
+                const float4_t o = part[w][mb][lane];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) g[r] += o[r];
+                if constexpr (kSwiglu) {
+                    const float4_t o2 = part[w][MB + mb][lane];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) u[r] += o2[r];
+                }
+            }
+            const long prow = chunk + mb * 16 + r16;
+            const long col = n0 + 4 * kg;
+            if (prow < row_hi) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (col + r >= p.N) continue;
+                    if constexpr (kSwiglu) p.c[prow * p.N + col + r] = swiglu_from_acc<T>(g[r], u[r]);
+                    else                   p.c[prow * p.N + col + r] = El::from_f32(g[r]);
+                }
+            }
+        }
+        __syncthreads();                                 // `part` is free for the next rows
     }
 }
 
@@ -367,6 +501,45 @@ int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const voi
     return PARAS_OK;
 }
 
+template <typename T>
+int run_ffn_few_rows(const void* x, const void* w_gate, const void* w_up, const void* w_down, const float* topw,
+                     const long* order, const long* inv_order, const long* offsets, void* out, void* workspace, long T_,
+                     int E, int k, long H, long I, hipStream_t s) {
+    const long R = T_ * k;
+    auto* h = static_cast<std::uint16_t*>(workspace);
+    auto* y = reinterpret_cast<std::uint16_t*>(static_cast<char*>(workspace) + align_up(static_cast<size_t>(R) * I * 2, 256));
+    FfnGemmParams g1{};
+    g1.a = static_cast<const std::uint16_t*>(x);
+    g1.b = static_cast<const std::uint16_t*>(w_gate);
+    g1.b2 = static_cast<const std::uint16_t*>(w_up);
+    g1.c = h;
+    g1.order = order;
+    g1.offsets = offsets;
+    g1.K = H; g1.N = I; g1.Nw = I; g1.R = R; g1.E = E; g1.k = k;
+    division_by(static_cast<unsigned>(k), &g1.div_m, &g1.div_s);
+    hipLaunchKernelGGL((grouped_few_rows_kernel<T, true, 2>), dim3(static_cast<unsigned>((I + 15) / 16), static_cast<unsigned>(E)),
+                       dim3(kFewWaves * 64), 0, s, g1);
+    PARAS_HIP_TRY(hipGetLastError());
+    FfnGemmParams g2{};
+    g2.a = h;
+    g2.b = static_cast<const std::uint16_t*>(w_down);
+    g2.b2 = g2.b;
+    g2.c = y;
+    g2.order = nullptr;
+    g2.offsets = offsets;
+    g2.K = I; g2.N = H; g2.Nw = H; g2.R = R; g2.E = E; g2.k = k;
+    hipLaunchKernelGGL((grouped_few_rows_kernel<T, false, 2>), dim3(static_cast<unsigned>((H + 15) / 16), static_cast<unsigned>(E)),
+                       dim3(kFewWaves * 64), 0, s, g2);
+    PARAS_HIP_TRY(hipGetLastError());
+    const long total = T_ * (H / 8);
+    long blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    hipLaunchKernelGGL((moe_combine_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, s, y, topw,
+                       inv_order, static_cast<std::uint16_t*>(out), T_, k, H);
+    PARAS_HIP_TRY(hipGetLastError());
+    return PARAS_OK;
+}
+
 // 256-row tiles when the experts are big enough for them: an expert's last tile is half empty on
 // average, so the rows per expert should be many times the tile, and there must be tiles for at
 // least half the CUs.
@@ -375,6 +548,14 @@ int run_ffn(const void* x, const void* w_gate, const void* w_up, const void* w_d
             const long* order, const long* inv_order, const long* offsets, void* out, void* workspace, long T_,
             int E, int k, long H, long I, hipStream_t s) {
     const long R = T_ * k;
+    // Up to 16 routed rows per expert on average the few-row kernels (an expert with more than 32 rows
+    // takes them 32 at a time).  8 experts, top-2, H = 4096, I = 14336, tiles against few-row kernels:
+    // 1 token 421 / 168 us, 8 tokens 615 / 397, 32 tokens 659 / 574, 64 tokens 663 / 667, 128 tokens
+    // 672 / 1124.  PARAS_MOE_FEW_ROWS = n moves the limit (0: never).
+    static const char* few_env = std::getenv("PARAS_MOE_FEW_ROWS");
+    const long few_limit = few_env != nullptr ? std::atol(few_env) : 16;
+    if (R <= few_limit * E && E <= 65535 && (I + 15) / 16 <= 0x7fffffffL)
+        return run_ffn_few_rows<T>(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, out, workspace, T_, E, k, H, I, s);
     const long wide_tiles = (R / Tile256::kBM) * ((H + 2 * kBN - 1) / (2 * kBN));
     if (R / E >= 4 * Tile256::kBM && wide_tiles >= 128)
         return run_ffn_shape<T, Tile256>(x, w_gate, w_up, w_down, topw, order, inv_order, offsets, out, workspace, T_, E, k, H, I, s);

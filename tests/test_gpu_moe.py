@@ -54,6 +54,27 @@ def test_route_quantised_logits_many_ties_and_skew():
     assert got[4][2].item() == 0 and got[4][5].item() == 3000
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T", [1, 7, 40, 64])
+def test_ffn_few_rows_per_expert(T, dtype):
+    """Decode-time batches run on the few-row kernels (a workgroup per 16 weight rows of an expert,
+    the expert's rows 32 at a time): experts without a row, an expert with more than 32 rows (most
+    tokens choose expert 3 first), a single token."""
+    E, k, H, I = 8, 2, 256, 512
+    torch.manual_seed(T)
+    x = torch.randn(T, H).to(dtype)
+    wg, wu, wd = (0.05 * torch.randn(E, I, H)).to(dtype), (0.05 * torch.randn(E, I, H)).to(dtype), (0.05 * torch.randn(E, H, I)).to(dtype)
+    logits = torch.randn(T, E)
+    logits[:, 3] += 6.0                    # everybody's first choice
+    logits[:, 5:] -= 9.0                   # nobody's choice
+    logits = logits.to(dtype)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    assert counts[3].item() == T and counts[5:].sum().item() == 0
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k)
+    want = O.moe_ffn(x, wg, wu, wd, topw.cpu(), order.cpu(), inv.cpu(), offsets.cpu(), k)
+    assert_ffn_close(out, want, dtype)
+
+
 def test_route_errors_and_empty():
     with pytest.raises(capi.ParasError, match="k out of range"):
         capi.moe_route(torch.randn(4, 8, device="cuda"), 9)
