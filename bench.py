@@ -423,8 +423,8 @@ def main() -> int:
         tf = flops / ms / 1e9
         results["linear"] = {
             "workload": "bf16 dense NT GEMM x W^T: M=16384 N=4096 K=4096 (nn.Linear of configs[2]'s tokens)",
-            "value": round(tf, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "kernel": "dense_gemm_nt_kernel<bf16>",
-            "algorithmic_flops_per_launch": flops, "roofline": roofline("mfma", tf, "dense_gemm_nt_kernel"),
+            "value": round(tf, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 4), "kernel": "dense_gemm_nt_quad16_kernel<bf16>",
+            "algorithmic_flops_per_launch": flops, "roofline": roofline("mfma", tf, "dense_gemm_nt_quad16_kernel"),
         }
         log(f"linear: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s ({tf / MFMA_BF16_PEAK_TFLOPS:.1%})")
         lin_got = yc[M - 64:].cpu()

@@ -190,6 +190,94 @@ __global__ __launch_bounds__(S::kThreads, (S::kGroups == 1 ? 3 : 2)) void dense_
             }
 }
 
+// The 256 x 256 tile of four waves on v_mfma_f32_16x16x32 (gemm_tile.h, namespace quad16): what the
+// dense product runs on from 144 tiles on.  Same-box timings against the eight-wave tile of
+// 32 x 32 x 16 MFMAs, which it replaces here: 16384 x 4096 x 4096 414.6 against 424.6 us (bench.py,
+// sustained: 415 against 427), 8192^3 806 against 836 us, N = 14336 1477 against 1500 us.
+template <typename T>
+__global__ __launch_bounds__(quad16::kThreads, 1) void dense_gemm_nt_quad16_kernel(const DenseParams p) {
+    using El = Elem<T>;
+    __shared__ __attribute__((aligned(16))) quad16::TileLds lds;
+    long bidx;
+    int mt, nu;
+    if (!tile_of_workgroup(p, blockIdx.x, bidx, mt, nu)) return;      // (the whole workgroup: nobody is left at a barrier)
+    const long row0 = static_cast<long>(mt) * quad16::kBM, n0 = static_cast<long>(nu) * 2 * kBN;
+    const std::uint16_t* A = p.a + bidx * p.sa;
+    const std::uint16_t* B = p.b + bidx * p.sb;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    unsigned a_off[8], b_off[2][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = tid + i * quad16::kThreads;
+        long arow = row0 + (c >> 3);
+        if (arow >= p.M) arow = p.M - 1;     // clamped rows are computed but never stored
+        a_off[i] = static_cast<unsigned>(arow * p.lda + (c & 7) * 8);
+    }
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * quad16::kThreads;
+            long brow = n0 + g * kBN + (c >> 3);
+            if (brow >= p.N) brow = p.N - 1;
+            b_off[g][i] = static_cast<unsigned>(brow * p.ldb + (c & 7) * 8);
+        }
+    const std::uint16_t* b_base[2] = {B, B};
+    quad16::float4v acc[8][8];
+    quad16::tile_mainloop<T>(A, a_off, b_base, b_off, p.K, lds, acc);
+
+    // epilogue: lane (l16 = lane % 16, kq = lane / 16) of block (i, j) holds row i*16 + l16 and columns
+    // 4 kq .. + 3 of column block j (group j / 4, columns wn*64 + (j % 4)*16 of it)
+    const int l16 = lane & 15, kq = lane >> 4;
+    std::uint16_t* C = p.c + bidx * p.sc;
+    const std::uint16_t* ADD = p.add ? p.add + bidx * p.sadd : nullptr;
+    // the plain product into rows of 8-byte aligned pieces: the conversion instruction, four columns per store;
+    // a row block in which a NaN turns up takes the software narrowing (which writes NaNs as the host's types do)
+    const bool plain = p.alpha == 1.0f && ADD == nullptr && p.ldc % 4 == 0 && p.sc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) & 7) == 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const long row = row0 + wm * 128 + i * 16 + l16;
+        bool nan_here = false;
+        if (plain) {
+            float probe = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) probe += acc[i][j][r];
+            nan_here = __builtin_amdgcn_ballot_w64(probe != probe) != 0;      // (an infinity minus an infinity counts as well)
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const long col = n0 + (j >> 2) * kBN + wn * 64 + (j & 3) * 16 + 4 * kq;
+            if (row >= p.M || col >= p.N) continue;
+            if (plain && col + 3 < p.N) {
+                std::uint16_t o[4];
+                if (__builtin_expect(nan_here, 0)) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[r] = El::from_f32(acc[i][j][r]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[r] = El::from_f32_finite(acc[i][j][r]);
+                }
+                u32x2 w2;
+                w2[0] = o[0] | (static_cast<std::uint32_t>(o[1]) << 16);
+                w2[1] = o[2] | (static_cast<std::uint32_t>(o[3]) << 16);
+                *reinterpret_cast<u32x2*>(C + row * p.ldc + col) = w2;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (col + r >= p.N) continue;
+                    float v = p.alpha * acc[i][j][r];
+                    if (ADD) v = fmaf(p.beta, El::to_f32(ADD[row * p.ld_add + col + r]), v);
+                    C[row * p.ldc + col + r] = El::from_f32(v);
+                }
+            }
+        }
+    }
+}
+
 // ---- few rows (M <= 128): the decode-time projections.  The product is bound by streaming the
 // weights once, so there is no tile and no LDS staging: a workgroup owns 16 weight rows, its eight
 // waves split the contraction (pieces of 64 dealt round-robin, so the eight read adjacent 128-byte
@@ -915,7 +1003,11 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
             blocks = static_cast<unsigned>(wgs);
         }
     }
-    if (use_wide) {
+    static const bool eight_waves = std::getenv("PARAS_GEMM_EIGHT_WAVES") != nullptr;     // the eight-wave tile of 32 x 32 x 16 MFMAs, for measurements
+    if (use_wide && !eight_waves) {
+        if (dtype == PARAS_BF16) hipLaunchKernelGGL((dense_gemm_nt_quad16_kernel<bf16_t>), dim3(blocks), dim3(quad16::kThreads), 0, s, p);
+        else                     hipLaunchKernelGGL((dense_gemm_nt_quad16_kernel<f16_t>), dim3(blocks), dim3(quad16::kThreads), 0, s, p);
+    } else if (use_wide) {
         if (dtype == PARAS_BF16) launch_dense<bf16_t, gemm::Tile256>(p, blocks, s);
         else                     launch_dense<f16_t, gemm::Tile256>(p, blocks, s);
     } else if (use_square) {

@@ -315,6 +315,114 @@ __device__ __forceinline__ void short_tile_mainloop(const std::uint16_t* a_base,
 
 }  // namespace wide
 
+// The 256 x (2 x 128) tile once more, for the dense kernel: four waves arranged 2 x 2, one wave per
+// SIMD, each with 128 x 128 as 8 x 8 blocks of v_mfma_f32_16x16x32 (four accumulator registers per
+// block, 256 in all: the accumulation half of the register file).  Per flop that instruction
+// moves half the accumulator data of the 32 x 32 x 16 one, and the part is power limited under
+// MFMA load: a register-only loop of it sustains 2.19 PFLOP/s where the 32 x 32 x 16 loop sustains
+// 1.90 - 1.94.  A k-step (32 elements of the contraction) is 64 MFMAs on 8 + 8 fragments: a
+// quarter of an LDS read per MFMA, i.e. half a read per 32 x 32 x 16's worth of flops (0.75 in the
+// eight-wave tile).  Staging, stages and the place of the barrier as in the eight-wave tile.  The
+// B fragment is the instruction's first operand, so a lane ends up with four adjacent COLUMNS of
+// one row (8-byte stores): acc[i][j][r] = row i*16 + lane%16, column block j, column 4*(lane/16) + r of it.
+namespace quad16 {
+
+constexpr int kThreads = 256;
+constexpr int kBM = 256;
+using wide::StageLds;
+using wide::TileLds;
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+    __device__ static __forceinline__ float4v run(i16x8 a, i16x8 b, float4v c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mma<f16_t> {
+    __device__ static __forceinline__ float4v run(i16x8 a, i16x8 b, float4v c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[8],
+                                              const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][4],
+                                              long K, TileLds& lds, float4v (&acc)[8][8]) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    u32x4 a_st[8], b_st[2][4];
+    auto load_one = [&](int idx, long k0) {              // idx 0..7: A chunks, 8..15: B chunks (g, i)
+        if (idx < 8) a_st[idx] = load16(a_base + k0 + a_off[idx]);
+        else         b_st[(idx - 8) >> 2][(idx - 8) & 3] = load16(b_base[(idx - 8) >> 2] + k0 + b_off[(idx - 8) >> 2][(idx - 8) & 3]);
+    };
+    auto store_one = [&](StageLds& st, int idx) {
+        const int i = idx < 8 ? idx : (idx - 8) & 3;
+        const int c = tid + i * kThreads;
+        const int off = (c >> 3) * kLS + (c & 7) * 8;
+        if (idx < 8) *reinterpret_cast<u32x4*>(&st.a[off]) = a_st[idx];
+        else         *reinterpret_cast<u32x4*>(&st.b[(idx - 8) >> 2][off]) = b_st[(idx - 8) >> 2][i];
+    };
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    const int a_off0 = (wm * 128 + l16) * kLS + kq * 8;
+    const int b_off0 = (wn * 64 + l16) * kLS + kq * 8;
+    const long k_tiles = K / kBK;
+    // fragments of a k-step (32 elements of the contraction): 8 of A (16 rows each), 8 of B (column
+    // blocks j: group j / 4, columns wn*64 + (j % 4)*16 ..); two register sets
+    i16x8 af[2][8], bf[2][8];
+    auto read_frag = [&](const StageLds& st, int buf, int f, int ks) {     // f 0..7: A block, 8..15: B block
+        if (f < 8) af[buf][f] = *reinterpret_cast<const i16x8*>(&st.a[a_off0 + f * 16 * kLS + ks * 32]);
+        else       bf[buf][f - 8] = *reinterpret_cast<const i16x8*>(&st.b[(f - 8) >> 2][b_off0 + ((f - 8) & 3) * 16 * kLS + ks * 32]);
+    };
+    auto compute = [&](const StageLds& cur_st, StageLds& nxt_st, long k_after, auto next_tag) {
+        constexpr bool kNext = decltype(next_tag)::value;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const bool last = ks == 1;
+            if (kNext && last) __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int slot = j * 8 + i;
+                    acc[i][j] = Mma<T>::run(bf[ks][j], af[ks][i], acc[i][j]);
+                    if ((slot & 3) == 0) {          // one fragment of the next k-step every fourth MFMA
+                        if (!last) read_frag(cur_st, 1, slot >> 2, 1);
+                        else if (kNext) read_frag(nxt_st, 0, slot >> 2, 0);
+                    }
+                    // the next k-tile into the other stage during the first k-step, one chunk every fourth MFMA, each
+                    // followed two MFMAs later by the global load of the same chunk of the tile after that
+                    if (kNext && !last && (slot & 3) == 1) store_one(nxt_st, slot >> 2);
+                    if (kNext && !last && (slot & 3) == 3) load_one(slot >> 2, k_after);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        }
+    };
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) load_one(idx, 0);
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) store_one(lds.st[0], idx);
+    __syncthreads();
+    if (k_tiles > 1) {
+#pragma unroll
+        for (int idx = 0; idx < 16; ++idx) load_one(idx, kBK);
+    }
+#pragma unroll
+    for (int f = 0; f < 16; ++f) read_frag(lds.st[0], 0, f, 0);
+    for (long kt = 0; kt + 1 < k_tiles; ++kt) {
+        const long after = kt + 2 < k_tiles ? kt + 2 : k_tiles - 1;   // the last tiles reload a tile nobody stores
+        compute(lds.st[kt & 1], lds.st[(kt + 1) & 1], after * kBK, std::true_type{});
+    }
+    compute(lds.st[(k_tiles - 1) & 1], lds.st[k_tiles & 1], 0, std::false_type{});
+}
+
+}  // namespace quad16
+
 // ---- epilogue helpers.  A lane (column lr, half lh) of a 32 x 32 accumulator block holds rows
 // (r/4)*8 + 4*lh + r%4, r = 0..15.  Stores go to `blk` (the block's first column in the tile's first
 // row: the same address in every lane, so it stays in scalar registers) plus a 32-bit byte offset:
