@@ -381,8 +381,8 @@ def main() -> int:
             "workload": "bf16 MoE layer T=8192 H=4096 E=8 top-2 I=14336: routing + grouped expert FFN (configs[4])",
             "value": round(T / ms_all * 1e3, 1), "unit": "tokens/s", "ms_per_step": round(ms_all, 4), "steps": msteps,
             "route_ms": round(ms_route, 4), "ffn_ms": round(ms_ffn, 4), "ffn_tflops": round(tf, 2),
-            "kernel": "grouped_gemm_kernel<bf16> (gate-up+SwiGLU, down) + moe_combine_kernel",
-            "algorithmic_flops_per_launch": flops, "roofline": roofline("mfma", tf, "grouped_gemm_kernel"),
+            "kernel": "grouped_gemm_quad16_kernel<bf16> (gate-up+SwiGLU, down) + moe_combine_kernel",
+            "algorithmic_flops_per_launch": flops, "roofline": roofline("mfma", tf, "grouped_gemm_quad16_kernel"),
         }
         log(f"moe: route {ms_route * 1e3:.1f} us, ffn {ms_ffn * 1e3:.1f} us = {tf:.1f} TFLOP/s ({tf / MFMA_BF16_PEAK_TFLOPS:.1%}), "
             f"layer {ms_all * 1e3:.1f} us = {T / ms_all * 1e3:.0f} tokens/s")

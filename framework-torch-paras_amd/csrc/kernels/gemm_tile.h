@@ -421,6 +421,68 @@ __device__ __forceinline__ void tile_mainloop(const std::uint16_t* a_base, const
     compute(lds.st[(k_tiles - 1) & 1], lds.st[k_tiles & 1], 0, std::false_type{});
 }
 
+// A tile of which at most 64 rows exist (the last tile of a group of rows): the four waves share those
+// rows instead of three of them idling through the contraction.  Wave w takes all four row blocks and
+// the 32 columns w of BOTH column groups (two blocks of 16 each), so a gate / up pair still meets in one
+// lane: 16 MFMAs per k-step and wave instead of 64, every product summed in the same order as in the full
+// tile (bit-identical results).  Only the first 64 A rows are staged (a_off[0], a_off[1]: this thread's two
+// chunks of them); two LDS stages, one barrier per k-tile.  acc[i][jj]: row block i, column block
+// jj = 2 g + cb: rows i*16 + lane%16, columns w*32 + cb*16 + 4*(lane/16) + r of group g.
+template <typename T>
+__device__ __forceinline__ void short_tile_mainloop(const std::uint16_t* a_base, const unsigned (&a_off)[8],
+                                                    const std::uint16_t* const (&b_base)[2], const unsigned (&b_off)[2][4],
+                                                    long K, TileLds& lds, float4v (&acc)[4][4]) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, kq = lane >> 4;
+    u32x4 a_st[2], b_st[2][4];
+    auto load_tile = [&](long k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a_st[i] = load16(a_base + k0 + a_off[i]);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) b_st[g][i] = load16(b_base[g] + k0 + b_off[g][i]);
+    };
+    auto store_tile = [&](StageLds& st) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * kThreads;
+            const int off = (c >> 3) * kLS + (c & 7) * 8;
+            if (i < 2) *reinterpret_cast<u32x4*>(&st.a[off]) = a_st[i];
+#pragma unroll
+            for (int g = 0; g < 2; ++g) *reinterpret_cast<u32x4*>(&st.b[g][off]) = b_st[g][i];
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) acc[i][jj] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int a_o = l16 * kLS + kq * 8;
+    const int b_o = (wave * 32 + l16) * kLS + kq * 8;
+    const long k_tiles = K / kBK;
+    load_tile(0);
+    store_tile(lds.st[0]);
+    __syncthreads();
+    for (long kt = 0; kt < k_tiles; ++kt) {
+        const StageLds& cur = lds.st[kt & 1];
+        if (kt + 1 < k_tiles) load_tile((kt + 1) * kBK);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            i16x8 af[4], bf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const i16x8*>(&cur.a[a_o + i * 16 * kLS + ks * 32]);
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) bf[jj] = *reinterpret_cast<const i16x8*>(&cur.b[jj >> 1][b_o + (jj & 1) * 16 * kLS + ks * 32]);
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i][jj] = Mma<T>::run(bf[jj], af[i], acc[i][jj]);
+        }
+        if (kt + 1 < k_tiles) store_tile(lds.st[(kt + 1) & 1]);
+        __syncthreads();
+    }
+}
+
 }  // namespace quad16
 
 // ---- epilogue helpers.  A lane (column lr, half lh) of a 32 x 32 accumulator block holds rows

@@ -192,6 +192,234 @@ __global__ __launch_bounds__(S::kThreads, 2) void grouped_gemm_kernel(const FfnG
     }
 }
 
+// f(integral_constant<int, I>) for I = 0 .. N-1
+template <int... I, typename F>
+__device__ __forceinline__ void quad16_static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void quad16_static_for(F&& f) {
+    quad16_static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
+}
+
+// A wave's queue of SwiGLU values that left the common tier (four of one lane per entry): laid over the
+// tile stages once the contraction is done.
+struct SwigluQueue {
+    static constexpr unsigned kEntries = 1024;
+    unsigned where[kEntries];       // (row in the tile) << 16 | column in the column unit
+    quad16::float4v gate[kEntries], up[kEntries];
+};
+static_assert(4 * sizeof(SwigluQueue) <= sizeof(quad16::TileLds), "four queues in the tile stages");
+
+// The same on the four-wave tile of v_mfma_f32_16x16x32 (gemm_tile.h, namespace quad16): what the layer
+// runs on when the experts are big enough for 256-row tiles.  Tile coordinates, the search for the
+// m-tile's expert and the staging offsets as above (a thread stages eight chunks of A and four per
+// column group of B); a lane of accumulator block (i, j) holds row i*16 + lane%16 and columns
+// 4*(lane/16) .. + 3 of column block j (group j / 4, columns wn*64 + (j % 4)*16 of it), so gate and
+// up of one output sit in blocks j and j + 4 of the same lane and an output row gets 8-byte stores.
+template <typename T, bool kSwiglu>
+__global__ __launch_bounds__(quad16::kThreads, 1) void grouped_gemm_quad16_kernel(const FfnGemmParams p) {
+    using El = Elem<T>;
+    constexpr int kBM = quad16::kBM;
+    __shared__ __attribute__((aligned(16))) quad16::TileLds lds;
+    int mt, nu;
+    {
+        const long L = blockIdx.x;
+        const int xcd = static_cast<int>(L & 7);
+        const long j = L >> 3;
+        const long per_group = static_cast<long>(p.mt_total) * p.ngt;
+        const long g = j / per_group, rem = j % per_group;
+        mt = static_cast<int>(rem / p.ngt);
+        nu = static_cast<int>((g * 8 + xcd) * p.ngt + rem % p.ngt);
+        if (nu >= p.n_units) return;
+    }
+    int e = 0;
+    long row0 = 0, row_end = 0;
+    {
+        int tiles_before = 0;
+        bool found = false;
+        for (int i = 0; i < p.E; ++i) {
+            const long lo = p.offsets[i], hi = p.offsets[i + 1];
+            const int tiles = static_cast<int>((hi - lo + kBM - 1) / kBM);
+            if (!found && mt < tiles_before + tiles) {
+                e = i;
+                row0 = lo + static_cast<long>(mt - tiles_before) * kBM;
+                row_end = hi;
+                found = true;
+            }
+            tiles_before += tiles;
+        }
+        if (!found) return;
+    }
+    const long n0 = static_cast<long>(nu) * (kSwiglu ? kBN : 2 * kBN);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, kq = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    unsigned a_off[8], b_off[2][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = tid + i * quad16::kThreads;
+        long prow = row0 + (c >> 3);
+        if (prow >= row_end) prow = row_end - 1;  // clamp: result rows beyond the expert are not stored
+        const long src = p.order ? static_cast<long>((static_cast<unsigned long long>(static_cast<unsigned>(p.order[prow])) * p.div_m) >> p.div_s) : prow;
+        a_off[i] = static_cast<unsigned>(src * p.K + (c & 7) * 8);
+    }
+    const std::uint16_t* const b_base[2] = {p.b + static_cast<long>(e) * p.Nw * p.K, p.b2 + static_cast<long>(e) * p.Nw * p.K};
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * quad16::kThreads;
+            long wrow = (kSwiglu ? n0 : n0 + g * kBN) + (c >> 3);
+            if (wrow >= p.Nw) wrow = p.Nw - 1;
+            b_off[g][i] = static_cast<unsigned>(wrow * p.K + (c & 7) * 8);
+        }
+    // four values of one output row: SwiGLU of the gate / up pairs, or the narrowed product
+    auto put4 = [&](long prow, long col, const quad16::float4v a0, const quad16::float4v a1, bool nan_here) __attribute__((always_inline)) {
+        if (prow >= row_end || col >= p.N) return;
+        std::uint16_t o[4];
+        if constexpr (kSwiglu) {
+            swiglu4_from_acc<T>(a0, a1, o);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = __builtin_expect(nan_here, 0) ? El::from_f32(a0[r]) : El::from_f32_finite(a0[r]);
+        }
+        if (col + 3 < p.N) {        // (N is a multiple of 64 here and the rows are 16-byte aligned)
+            u32x2 w2;
+            w2[0] = o[0] | (static_cast<std::uint32_t>(o[1]) << 16);
+            w2[1] = o[2] | (static_cast<std::uint32_t>(o[3]) << 16);
+            *reinterpret_cast<u32x2*>(p.c + prow * p.N + col) = w2;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (col + r < p.N) p.c[prow * p.N + col + r] = o[r];
+        }
+    };
+    auto any_nan = [&](float probe) { return __builtin_amdgcn_ballot_w64(probe != probe) != 0; };
+
+    if (row_end - row0 <= 64) {     // an expert's last tile with few rows: the waves share them
+        quad16::float4v sacc[4][4];
+        quad16::short_tile_mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, sacc);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const long prow = row0 + i * 16 + l16;
+            bool nan_here = false;
+            if (!kSwiglu) {
+                float probe = 0.f;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) probe += sacc[i][jj][r];
+                nan_here = any_nan(probe);
+            }
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) {
+                const long col = n0 + wave * 32 + cb * 16 + 4 * kq;
+                if (kSwiglu) {
+                    put4(prow, col, sacc[i][cb], sacc[i][2 + cb], false);
+                } else {
+                    put4(prow, col, sacc[i][cb], sacc[i][cb], nan_here);
+                    put4(prow, col + kBN, sacc[i][2 + cb], sacc[i][2 + cb], nan_here);
+                }
+            }
+        }
+        return;
+    }
+    quad16::float4v acc[8][8];
+    quad16::tile_mainloop<T>(p.a, a_off, b_base, b_off, p.K, lds, acc);
+    if constexpr (kSwiglu) {
+        // About one value in a thousand leaves the common tier of SwiGLU, and where one lane of the 64 does,
+        // the whole wave walks through the fp64 formula: at 128 values a lane that happened eight times a tile
+        // and cost 4 % of the kernel.  A lane whose four values do not all pass queues them (the accumulators
+        // and where they go) in the wave's share of the tile stages, which nobody reads any more; after
+        // the last row block (or when the next one might not fit) the wave works its queue off, one value per lane.
+        __syncthreads();
+        // (the lane's coordinates derived again, from a value the compiler cannot trace: none of this is to
+        // occupy a register during the contraction, which has none to spare)
+        int t = threadIdx.x;
+        asm volatile("" : "+v"(t));
+        const int lane = t & 63, wave = t >> 6, l16 = t & 15, kq = (t >> 4) & 3, wm = t >> 7, wn = (t >> 6) & 1;
+        SwigluQueue& q = reinterpret_cast<SwigluQueue*>(&lds)[wave];
+        const unsigned long long lanes_below = (1ull << lane) - 1ull;
+        unsigned queued = 0;      // uniform
+        auto work_off = [&]() __attribute__((always_inline)) {
+            for (unsigned idx = lane; idx < 4 * queued; idx += 64) {
+                const unsigned e = idx >> 2, r = idx & 3, where = q.where[e];
+                const float a0 = reinterpret_cast<const float*>(&q.gate[e])[r];
+                const float a1 = reinterpret_cast<const float*>(&q.up[e])[r];
+                const long qcol = n0 + (where & 0xFFFFu) + r;
+                const std::uint16_t v = swiglu_from_acc<T>(a0, a1);
+                if (qcol < p.N) p.c[(row0 + (where >> 16)) * p.N + qcol] = v;
+            }
+            queued = 0;
+        };
+        quad16_static_for<8>([&](auto I) __attribute__((always_inline)) {
+            constexpr int i = decltype(I)::value;
+            const int trow = wm * 128 + i * 16 + l16;
+            const long prow = row0 + trow;
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb) {
+                const int tcol = wn * 64 + jb * 16 + 4 * kq;
+                const long col = n0 + tcol;
+                const bool live = prow < row_end && col < p.N;
+                std::uint16_t o[4];
+                const bool ok = swiglu4_common_tier<T>(acc[i][jb], acc[i][4 + jb], o);
+                if (live && ok) {
+                    if (col + 3 < p.N) {
+                        u32x2 w2;
+                        w2[0] = o[0] | (static_cast<std::uint32_t>(o[1]) << 16);
+                        w2[1] = o[2] | (static_cast<std::uint32_t>(o[3]) << 16);
+                        *reinterpret_cast<u32x2*>(p.c + prow * p.N + col) = w2;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (col + r < p.N) p.c[prow * p.N + col + r] = o[r];
+                    }
+                }
+                const unsigned long long left = __builtin_amdgcn_ballot_w64(live && !ok);
+                if (left != 0) {
+                    if (live && !ok) {
+                        const unsigned slot = queued + static_cast<unsigned>(__builtin_popcountll(left & lanes_below));
+                        q.where[slot] = (static_cast<unsigned>(trow) << 16) | static_cast<unsigned>(tcol);
+                        q.gate[slot] = acc[i][jb];
+                        q.up[slot] = acc[i][4 + jb];
+                    }
+                    queued += static_cast<unsigned>(__builtin_popcountll(left));
+                }
+            }
+            // a row block queues 4 x 64 entries at most
+            if (i == 7 || queued > SwigluQueue::kEntries - 256) work_off();
+        });
+        return;
+    }
+    // (row blocks as constants of the front end: the optimiser's unroller gives up on a loop of 128
+    // SwiGLU values with their exact tier, and the accumulators would move to scratch memory)
+    quad16_static_for<8>([&](auto I) __attribute__((always_inline)) {
+        constexpr int i = decltype(I)::value;
+        const long prow = row0 + wm * 128 + i * 16 + l16;
+        bool nan_here = false;
+        if (!kSwiglu) {
+            float probe = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) probe += acc[i][j][r];
+            nan_here = any_nan(probe);
+        }
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb) {
+            const long col = n0 + wn * 64 + jb * 16 + 4 * kq;
+            if (kSwiglu) {
+                put4(prow, col, acc[i][jb], acc[i][4 + jb], false);
+            } else {
+                put4(prow, col, acc[i][jb], acc[i][jb], nan_here);
+                put4(prow, col + kBN, acc[i][4 + jb], acc[i][4 + jb], nan_here);
+            }
+        }
+    });
+}
+
 // ---- few rows per expert (decode-time batches): the layer is bound by streaming every active
 // expert's weights once, which 128-row tiles with a handful of live rows do at half the memory
 // rate (and a single token, two active experts, at a fifth of it: its down-projection is 32
@@ -475,7 +703,14 @@ int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const voi
         return static_cast<unsigned>(groups * 8 * g.ngt * g.mt_total);
     };
     plan(g1);
-    hipLaunchKernelGGL((grouped_gemm_kernel<T, true, S>), dim3(grid_of(g1)), dim3(S::kThreads), 0, s, g1);
+    // 256-row tiles: the four-wave tile of 16 x 16 x 32 MFMAs (PARAS_GEMM_EIGHT_WAVES: the eight-wave tile of
+    // 32 x 32 x 16 ones, for measurements)
+    static const bool eight_waves = std::getenv("PARAS_GEMM_EIGHT_WAVES") != nullptr;
+    constexpr bool kBig = S::kBM == 256;
+    if (kBig && !eight_waves)
+        hipLaunchKernelGGL((grouped_gemm_quad16_kernel<T, true>), dim3(grid_of(g1)), dim3(quad16::kThreads), 0, s, g1);
+    else
+        hipLaunchKernelGGL((grouped_gemm_kernel<T, true, S>), dim3(grid_of(g1)), dim3(S::kThreads), 0, s, g1);
     PARAS_HIP_TRY(hipGetLastError());
 
     FfnGemmParams g2{};
@@ -489,7 +724,10 @@ int run_ffn_shape(const void* x, const void* w_gate, const void* w_up, const voi
     g2.mt_total = mt_total;
     g2.n_units = static_cast<int>((H + 2 * kBN - 1) / (2 * kBN));
     plan(g2);
-    hipLaunchKernelGGL((grouped_gemm_kernel<T, false, S>), dim3(grid_of(g2)), dim3(S::kThreads), 0, s, g2);
+    if (kBig && !eight_waves)
+        hipLaunchKernelGGL((grouped_gemm_quad16_kernel<T, false>), dim3(grid_of(g2)), dim3(quad16::kThreads), 0, s, g2);
+    else
+        hipLaunchKernelGGL((grouped_gemm_kernel<T, false, S>), dim3(grid_of(g2)), dim3(S::kThreads), 0, s, g2);
     PARAS_HIP_TRY(hipGetLastError());
 
     const long total = T_ * (H / 8);

@@ -103,6 +103,32 @@ __device__ __forceinline__ typename Elem<T>::store_t swiglu_from_acc(float a0, f
     return swiglu_one<T>(E::from_f32(a0), E::from_f32(a1));
 }
 
+// The common tier of four of them at once (V: a vector of four floats), without a branch in between, so
+// the exp / rcp chains overlap in a wave that has its SIMD to itself.  Returns whether all four passed
+// their bounds: o then holds the results; otherwise the caller sends the four through swiglu_from_acc.
+template <typename T, typename V>
+__device__ __forceinline__ bool swiglu4_common_tier(const V a0, const V a1, typename Elem<T>::store_t (&o)[4]) {
+    using E = Elem<T>;
+    static_assert(sizeof(typename E::store_t) == 2, "16-bit dtypes only");
+    bool ok = true;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const float g = E::to_f32(E::from_f32_finite(a0[r]));
+        const float u = E::to_f32(E::from_f32_finite(a1[r]));
+        const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);
+        const float y = g * __builtin_amdgcn_rcpf(1.0f + e) * u;
+        ok = ok & (narrow_is_safe<T>(y, kSwigluUlps) & (fabsf(g - 26.0f) <= 34.0f));
+        o[r] = E::from_f32_finite(y);
+    }
+    return ok;
+}
+template <typename T, typename V>
+__device__ __forceinline__ void swiglu4_from_acc(const V a0, const V a1, typename Elem<T>::store_t (&o)[4]) {
+    if (__builtin_expect(swiglu4_common_tier<T>(a0, a1, o), 1)) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = swiglu_from_acc<T>(a0[r], a1[r]);
+}
+
 // ---- SwiGLU backward -----------------------------------------------------------
 // Host definition (csrc/ops/fused_ops.cpp:218-226), in fp64:
 //   s = 1/(1+exp(-g));  dup = (dy*g)*s;  dgate = (dy*u) * (s * (1 + g*(1-s)))
