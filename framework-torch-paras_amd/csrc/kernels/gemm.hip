@@ -72,7 +72,8 @@ __device__ __forceinline__ bool tile_of_workgroup(const DenseParams& p, long wg,
     return block < p.xcd_blocks && mt < p.m_tiles && nu < p.n_units;
 }
 
-// S = Tile256 (8 waves, 256 x 256; for problems with at least 144 such tiles), Tile128 (4 waves,
+// S = Tile256 (8 waves, 256 x 256 on 32 x 32 x 16 MFMAs: launched only when PARAS_GEMM_EIGHT_WAVES is set,
+// the problems of at least 144 such tiles run on dense_gemm_nt_quad16_kernel below), Tile128 (4 waves,
 // 128 x 256) or Tile128x128 (4 waves, one column group; when there would be fewer than 512 tiles of 128 x 256).
 // kPartial: the contraction is split over p.splits workgroups per tile (the few-tile problems of 33 to
 // 128 rows: a projection at decode batch sizes has 32 to 112 tiles for 256 CUs); each writes its

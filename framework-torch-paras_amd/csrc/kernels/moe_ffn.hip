@@ -16,9 +16,11 @@
 //
 // Tiling (gemm_tile.h): a workgroup computes 128 or 256 routed rows x two
 // 128-column groups (gate and up columns n0..n0+127 for GEMM 1; columns
-// n0..n0+255 for GEMM 2), k-tile 64, waves arranged 2x2 or 4x2 with 64x64 per
-// column group each (128 fp32 accumulators per lane); 256 rows when the
-// experts hold enough rows for them.  Global -> registers -> LDS with the next
+// n0..n0+255 for GEMM 2), k-tile 64.  128 rows: waves arranged 2x2 with 64x64
+// per column group each (128 fp32 accumulators per lane).  256 rows, when the
+// experts hold enough rows for them: four waves with 128 x 128 each on
+// v_mfma_f32_16x16x32 (256 accumulators per lane; grouped_gemm_quad16_kernel).
+// Global -> registers -> LDS with the next
 // k-tile's loads in flight during the MFMAs.  Rows of one expert are contiguous
 // in the routed order; m-tiles never straddle experts (the grid is sized for the
 // worst case and surplus workgroups exit).  The block index is unscrambled so
