@@ -172,6 +172,41 @@ def test_gemm_nt_many_tiles_with_ragged_edges(dtype):
     assert torch.equal(capi.gemm_nt(a * 2, b)[big], (out * 2)[big])
 
 
+_EIGHT_WAVES_CHILD = r"""
+import hashlib, sys, torch
+sys.path.insert(0, sys.argv[1])
+import capi
+torch.manual_seed(33)
+a = torch.randn(4, 2100, 128).bfloat16().cuda()
+b = (0.1 * torch.randn(4, 2100, 128)).bfloat16().cuda()
+out = capi.gemm_nt(a, b)
+T, E, k, H, I = 4096, 2, 2, 1024, 512
+logits, x = torch.randn(T, E).bfloat16().cuda(), torch.randn(T, H).bfloat16().cuda()
+wg, wu = (0.03 * torch.randn(E, I, H)).bfloat16().cuda(), (0.03 * torch.randn(E, I, H)).bfloat16().cuda()
+wd = (0.03 * torch.randn(E, H, I)).bfloat16().cuda()
+topi, topw, order, inv, counts, offsets = capi.moe_route(logits, k)
+y = capi.moe_ffn(x, wg, wu, wd, topw, order, inv, offsets, k)
+for t in (out, y):
+    print(hashlib.sha256(t.cpu().view(torch.int16).numpy().tobytes()).hexdigest())
+"""
+
+
+def test_256_row_tiles_on_eight_waves_give_the_same_bits():
+    """PARAS_GEMM_EIGHT_WAVES=1 (read once per process, hence the child process) sends the 256-row tiles of the
+    dense product and of the expert FFN to the eight-wave kernels on 32 x 32 x 16 MFMAs.  They add the same
+    products in the same order as the four-wave kernels on 16 x 16 x 32: identical outputs, compared by digest."""
+    import os, subprocess, sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    def run(extra):
+        env = {k: v for k, v in os.environ.items() if k != "PARAS_GEMM_EIGHT_WAVES"}
+        env.update(extra)
+        r = subprocess.run([sys.executable, "-c", _EIGHT_WAVES_CHILD, here], env=env, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        return r.stdout.split()
+    four, eight = run({}), run({"PARAS_GEMM_EIGHT_WAVES": "1"})
+    assert len(four) == 2 and four == eight
+
+
 def test_gemm_nt_256_row_tiles_agree_with_128_row_tiles():
     """A batch of four problems is big enough for the 256-row tiles, each problem alone is not:
     both forms add the same products in the same order, so they agree bit for bit (ragged M and
