@@ -219,6 +219,35 @@ def test_ffn_256_row_tiles_with_most_gates_outside_the_common_range(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_ffn_256_row_tiles_with_nan_inf_and_zero_rows(dtype):
+    """A NaN, an infinity and an all-zero row among the tokens of a layer big enough for the 256-row tiles:
+    those tokens come out as the oracle has them (NaNs in the same places, exact zeros), and their
+    neighbours in the same tiles are untouched."""
+    torch.manual_seed(29)
+    T, H, E, k, I = 4096, 1024, 2, 2, 512
+    logits = torch.randn(T, E).to(dtype)
+    x = torch.randn(T, H).to(dtype)
+    x[5, 3] = float("nan")
+    x[700, 10] = float("inf")
+    x[1500] = 0
+    wg, wu = (0.03 * torch.randn(E, I, H)).to(dtype), (0.03 * torch.randn(E, I, H)).to(dtype)
+    wd = (0.03 * torch.randn(E, H, I)).to(dtype)
+    topi, topw, order, inv, counts, offsets = capi.moe_route(logits.cuda(), k)
+    out = capi.moe_ffn(x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), topw, order, inv, offsets, k).cpu()
+    sel = torch.tensor([4, 5, 6, 699, 700, 701, 1499, 1500, 1501] + torch.randperm(T)[:23].tolist())
+    r = O.moe_route(logits[sel], k)
+    ref = O.moe_ffn(x[sel], wg, wu, wd, r[1], r[2], r[3], r[5], k, gemm="aten")
+    got = out[sel]
+    assert torch.equal(got.isnan(), ref.isnan())
+    assert bool(ref[1].isnan().all()) and bool(ref[4].isnan().any())        # the NaN token, the infinite one
+    assert torch.equal(got[7], torch.zeros(H, dtype=dtype)) and torch.equal(ref[7], torch.zeros(H, dtype=dtype))
+    fin = ~ref.isnan().any(dim=1)
+    assert int(fin.sum()) >= 30
+    assert_ffn_close(got[fin], ref[fin], dtype)
+    assert int(out.isnan().any(dim=1).sum()) == 2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_ffn_rows_in_the_last_tile_of_every_expert(dtype):
     """256-row tiles and experts whose last tiles hold 1, 40, 64, 65, 200 and 256 rows (a tile of at
     most 64 rows is shared out among the waves differently): every token with a row in some
