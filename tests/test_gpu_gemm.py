@@ -207,6 +207,36 @@ def test_256_row_tiles_on_eight_waves_give_the_same_bits():
     assert len(four) == 2 and four == eight
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(4352, 4096, 256), (700, 512, 128), (64, 1024, 512), (8, 512, 256)])
+def test_gemm_nt_nan_and_infinity_go_where_ieee_sends_them(shape, dtype):
+    """A NaN in one row of A, an infinity in one row of B, on every tile form (256-row, 128-row, the
+    split contraction of few rows, the weight-streaming kernel): NaNs exactly where fp32 arithmetic
+    puts them (that row, that column; in bfloat16 with the host's NaN encoding), infinities with their signs,
+    everything else as without them."""
+    M, N, K = shape
+    torch.manual_seed(M)
+    a = torch.randn(M, K).to(dtype)
+    b = (0.1 * torch.randn(N, K)).to(dtype)
+    clean = capi.gemm_nt(a.cuda(), b.cuda()).cpu()
+    a[M // 3, 5] = float("nan")
+    b[N // 2, 7] = float("inf")
+    got = capi.gemm_nt(a.cuda(), b.cuda()).cpu()
+    ref = (a.float() @ b.float().T).to(dtype)
+    assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got.isinf(), ref.isinf())
+    assert bool(got[M // 3].isnan().all()) and bool(got[:, N // 2].isinf().sum() >= M - 2)
+    assert torch.equal(got[got.isinf()], ref[ref.isinf()])
+    if dtype == torch.bfloat16:
+        # one NaN encoding in bfloat16, the oracle's; float16 keeps the sign of the fp32 NaN, and which sign
+        # a NaN sum gets is the adder's choice (the matrix cores and a CPU differ), so only bf16 is held to bits
+        want_row = O.matmul_nt(a[M // 3: M // 3 + 1], b)
+        assert torch.equal(got[M // 3: M // 3 + 1].view(torch.int16), want_row.view(torch.int16))
+    keep = torch.ones(M, N, dtype=torch.bool)
+    keep[M // 3] = False
+    keep[:, N // 2] = False
+    assert torch.equal(got[keep], clean[keep])
+
+
 def test_gemm_nt_256_row_tiles_agree_with_128_row_tiles():
     """A batch of four problems is big enough for the 256-row tiles, each problem alone is not:
     both forms add the same products in the same order, so they agree bit for bit (ragged M and
