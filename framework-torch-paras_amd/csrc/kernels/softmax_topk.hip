@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 
 #include "core/device_context.h"
 #include "core/device_math.h"
@@ -116,6 +117,82 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(const typename
     for (int i = 0; i < EPT; ++i) {
         const int j = threadIdx.x + i * kBlock;
         if (j < n) outr[j] = EO::from_f64(v[i] / sum);
+    }
+}
+
+// 16-bit rows of 264 .. 4096 elements, a multiple of 8, 16-byte aligned, output in the input's dtype:
+// the same arithmetic as softmax_rows_reg_kernel in fewer instructions (that kernel spends two
+// thirds of its 113 per element on widening, narrowing and the tests of a ragged row).  A thread
+// takes NV pieces of eight elements with 16-byte loads and stores; the maximum is taken on the
+// floats (the widening is exact and v_max_f32 passes a NaN by, as the host's `v > m` does); the
+// difference to it, the exponential, the sum and the division are in fp64 as before; the quotients
+// are narrowed double -> float -> T by the conversion instructions when the sum is a positive
+// finite number (every quotient then lies in [0, 1]), and with the host's NaN rules otherwise.
+// BLK threads per row (64, 128 or 256: the fewest that cover the row, since every thread pays for its
+// eight exponentials whether the row reaches it or not).
+template <typename T, int NV, int BLK>
+__global__ __launch_bounds__(BLK) void softmax_rows_vec_kernel(const std::uint16_t* __restrict__ x, std::uint16_t* __restrict__ out, int n) {
+    using E = Elem<T>;
+    constexpr int kBlock = BLK, kWaves = BLK / kWave;
+    __shared__ float m_slots[kWaves];
+    __shared__ double s_slots[kWaves];
+    const std::uint16_t* xr = x + static_cast<long>(blockIdx.x) * n;
+    std::uint16_t* outr = out + static_cast<long>(blockIdx.x) * n;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int pieces = n >> 3;
+    float f[NV][8];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int pc = threadIdx.x + i * kBlock;
+        u32x4 w = {0xFF80FF80u, 0xFF80FF80u, 0xFF80FF80u, 0xFF80FF80u};       // (bf16 -inf twice; replaced below for f16)
+        if (sizeof(T) == 2 && !std::is_same<T, bf16_t>::value) w = u32x4{0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u};
+        if (pc < pieces) w = *reinterpret_cast<const u32x4*>(xr + 8 * pc);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            f[i][e] = E::to_f32(static_cast<std::uint16_t>(w[e >> 1] >> (16 * (e & 1))));
+            m = __builtin_fmaxf(m, f[i][e]);
+        }
+    }
+    m = wave_max(m);
+    if (lane == 0) m_slots[wave] = m;
+    __syncthreads();
+    m = m_slots[0];
+#pragma unroll
+    for (int i = 1; i < kWaves; ++i) m = __builtin_fmaxf(m, m_slots[i]);
+    const double md = static_cast<double>(m);
+    double ex[NV][8], sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            ex[i][e] = exp(static_cast<double>(f[i][e]) - md);       // (lanes past the row's end: exp(-inf - m) = 0, or a NaN when the sum is one anyway)
+            sum += ex[i][e];
+        }
+    sum = wave_sum(sum);
+    if (lane == 0) s_slots[wave] = sum;
+    __syncthreads();
+    sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) sum += s_slots[i];
+    const bool plain = sum > 0.0 && sum <= 1.0e300;        // wave-uniform (false for a NaN)
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int pc = threadIdx.x + i * kBlock;
+        std::uint16_t o[8];
+        if (plain) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = E::from_f32_finite(static_cast<float>(ex[i][e] / sum));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = E::from_f64(ex[i][e] / sum);
+        }
+        if (pc < pieces) {
+            u32x4 w;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) w[q] = o[2 * q] | (static_cast<std::uint32_t>(o[2 * q + 1]) << 16);
+            *reinterpret_cast<u32x4*>(outr + 8 * pc) = w;
+        }
     }
 }
 
@@ -540,6 +617,18 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
     if (n <= 16 * kBlock) {
         const bool widen = dtype_out == PARAS_F32 && sizeof(SI) == 2;
         const auto* xs = static_cast<const SI*>(x);
+        if constexpr (sizeof(SI) == 2) {
+            if (!widen && n % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+                const auto* x16 = static_cast<const std::uint16_t*>(x);
+                auto* o16 = static_cast<std::uint16_t*>(out);
+                if (n <= 512)       hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 1, 64>), g, dim3(64), 0, s, x16, o16, (int)n);
+                else if (n <= 1024) hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 1, 128>), g, dim3(128), 0, s, x16, o16, (int)n);
+                else if (n <= 2048) hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 1, 256>), g, b, 0, s, x16, o16, (int)n);
+                else                hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 2, 256>), g, b, 0, s, x16, o16, (int)n);
+                PARAS_HIP_TRY(hipGetLastError());
+                return PARAS_OK;
+            }
+        }
         if (n <= 4 * kBlock) {
             if (widen) hipLaunchKernelGGL((softmax_rows_reg_kernel<TI, float, 4>), g, b, 0, s, xs, static_cast<float*>(out), (int)n);
             else       hipLaunchKernelGGL((softmax_rows_reg_kernel<TI, TI, 4>), g, b, 0, s, xs, static_cast<SI*>(out), (int)n);

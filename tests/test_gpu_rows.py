@@ -68,6 +68,34 @@ def test_topk_reference_tie_literal_and_torch_parity():
         capi.topk_rows(y.cuda(), 300)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [264, 1024, 2048, 2056, 4096])
+def test_softmax_16_bit_rows_in_pieces_of_eight(dtype, n):
+    """Row lengths that are a multiple of eight (the kernel with 16-byte loads and stores), with the rows
+    the host treats specially among ordinary ones: a NaN in the row, a row of NaNs, +inf and -inf
+    in a row, a row of -inf, a constant row, a row with a spread of 200 (most weights underflow)."""
+    torch.manual_seed(n)
+    x = (3 * torch.randn(9, n)).to(dtype)
+    nan, inf = float("nan"), float("inf")
+    x[1, n // 2] = nan
+    x[2] = nan
+    x[3, 7], x[3, n - 1] = inf, -inf
+    x[4] = -inf
+    x[5] = 1.5
+    x[6] = (torch.linspace(-100, 100, n)).to(dtype)
+    x[7, 0] = -inf
+    got, want = capi.softmax_rows(x.cuda()).cpu(), O.softmax_last(x)
+    assert torch.equal(got.isnan(), want.isnan())
+    diff = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()[~want.isnan()]
+    assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) <= 1e-3
+    assert torch.equal(got.view(torch.int16)[want.isnan()], want.view(torch.int16)[want.isnan()])      # the host's NaN encoding
+    assert torch.equal(got[5], want[5]) and bool((got[7, 0] == 0).item())
+    # a view at an odd offset takes the element-wise kernel: same values
+    buf = torch.zeros(9 * n + 1, dtype=dtype, device="cuda")
+    buf[1:] = x.cuda().flatten()
+    assert torch.equal(capi.softmax_rows(buf[1:].view(9, n)).cpu().view(torch.int16), got.view(torch.int16))
+
+
 def test_short_rows_with_nan_and_infinities():
     """The one-wave-per-row kernels keep the host engine's conventions: a NaN never becomes the
     row maximum of a softmax; a top-k slot with no candidate reports index -1 and value 0."""
