@@ -125,6 +125,65 @@ __global__ __launch_bounds__(kBlock) void scale_mask_softmax_rows_kernel(const R
     }
 }
 
+// The same for rows of up to kBlock * EPT keys, with each thread's scores held in registers: the scaled,
+// masked and narrowed score is formed once instead of three times, there is one exponential per
+// score instead of two, and none at all for the keys a causal row cannot see (their weights are
+// 0 / sum, as exp(-inf - m) / sum is).  Same sums in the same order as the kernel above.
+template <typename T, int EPT>
+__global__ __launch_bounds__(kBlock) void scale_mask_softmax_rows_reg_kernel(const RowsParams p) {
+    using E = Elem<T>;
+    using S = typename E::store_t;
+    __shared__ double slots[kWaves];
+    for (long r = blockIdx.x; r < p.heads * p.rows; r += gridDim.x) {
+        const long hh = r / p.rows, ri = r % p.rows;
+        const long hg = p.h0 + hh, i = p.i0 + ri;
+        const long b = p.b + hg / p.Hq, h = hg % p.Hq;
+        S* row = static_cast<S*>(p.scores) + hh * p.head_stride + ri * p.Lk;
+        const long mrow = b * p.ms[0] + h * p.ms[1] + i * p.ms[2];
+        const long seen = p.is_causal ? (i + 1 < p.Lk ? i + 1 : p.Lk) : p.Lk;      // keys past it are masked
+        double v[EPT];
+        double m = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+            const long j = threadIdx.x + static_cast<long>(e) * kBlock;
+            double s = -INFINITY;
+            if (j < seen) {
+                s = E::to_f64(E::from_f64(E::to_f64(row[j]) * p.scale));
+                if (p.mask_kind == 1 && !p.is_causal) {
+                    if (static_cast<const unsigned char*>(p.mask)[mrow + j * p.ms[3]] == 0) s = -INFINITY;
+                } else if (p.mask_kind == 2 && !p.is_causal) {
+                    s = E::to_f64(E::from_f64(s + E::to_f64(static_cast<const S*>(p.mask)[mrow + j * p.ms[3]])));
+                }
+            }
+            v[e] = s;
+            m = fmax(m, s);
+        }
+        m = block_reduce(m, slots, true);
+        double sum = 0.0;
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+            const long j = threadIdx.x + static_cast<long>(e) * kBlock;
+            v[e] = j < seen ? exp(v[e] - m) : 0.0;
+            sum += v[e];
+        }
+        sum = block_reduce(sum, slots, false);
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+            const long j = threadIdx.x + static_cast<long>(e) * kBlock;
+            if (j < p.Lk) row[j] = E::from_f64(v[e] / sum);
+        }
+        if (p.lse && threadIdx.x == 0) p.lse[(b * p.Hq + h) * p.Lq + i] = static_cast<float>(m + log(sum));
+        __syncthreads();     // slots are reused by the next row
+    }
+}
+
+template <typename T>
+void launch_rows(const RowsParams& rp, unsigned grid, hipStream_t s) {
+    if (rp.Lk <= 4 * kBlock)       hipLaunchKernelGGL((scale_mask_softmax_rows_reg_kernel<T, 4>), dim3(grid), dim3(kBlock), 0, s, rp);
+    else if (rp.Lk <= 16 * kBlock) hipLaunchKernelGGL((scale_mask_softmax_rows_reg_kernel<T, 16>), dim3(grid), dim3(kBlock), 0, s, rp);
+    else                           hipLaunchKernelGGL((scale_mask_softmax_rows_kernel<T>), dim3(grid), dim3(kBlock), 0, s, rp);
+}
+
 struct Plan {
     long heads;        // q heads per piece (a multiple of rep, or rep itself)
     long rows;         // query rows per piece
@@ -234,10 +293,10 @@ int launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hip
                 const long nrows = nh * nr;
                 const unsigned grid = static_cast<unsigned>(nrows < 256L * 64 ? nrows : 256L * 64);
                 switch (a.dtype) {
-                    case PARAS_F32:  hipLaunchKernelGGL((scale_mask_softmax_rows_kernel<float>), dim3(grid), dim3(kBlock), 0, s, rp); break;
-                    case PARAS_F64:  hipLaunchKernelGGL((scale_mask_softmax_rows_kernel<double>), dim3(grid), dim3(kBlock), 0, s, rp); break;
-                    case PARAS_BF16: hipLaunchKernelGGL((scale_mask_softmax_rows_kernel<bf16_t>), dim3(grid), dim3(kBlock), 0, s, rp); break;
-                    default:         hipLaunchKernelGGL((scale_mask_softmax_rows_kernel<f16_t>), dim3(grid), dim3(kBlock), 0, s, rp); break;
+                    case PARAS_F32:  launch_rows<float>(rp, grid, s); break;
+                    case PARAS_F64:  launch_rows<double>(rp, grid, s); break;
+                    case PARAS_BF16: launch_rows<bf16_t>(rp, grid, s); break;
+                    default:         launch_rows<f16_t>(rp, grid, s); break;
                 }
                 PARAS_HIP_TRY(hipGetLastError());
 
