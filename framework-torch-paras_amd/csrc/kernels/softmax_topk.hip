@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(const typename
     }
 }
 
-// 16-bit rows of 264 .. 4096 elements, a multiple of 8, 16-byte aligned, output in the input's dtype:
+// 16-bit rows of 264 .. 32768 elements, a multiple of 8, 16-byte aligned, output in the input's dtype:
 // the same arithmetic as softmax_rows_reg_kernel in fewer instructions (that kernel spends two
 // thirds of its 113 per element on widening, narrowing and the tests of a ragged row).  A thread
 // takes NV pieces of eight elements with 16-byte loads and stores; the maximum is taken on the
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(const typename
 // difference to it, the exponential, the sum and the division are in fp64 as before; the quotients
 // are narrowed double -> float -> T by the conversion instructions when the sum is a positive
 // finite number (every quotient then lies in [0, 1]), and with the host's NaN rules otherwise.
-// BLK threads per row (64, 128 or 256: the fewest that cover the row, since every thread pays for its
+// BLK threads per row (64, 128, 256 or 1024: the fewest that cover the row with at most four pieces each, since every thread pays for its
 // eight exponentials whether the row reaches it or not).
 template <typename T, int NV, int BLK>
 __global__ __launch_bounds__(BLK) void softmax_rows_vec_kernel(const std::uint16_t* __restrict__ x, std::uint16_t* __restrict__ out, int n) {
@@ -638,6 +638,18 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
         }
         PARAS_HIP_TRY(hipGetLastError());
         return PARAS_OK;
+    }
+    if constexpr (sizeof(SI) == 2) {
+        // up to 32768 elements the exponentials of a 16-bit row still fit the registers of a workgroup (one
+        // exponential per element instead of two, one read of the row instead of three)
+        if (dtype_out != PARAS_F32 && n <= 32 * 1024 && n % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+            const auto* x16 = static_cast<const std::uint16_t*>(x);
+            auto* o16 = static_cast<std::uint16_t*>(out);
+            if (n <= 8 * 1024) hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 4, 256>), g, b, 0, s, x16, o16, (int)n);
+            else               hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 4, 1024>), g, dim3(1024), 0, s, x16, o16, (int)n);
+            PARAS_HIP_TRY(hipGetLastError());
+            return PARAS_OK;
+        }
     }
     const bool widen_long = dtype_out == PARAS_F32 && sizeof(SI) == 2;
     if (rows <= 2048) {           // few long rows: a CU's worth of wavefronts per row

@@ -69,7 +69,7 @@ def test_topk_reference_tie_literal_and_torch_parity():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("n", [264, 1024, 2048, 2056, 4096])
+@pytest.mark.parametrize("n", [264, 1024, 2048, 2056, 4096, 4104, 8192, 8200, 32768])
 def test_softmax_16_bit_rows_in_pieces_of_eight(dtype, n):
     """Row lengths that are a multiple of eight (the kernel with 16-byte loads and stores), with the rows
     the host treats specially among ordinary ones: a NaN in the row, a row of NaNs, +inf and -inf
