@@ -120,37 +120,47 @@ __global__ __launch_bounds__(kBlock) void softmax_rows_reg_kernel(const typename
     }
 }
 
-// 16-bit rows of 264 .. 32768 elements, a multiple of 8, 16-byte aligned, output in the input's dtype:
-// the same arithmetic as softmax_rows_reg_kernel in fewer instructions (that kernel spends two
-// thirds of its 113 per element on widening, narrowing and the tests of a ragged row).  A thread
-// takes NV pieces of eight elements with 16-byte loads and stores; the maximum is taken on the
-// floats (the widening is exact and v_max_f32 passes a NaN by, as the host's `v > m` does); the
-// difference to it, the exponential, the sum and the division are in fp64 as before; the quotients
-// are narrowed double -> float -> T by the conversion instructions when the sum is a positive
-// finite number (every quotient then lies in [0, 1]), and with the host's NaN rules otherwise.
-// BLK threads per row (64, 128, 256 or 1024: the fewest that cover the row with at most four pieces each, since every thread pays for its
-// eight exponentials whether the row reaches it or not).
+// 16-bit and fp32 rows of up to 32768 elements in whole 16-byte pieces, 16-byte aligned, output in the
+// input's dtype: the same arithmetic as softmax_rows_reg_kernel in fewer instructions (that kernel
+// spends two thirds of its 113 per element on widening, narrowing and the tests of a ragged row).
+// A thread takes NV pieces (eight 16-bit elements or four floats) with 16-byte loads and stores; the
+// maximum is taken on floats (the widening is exact and v_max_f32 passes a NaN by, as the host's
+// `v > m` does); the difference to it, the exponential, the sum and the division are in fp64 as
+// before; 16-bit quotients are narrowed double -> float -> T by the conversion instructions when
+// the sum is a positive finite number (every quotient then lies in [0, 1]), and with the host's NaN
+// rules otherwise.  BLK threads per row (64, 128, 256 or 1024: the fewest that cover the row with
+// at most 32 elements each, since every thread pays for its exponentials whether the row reaches
+// it or not).
 template <typename T, int NV, int BLK>
-__global__ __launch_bounds__(BLK) void softmax_rows_vec_kernel(const std::uint16_t* __restrict__ x, std::uint16_t* __restrict__ out, int n) {
+__global__ __launch_bounds__(BLK) void softmax_rows_vec_kernel(const typename Elem<T>::store_t* __restrict__ x,
+                                                               typename Elem<T>::store_t* __restrict__ out, int n) {
     using E = Elem<T>;
+    using S = typename E::store_t;
     constexpr int kBlock = BLK, kWaves = BLK / kWave;
+    constexpr int EPV = 16 / static_cast<int>(sizeof(S));          // elements per piece
+    static_assert(EPV == 8 || EPV == 4, "16-bit or 32-bit elements");
     __shared__ float m_slots[kWaves];
     __shared__ double s_slots[kWaves];
-    const std::uint16_t* xr = x + static_cast<long>(blockIdx.x) * n;
-    std::uint16_t* outr = out + static_cast<long>(blockIdx.x) * n;
+    const S* xr = x + static_cast<long>(blockIdx.x) * n;
+    S* outr = out + static_cast<long>(blockIdx.x) * n;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int pieces = n >> 3;
-    float f[NV][8];
+    const int pieces = n / EPV;
+    // minus infinity in every element, for the lanes past the row's end
+    constexpr std::uint32_t kFill = EPV == 4 ? 0xFF800000u : (std::is_same<T, bf16_t>::value ? 0xFF80FF80u : 0xFC00FC00u);
+    float f[NV][EPV];
     float m = -INFINITY;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int pc = threadIdx.x + i * kBlock;
-        u32x4 w = {0xFF80FF80u, 0xFF80FF80u, 0xFF80FF80u, 0xFF80FF80u};       // (bf16 -inf twice; replaced below for f16)
-        if (sizeof(T) == 2 && !std::is_same<T, bf16_t>::value) w = u32x4{0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u, 0xFC00FC00u};
-        if (pc < pieces) w = *reinterpret_cast<const u32x4*>(xr + 8 * pc);
+        u32x4 w = {kFill, kFill, kFill, kFill};
+        if (pc < pieces) w = *reinterpret_cast<const u32x4*>(xr + EPV * pc);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            f[i][e] = E::to_f32(static_cast<std::uint16_t>(w[e >> 1] >> (16 * (e & 1))));
+        for (int e = 0; e < EPV; ++e) {
+            if constexpr (EPV == 4) {
+                const std::uint32_t bits = w[e];
+                f[i][e] = __builtin_bit_cast(float, bits);
+            }
+            else                    f[i][e] = E::to_f32(static_cast<S>(w[e >> 1] >> (16 * (e & 1))));
             m = __builtin_fmaxf(m, f[i][e]);
         }
     }
@@ -161,11 +171,11 @@ __global__ __launch_bounds__(BLK) void softmax_rows_vec_kernel(const std::uint16
 #pragma unroll
     for (int i = 1; i < kWaves; ++i) m = __builtin_fmaxf(m, m_slots[i]);
     const double md = static_cast<double>(m);
-    double ex[NV][8], sum = 0.0;
+    double ex[NV][EPV], sum = 0.0;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < EPV; ++e) {
             ex[i][e] = exp(static_cast<double>(f[i][e]) - md);       // (lanes past the row's end: exp(-inf - m) = 0, or a NaN when the sum is one anyway)
             sum += ex[i][e];
         }
@@ -179,21 +189,48 @@ __global__ __launch_bounds__(BLK) void softmax_rows_vec_kernel(const std::uint16
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int pc = threadIdx.x + i * kBlock;
-        std::uint16_t o[8];
-        if (plain) {
+        u32x4 w;
+        if constexpr (EPV == 4) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = E::from_f32_finite(static_cast<float>(ex[i][e] / sum));
+            for (int e = 0; e < 4; ++e) {
+                const float q = static_cast<float>(ex[i][e] / sum);
+                w[e] = __builtin_bit_cast(std::uint32_t, q);
+            }
         } else {
+            std::uint16_t o[8];
+            if (plain) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = E::from_f64(ex[i][e] / sum);
-        }
-        if (pc < pieces) {
-            u32x4 w;
+                for (int e = 0; e < 8; ++e) o[e] = E::from_f32_finite(static_cast<float>(ex[i][e] / sum));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = E::from_f64(ex[i][e] / sum);
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q) w[q] = o[2 * q] | (static_cast<std::uint32_t>(o[2 * q + 1]) << 16);
-            *reinterpret_cast<u32x4*>(outr + 8 * pc) = w;
         }
+        if (pc < pieces) *reinterpret_cast<u32x4*>(outr + EPV * pc) = w;
     }
+}
+
+// Rows in whole 16-byte pieces at 16-byte aligned addresses, up to 32768 elements, same dtype out: the kernel above.
+template <typename T>
+bool launch_softmax_vec(const void* x, void* out, long rows, long n, hipStream_t s) {
+    using S = typename Elem<T>::store_t;
+    constexpr long EPV = 16 / sizeof(S);
+    if (n % EPV != 0 || n > 32 * 1024 || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) != 0) return false;
+    const dim3 g(static_cast<unsigned>(rows));
+    const auto* xs = static_cast<const S*>(x);
+    auto* os = static_cast<S*>(out);
+    const long pieces = n / EPV;
+    constexpr int kMost = 32 / EPV;        // pieces per thread at most: 32 exponentials in registers
+    if (pieces <= 64)        hipLaunchKernelGGL((softmax_rows_vec_kernel<T, 1, 64>), g, dim3(64), 0, s, xs, os, (int)n);
+    else if (pieces <= 128)  hipLaunchKernelGGL((softmax_rows_vec_kernel<T, 1, 128>), g, dim3(128), 0, s, xs, os, (int)n);
+    else if (pieces <= 256)  hipLaunchKernelGGL((softmax_rows_vec_kernel<T, 1, 256>), g, dim3(256), 0, s, xs, os, (int)n);
+    else if (pieces <= 512)  hipLaunchKernelGGL((softmax_rows_vec_kernel<T, 2, 256>), g, dim3(256), 0, s, xs, os, (int)n);
+    else if (pieces <= 1024) hipLaunchKernelGGL((softmax_rows_vec_kernel<T, 4, 256>), g, dim3(256), 0, s, xs, os, (int)n);
+    else if (pieces <= 256 * kMost)  hipLaunchKernelGGL((softmax_rows_vec_kernel<T, kMost, 256>), g, dim3(256), 0, s, xs, os, (int)n);
+    else                     hipLaunchKernelGGL((softmax_rows_vec_kernel<T, kMost, 1024>), g, dim3(1024), 0, s, xs, os, (int)n);
+    return true;
 }
 
 // (value, index) order of the reference: larger value first (smaller when !largest), then lower index.
@@ -617,14 +654,8 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
     if (n <= 16 * kBlock) {
         const bool widen = dtype_out == PARAS_F32 && sizeof(SI) == 2;
         const auto* xs = static_cast<const SI*>(x);
-        if constexpr (sizeof(SI) == 2) {
-            if (!widen && n % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
-                const auto* x16 = static_cast<const std::uint16_t*>(x);
-                auto* o16 = static_cast<std::uint16_t*>(out);
-                if (n <= 512)       hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 1, 64>), g, dim3(64), 0, s, x16, o16, (int)n);
-                else if (n <= 1024) hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 1, 128>), g, dim3(128), 0, s, x16, o16, (int)n);
-                else if (n <= 2048) hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 1, 256>), g, b, 0, s, x16, o16, (int)n);
-                else                hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 2, 256>), g, b, 0, s, x16, o16, (int)n);
+        if constexpr (sizeof(SI) == 2 || sizeof(SI) == 4) {
+            if (!widen && launch_softmax_vec<TI>(x, out, rows, n, s)) {
                 PARAS_HIP_TRY(hipGetLastError());
                 return PARAS_OK;
             }
@@ -639,14 +670,10 @@ int launch_softmax(const void* x, void* out, long rows, long n, int dtype_out, h
         PARAS_HIP_TRY(hipGetLastError());
         return PARAS_OK;
     }
-    if constexpr (sizeof(SI) == 2) {
-        // up to 32768 elements the exponentials of a 16-bit row still fit the registers of a workgroup (one
+    if constexpr (sizeof(SI) == 2 || sizeof(SI) == 4) {
+        // up to 32768 elements the exponentials of a row still fit the registers of a workgroup (one
         // exponential per element instead of two, one read of the row instead of three)
-        if (dtype_out != PARAS_F32 && n <= 32 * 1024 && n % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
-            const auto* x16 = static_cast<const std::uint16_t*>(x);
-            auto* o16 = static_cast<std::uint16_t*>(out);
-            if (n <= 8 * 1024) hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 4, 256>), g, b, 0, s, x16, o16, (int)n);
-            else               hipLaunchKernelGGL((softmax_rows_vec_kernel<TI, 4, 1024>), g, dim3(1024), 0, s, x16, o16, (int)n);
+        if (!(dtype_out == PARAS_F32 && sizeof(SI) == 2) && launch_softmax_vec<TI>(x, out, rows, n, s)) {
             PARAS_HIP_TRY(hipGetLastError());
             return PARAS_OK;
         }

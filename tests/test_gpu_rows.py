@@ -68,9 +68,9 @@ def test_topk_reference_tie_literal_and_torch_parity():
         capi.topk_rows(y.cuda(), 300)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("n", [264, 1024, 2048, 2056, 4096, 4104, 8192, 8200, 32768])
-def test_softmax_16_bit_rows_in_pieces_of_eight(dtype, n):
+def test_softmax_rows_in_whole_16_byte_pieces(dtype, n):
     """Row lengths that are a multiple of eight (the kernel with 16-byte loads and stores), with the rows
     the host treats specially among ordinary ones: a NaN in the row, a row of NaNs, +inf and -inf
     in a row, a row of -inf, a constant row, a row with a spread of 200 (most weights underflow)."""
@@ -86,14 +86,23 @@ def test_softmax_16_bit_rows_in_pieces_of_eight(dtype, n):
     x[7, 0] = -inf
     got, want = capi.softmax_rows(x.cuda()).cpu(), O.softmax_last(x)
     assert torch.equal(got.isnan(), want.isnan())
-    diff = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()[~want.isnan()]
-    assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) <= 1e-3
-    assert torch.equal(got.view(torch.int16)[want.isnan()], want.view(torch.int16)[want.isnan()])      # the host's NaN encoding
+    bits = torch.int32 if dtype == torch.float32 else torch.int16
+    if dtype == torch.float32:
+        assert torch.allclose(got, want, rtol=1e-6, atol=0, equal_nan=True)
+    else:
+        diff = (got.view(bits).int() - want.view(bits).int()).abs()[~want.isnan()]
+        assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) <= 1e-3
+        assert torch.equal(got.view(bits)[want.isnan()], want.view(bits)[want.isnan()])      # the host's NaN encoding
     assert torch.equal(got[5], want[5]) and bool((got[7, 0] == 0).item())
     # a view at an odd offset takes the element-wise kernel: same values
     buf = torch.zeros(9 * n + 1, dtype=dtype, device="cuda")
     buf[1:] = x.cuda().flatten()
-    assert torch.equal(capi.softmax_rows(buf[1:].view(9, n)).cpu().view(torch.int16), got.view(torch.int16))
+    other = capi.softmax_rows(buf[1:].view(9, n)).cpu()
+    if dtype == torch.float32:
+        assert torch.allclose(other, got, rtol=1e-6, atol=0, equal_nan=True)       # (another order of the row's sum)
+    else:
+        odiff = (other.view(bits).int() - got.view(bits).int()).abs()[~want.isnan()]
+        assert int(odiff.max()) <= 1 and float((odiff > 0).float().mean()) <= 1e-3
 
 
 def test_short_rows_with_nan_and_infinities():
