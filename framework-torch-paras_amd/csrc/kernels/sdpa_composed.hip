@@ -13,6 +13,7 @@
 // ops do, so results differ from the general kernel (which sums the products
 // in fp64) only through the products' summation order.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 
 #include <algorithm>
 #include <cmath>
@@ -177,8 +178,106 @@ __global__ __launch_bounds__(kBlock) void scale_mask_softmax_rows_reg_kernel(con
     }
 }
 
+// fp32 score rows without a mask tensor (causal or not), a multiple of four keys long and 16-byte aligned:
+// the same arithmetic with 16-byte loads and stores, four scores a piece and NV pieces a thread, BLK threads
+// a row (the fewest that cover it).  The maximum is taken on the scaled floats (v_max_f32 passes a NaN
+// by, as fmax does), the pieces a causal row cannot see cost no exponential, and nothing is tested
+// per element but the diagonal.
+template <int NV, int BLK>
+__global__ __launch_bounds__(BLK) void scale_softmax_rows_f32_vec_kernel(const RowsParams p) {
+    constexpr int kNW = BLK / kWave;
+    __shared__ float m_slots[kNW];
+    __shared__ double s_slots[kNW];
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int pieces = static_cast<int>(p.Lk >> 2);
+    for (long r = blockIdx.x; r < p.heads * p.rows; r += gridDim.x) {
+        const long hh = r / p.rows, ri = r % p.rows;
+        const long hg = p.h0 + hh, i = p.i0 + ri;
+        const long b = p.b + hg / p.Hq, h = hg % p.Hq;
+        float* row = static_cast<float*>(p.scores) + hh * p.head_stride + ri * p.Lk;
+        const long seen = p.is_causal ? (i + 1 < p.Lk ? i + 1 : p.Lk) : p.Lk;      // keys past it are masked
+        float f[NV][4];
+        float m = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int pc = threadIdx.x + v * BLK;
+            const long j0 = 4L * pc;
+            u32x4 w = {0u, 0u, 0u, 0u};
+            if (pc < pieces && j0 < seen) w = *reinterpret_cast<const u32x4*>(row + j0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const std::uint32_t bits = w[e];
+                const float sc = static_cast<float>(static_cast<double>(__builtin_bit_cast(float, bits)) * p.scale);
+                f[v][e] = j0 + e < seen ? sc : -INFINITY;
+                m = __builtin_fmaxf(m, f[v][e]);
+            }
+        }
+        m = wave_max(m);
+        __syncthreads();                 // (the slots of the row before have been read)
+        if (lane == 0) m_slots[wave] = m;
+        __syncthreads();
+        m = m_slots[0];
+#pragma unroll
+        for (int k = 1; k < kNW; ++k) m = __builtin_fmaxf(m, m_slots[k]);
+        const double md = static_cast<double>(m);
+        double ex[NV][4], sum = 0.0;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const long j0 = 4L * (threadIdx.x + v * BLK);
+            if (j0 < seen) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ex[v][e] = j0 + e < seen ? exp(static_cast<double>(f[v][e]) - md) : 0.0;
+                    sum += ex[v][e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ex[v][e] = 0.0;
+            }
+        }
+        sum = wave_sum(sum);
+        if (lane == 0) s_slots[wave] = sum;
+        __syncthreads();
+        sum = 0.0;
+#pragma unroll
+        for (int k = 0; k < kNW; ++k) sum += s_slots[k];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int pc = threadIdx.x + v * BLK;
+            if (pc < pieces) {
+                u32x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float q = static_cast<float>(ex[v][e] / sum);
+                    w[e] = __builtin_bit_cast(std::uint32_t, q);
+                }
+                *reinterpret_cast<u32x4*>(row + 4L * pc) = w;
+            }
+        }
+        if (p.lse && threadIdx.x == 0) p.lse[(b * p.Hq + h) * p.Lq + i] = static_cast<float>(md + log(sum));
+    }
+}
+
+bool launch_rows_f32_vec(const RowsParams& rp, unsigned grid, hipStream_t s) {
+    if (rp.mask_kind != 0 && !rp.is_causal) return false;
+    if (rp.Lk % 4 != 0 || rp.Lk > 32 * 1024 || rp.head_stride % 4 != 0 || (reinterpret_cast<uintptr_t>(rp.scores) & 15) != 0) return false;
+    const long pieces = rp.Lk / 4;
+    const dim3 g(grid);
+    if (pieces <= 64)        hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<1, 64>), g, dim3(64), 0, s, rp);
+    else if (pieces <= 128)  hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<1, 128>), g, dim3(128), 0, s, rp);
+    else if (pieces <= 256)  hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<1, 256>), g, dim3(256), 0, s, rp);
+    else if (pieces <= 512)  hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<2, 256>), g, dim3(256), 0, s, rp);
+    else if (pieces <= 1024) hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<4, 256>), g, dim3(256), 0, s, rp);
+    else if (pieces <= 2048) hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<8, 256>), g, dim3(256), 0, s, rp);
+    else                     hipLaunchKernelGGL((scale_softmax_rows_f32_vec_kernel<8, 1024>), g, dim3(1024), 0, s, rp);
+    return true;
+}
+
 template <typename T>
 void launch_rows(const RowsParams& rp, unsigned grid, hipStream_t s) {
+    if constexpr (std::is_same<T, float>::value) {
+        if (launch_rows_f32_vec(rp, grid, s)) return;
+    }
     if (rp.Lk <= 4 * kBlock)       hipLaunchKernelGGL((scale_mask_softmax_rows_reg_kernel<T, 4>), dim3(grid), dim3(kBlock), 0, s, rp);
     else if (rp.Lk <= 16 * kBlock) hipLaunchKernelGGL((scale_mask_softmax_rows_reg_kernel<T, 16>), dim3(grid), dim3(kBlock), 0, s, rp);
     else                           hipLaunchKernelGGL((scale_mask_softmax_rows_kernel<T>), dim3(grid), dim3(kBlock), 0, s, rp);
