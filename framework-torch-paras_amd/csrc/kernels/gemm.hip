@@ -43,6 +43,10 @@ struct DenseParams {
     int  swapped;               // few-row kernels only: a and b have changed places (few output COLUMNS, many rows), so a
                                 // result (row of a, row of b) belongs at c[row of b][row of a], and the addend likewise
     int  xcd_blocks, xcd_blocks_n;   // XCD-blocked tile order: blocks of kXcdBlockM x kXcdBlockN tiles per batch (0: plain order), blocks along n
+    int  causal_kind;           // fp32 MFMA kernel, for causal attention: 1 = the product is a score matrix of which row r only needs
+                                // columns <= r + causal_first (tiles wholly beyond are left unwritten); 2 = a is such a matrix after
+                                // its softmax (zeros beyond), so row tile r0 contracts over k < r0 + 128 + causal_first only; 0 = neither
+    long causal_first;          // index of row 0 among the queries
 };
 
 // Workgroup w runs on XCD w % 8, each with an L2 of its own.  In the plain order (column units
@@ -729,6 +733,12 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_f32_mfma_kernel(const float* _
     const float* A = a + bidx * p.sa;
     const float* B = b + bidx * p.sb;
     const long row0 = static_cast<long>(blockIdx.y) * kF32BM, col0 = static_cast<long>(blockIdx.x) * kF32BN;
+    if (p.causal_kind == 1 && col0 > row0 + (kF32BM - 1) + p.causal_first) return;      // no query of this tile sees any of its keys
+    long K = p.K;           // (the contraction as far as this tile needs it)
+    if (p.causal_kind == 2) {
+        const long upto = (row0 + kF32BM + p.causal_first + kF32BK - 1) / kF32BK * kF32BK;
+        if (upto < K) K = upto;
+    }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lr = lane & 31, lh = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
@@ -743,12 +753,12 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_f32_mfma_kernel(const float* _
             float4_t v = {0.f, 0.f, 0.f, 0.f};
             if (row < limit) {
                 const float* src = base + row * ld + k;
-                if (kVec && k + 3 < p.K) {
+                if (kVec && k + 3 < K) {
                     v = *reinterpret_cast<const float4_t*>(src);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (k + e < p.K) v[e] = src[e];
+                        if (k + e < K) v[e] = src[e];
                 }
             }
             st[i] = v;
@@ -770,7 +780,7 @@ __global__ __launch_bounds__(256, 2) void gemm_nt_f32_mfma_kernel(const float* _
         for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-    const long k_tiles = (p.K + kF32BK - 1) / kF32BK;
+    const long k_tiles = (K + kF32BK - 1) / kF32BK;
     fetch(A, p.lda, p.M, row0, 0, a_st);
     fetch(B, p.ldb, p.N, col0, 0, b_st);
     stash(as[0], a_st);
@@ -840,6 +850,14 @@ void launch_dense(const DenseParams& p, unsigned grid, hipStream_t s) {
 }  // namespace
 }  // namespace paras
 
+namespace paras {
+// paras_gemm_nt_ws with the two hints for causal attention (DenseParams::causal_kind, ::causal_first); also declared in sdpa_internal.h
+int gemm_nt_causal(const void* a, const void* b, const void* addend, void* c, int64_t M, int64_t N, int64_t K,
+                   int64_t lda, int64_t ldb, int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
+                   int64_t stride_b, int64_t stride_c, int64_t stride_add, double alpha, double beta, int dtype,
+                   void* workspace, size_t workspace_bytes, void* stream, int causal_kind, long causal_first);
+}  // namespace paras
+
 extern "C" {
 
 size_t paras_gemm_nt_workspace(int64_t M, int64_t N, int64_t K, int64_t batch, int dtype) {
@@ -865,6 +883,17 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
                      int64_t lda, int64_t ldb, int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
                      int64_t stride_b, int64_t stride_c, int64_t stride_add, double alpha, double beta, int dtype,
                      void* workspace, size_t workspace_bytes, void* stream) {
+    return paras::gemm_nt_causal(a, b, addend, c, M, N, K, lda, ldb, ldc, ld_add, batch, stride_a, stride_b, stride_c, stride_add, alpha, beta,
+                                 dtype, workspace, workspace_bytes, stream, 0, 0);
+}
+
+}  // extern "C"
+
+// paras_gemm_nt_ws, and for the attention route that multiplies causal score matrices (DenseParams::causal_kind)
+int paras::gemm_nt_causal(const void* a, const void* b, const void* addend, void* c, int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
+                          int64_t stride_b, int64_t stride_c, int64_t stride_add, double alpha, double beta, int dtype,
+                          void* workspace, size_t workspace_bytes, void* stream, int causal_kind, long causal_first) {
     using namespace paras;
     PARAS_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "paras_gemm_nt: negative shape");
     if (M == 0 || N == 0 || batch == 0) return PARAS_OK;
@@ -886,6 +915,7 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
     p.sa = stride_a; p.sb = stride_b; p.sc = stride_c; p.sadd = stride_add;
     p.alpha = static_cast<float>(alpha); p.beta = static_cast<float>(beta);
     p.alpha64 = alpha; p.beta64 = beta;
+    p.causal_kind = causal_kind; p.causal_first = causal_first;
     // What the MFMA kernels take: 16-bit floats, K a positive multiple of 64, 16-byte aligned operand
     // rows, operands of fewer than 2^32 elements.  Everything else runs on the general kernel.
     const bool mfma_ok = (dtype == PARAS_BF16 || dtype == PARAS_F16) && K > 0 && K % gemm::kBK == 0 &&
@@ -1021,5 +1051,3 @@ int paras_gemm_nt_ws(const void* a, const void* b, const void* addend, void* c, 
     PARAS_HIP_TRY(hipGetLastError());
     return PARAS_OK;
 }
-
-}  // extern "C"

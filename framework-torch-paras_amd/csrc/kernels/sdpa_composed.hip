@@ -379,8 +379,10 @@ int launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hip
                 const char* kp = static_cast<const char*>(a.k) + (b * a.k_strides[0] + hkv0 * a.k_strides[1]) * es;
                 // q heads of one kv head share its keys (stride 0); with one q head per kv head the heads step together
                 const long k_step = rep == 1 ? a.k_strides[1] : 0;
-                int rc = paras_gemm_nt(qp, kp, nullptr, sc, nr, a.Lk, a.D, a.q_strides[2], a.k_strides[2], a.Lk, 0, nh, a.q_strides[1],
-                                       k_step, head_stride, 0, 1.0, 0.0, a.dtype, stream);
+                // (causal: the score tiles wholly past the diagonal are neither formed nor, below, multiplied -- the row
+                // kernels read a row only as far as its query sees and write all of it)
+                int rc = gemm_nt_causal(qp, kp, nullptr, sc, nr, a.Lk, a.D, a.q_strides[2], a.k_strides[2], a.Lk, 0, nh, a.q_strides[1],
+                                        k_step, head_stride, 0, 1.0, 0.0, a.dtype, nullptr, 0, stream, a.is_causal ? 1 : 0, i0);
                 if (rc != PARAS_OK) return rc;
 
                 RowsParams rp{};
@@ -401,8 +403,8 @@ int launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hip
 
                 const char* vp = vt + ((b * a.Hkv + hkv0) * a.Dv * a.Lk) * es;
                 char* op = static_cast<char*>(a.out) + (((b * a.Hq + h0) * a.Lq + i0) * a.Dv) * es;
-                rc = paras_gemm_nt(sc, vp, nullptr, op, nr, a.Dv, a.Lk, a.Lk, a.Lk, a.Dv, 0, nh, head_stride,
-                                   rep == 1 ? a.Dv * a.Lk : 0, a.Lq * a.Dv, 0, 1.0, 0.0, a.dtype, stream);
+                rc = gemm_nt_causal(sc, vp, nullptr, op, nr, a.Dv, a.Lk, a.Lk, a.Lk, a.Dv, 0, nh, head_stride,
+                                    rep == 1 ? a.Dv * a.Lk : 0, a.Lq * a.Dv, 0, 1.0, 0.0, a.dtype, nullptr, 0, stream, a.is_causal ? 2 : 0, i0);
                 if (rc != PARAS_OK) return rc;
             }
         }

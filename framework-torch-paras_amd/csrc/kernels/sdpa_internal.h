@@ -34,6 +34,15 @@ bool   composed_supported(const paras_sdpa_args& a);
 size_t composed_workspace(const paras_sdpa_args& a);
 int    launch_composed(const paras_sdpa_args& a, void* workspace, void* stream, hipStream_t s);
 
+// paras_gemm_nt_ws (gemm.hip) with two hints for causal attention, which the fp32 matrix-core kernel
+// uses and the others ignore: causal_kind 1 = the product is a score matrix of which row r only needs
+// columns <= r + causal_first (tiles wholly beyond stay unwritten), 2 = `a` is such a matrix after
+// its softmax (zeros beyond the diagonal), so a tile of rows contracts only as far as its last row sees.
+int gemm_nt_causal(const void* a, const void* b, const void* addend, void* c, int64_t M, int64_t N, int64_t K,
+                   int64_t lda, int64_t ldb, int64_t ldc, int64_t ld_add, int64_t batch, int64_t stride_a,
+                   int64_t stride_b, int64_t stride_c, int64_t stride_add, double alpha, double beta, int dtype,
+                   void* workspace, size_t workspace_bytes, void* stream, int causal_kind, long causal_first);
+
 // Everything else (fp32/fp64, any head size, other layouts).
 size_t generic_workspace(const paras_sdpa_args& a);
 int    launch_generic(const paras_sdpa_args& a, void* workspace, hipStream_t s);
